@@ -1,0 +1,261 @@
+/*
+ * retro_mi355.h — C ABI of libretro_mi355.so: MI355X (gfx950) kernels and host
+ * services for RetroInfer's wave-index attention path.
+ *
+ * Conventions
+ *  - Every pointer is a raw address: device memory unless the comment says "host".
+ *    The library never allocates, frees or keeps tensor memory; buffers are borrowed
+ *    for the duration of the call.  The only exception is the host wave buffer
+ *    (ri_wavebuf_*), which — like the reference's WaveBufferCPU — remembers the pinned
+ *    host arrays registered with set_indices/set_kv, so the caller keeps them alive.
+ *  - `stream` is a hipStream_t passed as void* (NULL = the default stream).  Kernels
+ *    are only enqueued; nothing synchronises unless stated.
+ *  - Element type of K/V/centroid/query data is bfloat16 (uint16 bit patterns).
+ *    head_dim must be 128 (the reference hard-codes it: gather_copy.cu:196-199).
+ *  - Return value: RI_OK (0) or a negative RI_ERR_* code; ri_status_string() names it
+ *    and ri_last_hip_error() returns the HIP error behind RI_ERR_LAUNCH.
+ *  - "group" g = batch * kv_heads + kv_head, BG groups in total; gs = query heads per
+ *    KV head (<= 16).
+ *
+ * Each entry point cites the reference interface (file:line under the reference tree)
+ * it stands in for.
+ */
+#ifndef RETRO_MI355_H
+#define RETRO_MI355_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef void* ri_stream_t;
+
+enum {
+  RI_OK = 0,
+  RI_ERR_ARG = -1,       /* bad shape / null pointer / unsupported size */
+  RI_ERR_LAUNCH = -2,    /* HIP reported an error at launch: see ri_last_hip_error() */
+  RI_ERR_WORKSPACE = -3, /* workspace too small */
+  RI_ERR_STATE = -4      /* host object used out of order */
+};
+
+const char* ri_status_string(int status);
+int ri_last_hip_error(void);
+/* ABI version: bumped when a signature changes. */
+int ri_abi_version(void);
+
+/* ------------------------------------------------------------------------------------
+ * (2) Centroid scoring
+ * ---------------------------------------------------------------------------------- */
+
+/* Replaces retroinfer_kernels.batch_gemm_softmax
+ * (library/retroinfer/retroinfer_kernels/src/batch_gemm_softmax.cu:171-198, pybind :201-209).
+ *   A [batch, m, k] queries, B [batch, n, k] centroids (both bf16, k == 128, m <= 16,
+ *   n % 8 == 0), D [batch, m, n] bf16 = bf16(alpha * A·Bᵀ), Softmax [batch, m, n] bf16 =
+ *   bf16(exp(float(D) - rowmax) / rowsum) with rowmax/rowsum taken from the fp32 logits.
+ *   Norm/Sum [batch, ceil(n/256), m] fp32: per-256-column partials; on return slot
+ *   [batch, 0, :] holds the final row max and 1/rowsum (as the reference leaves them).
+ *   beta must be 0. */
+int ri_batch_gemm_softmax(const void* A, const void* B, void* D, float* Norm, float* Sum,
+                          void* Softmax, int batch_count, int m, int n, int k, float alpha,
+                          float beta, ri_stream_t stream);
+
+/* Fused scoring + selection: replaces the sequence batch_gemm_softmax → torch.sum →
+ * masked_fill_ → torch.topk → cluster_ids.copy_ (cache_hub/retroinfer_cache.py:569-575).
+ *   q          [BG, gs, 128] bf16
+ *   centroids  [BG, nc, 128] bf16
+ *   mask       [BG, nc] uint8 (1 = empty cluster, scored as finfo(bf16).min) or NULL
+ *   cluster_size_i32 [BG, nc] int32 token count per cluster, or NULL (then no row table)
+ *   cluster_start    [BG, nc] int32 first row of the cluster in the cluster-contiguous
+ *                    K/V store, or NULL
+ * Outputs
+ *   logits     [BG, gs, nc] fp32  = scale * q·c  (kept for the estimation zone)
+ *   dist       [BG, nc] bf16 score or NULL
+ *   cI         [BG, np+es] int64 or NULL: retrieval ids in rank order (score descending,
+ *              ties by ascending id) followed by estimation ids in ascending id order
+ *   ret_ids    [BG, np] int32, est_ids [BG, es] int32 (same content as cI)
+ *   ret_tok_off[BG, np+1] int32: exclusive token prefix of the retrieval clusters after
+ *              the reference's buffer cut-off (stop before the first cluster whose pages
+ *              push the running total over max_pages; wave_buffer_cpu.cpp:207-216)
+ *   row_src    [BG, row_src_stride] int32: store row of every retrieved token, or NULL
+ *   meta       [BG, 4] int32: {clusters kept, retrieved tokens, pages used, 0}
+ * workspace: ri_score_select_workspace_bytes(BG, gs, nc) bytes of device memory. */
+size_t ri_score_select_workspace_bytes(int BG, int gs, int nc);
+int ri_score_select(const void* q, const void* centroids, const uint8_t* mask,
+                    const int32_t* cluster_size_i32, const int32_t* cluster_start,
+                    float* logits, void* dist, int64_t* cI, int32_t* ret_ids,
+                    int32_t* est_ids, int32_t* ret_tok_off, int32_t* row_src,
+                    int row_src_stride, int32_t* meta, int BG, int gs, int nc, int np, int es,
+                    int page, int max_pages, float scale, void* workspace,
+                    size_t workspace_bytes, ri_stream_t stream);
+
+/* ------------------------------------------------------------------------------------
+ * (4) Weighted flash decoding
+ * ---------------------------------------------------------------------------------- */
+
+/* Replaces weighted_flash_decoding(q, k, v[, weight], previous_out=, previous_lse=,
+ * cache_seqlens=, return_softmax_lse=) as called at cache_hub/retroinfer_cache.py:611-617
+ * and :666-674 (the callee is an external fork that is not part of the reference tree).
+ *   q [BG, gs, 128], k/v [BG, kv_stride rows, 128] bf16 (row r of group g at
+ *   (g*kv_stride + r)*128), weight [BG, S] bf16 or NULL (multiplies each key's term in the
+ *   softmax denominator only), cache_seqlens [BG] int32 or NULL (then every group has S
+ *   rows), prev_out [BG, gs, 128] bf16 + prev_lse [BG, gs] fp32 or both NULL,
+ *   out [BG, gs, 128] bf16, lse_out [BG, gs] fp32 or NULL.
+ *   out = (e^{prev_lse}·prev_out + Σ_r e^{s_r} v_r) / (e^{prev_lse} + Σ_r w_r e^{s_r}),
+ *   s_r = scale·q·k_r;  lse_out = log of that denominator. */
+size_t ri_flash_decoding_workspace_bytes(int BG, int gs);
+int ri_weighted_flash_decoding(const void* q, const void* k, const void* v, const void* weight,
+                               const int32_t* cache_seqlens, const void* prev_out,
+                               const float* prev_lse, void* out, float* lse_out, int BG,
+                               int gs, int S, int64_t kv_stride, float scale, void* workspace,
+                               size_t workspace_bytes, ri_stream_t stream);
+
+/* Fused wave-index attention over a device-resident cluster store: replaces steps 4-8 of
+ * retroinfer_cache.compute (gather_copy_vectors → weighted_flash_decoding →
+ * gather_copy_and_concat → weighted_flash_decoding, cache_hub/retroinfer_cache.py:598-674)
+ * when every cluster's K/V already sits in device memory, reading K/V in place through
+ * the row table instead of staging them in an execution buffer.
+ *   steady_k/v [BG, steady_stride, 128]: first static_len rows attended
+ *   store_k/v  [BG, store_stride, 128]: cluster-contiguous K/V
+ *   row_src, meta, est_ids, logits: as written by ri_score_select
+ *   value_sum [BG, nc, 128] bf16, cluster_size_bf16 [BG, nc] bf16 (estimation weights)
+ *   es may be 0 (no estimation zone).  out [BG, gs, 128] bf16; valid_lengths [BG] int32 or
+ *   NULL receives static_len + retrieved tokens (what gather_copy_and_concat reports). */
+size_t ri_wave_attention_workspace_bytes(int BG, int gs);
+int ri_wave_attention(const void* q, const void* steady_k, const void* steady_v,
+                      int64_t steady_stride, int static_len, const void* store_k,
+                      const void* store_v, int64_t store_stride, const int32_t* row_src,
+                      int row_src_stride, const int32_t* meta, const int32_t* est_ids,
+                      const float* logits, const void* value_sum,
+                      const void* cluster_size_bf16, void* out, int32_t* valid_lengths,
+                      int BG, int gs, int nc, int es, float scale, void* workspace,
+                      size_t workspace_bytes, ri_stream_t stream);
+
+/* ------------------------------------------------------------------------------------
+ * (3) Wave-buffer copies
+ * ---------------------------------------------------------------------------------- */
+
+/* Replaces gather_copy_vectors (gather_copy.cu:25-96, kernel copy_kernel.cuh:43-88):
+ * dst_keys[g, i] = src_keys[g, idx[g, copy_start+i]] for i < copy_num, same for values and
+ * the 2-byte metadata.  idx [groups, index_size] int64. */
+int ri_gather_copy_vectors(const void* src_keys, void* dst_keys, const void* src_values,
+                           void* dst_values, const void* src_meta, void* dst_meta,
+                           const int64_t* idx, int groups, int data_length, int buffer_length,
+                           int index_size, int copy_start, int copy_num, ri_stream_t stream);
+
+/* Replaces gather_copy_and_concat (gather_copy.cu:100-212, kernel copy_kernel.cuh:215-329).
+ * Per group: dst = [src1[0:copy_vectors1] | src2 blocks | src3 blocks]; src2 (cluster store,
+ * may be pinned host memory mapped into the device) is indexed by start vector, src3 (block
+ * cache [groups, data_length3, 8, 128]) by block id; each block copies sizes[] (<= 8)
+ * vectors to dst offset copy_vectors1 (+ all src2 vectors for src3) + dst_off[].  Index
+ * arrays [groups, offset_length] int32 and counts [groups] int32 may live in pinned host
+ * memory.  valid_lengths[g] = total vectors written. */
+int ri_gather_copy_and_concat(const void* k1, const void* k2, const void* k3, void* kdst,
+                              const void* v1, const void* v2, const void* v3, void* vdst,
+                              const int32_t* off2, const int32_t* sizes2, const int32_t* dst2,
+                              const int32_t* num2, const int32_t* off3, const int32_t* sizes3,
+                              const int32_t* dst3, const int32_t* num3, int32_t* valid_lengths,
+                              int groups, int data_length1, int data_length2, int data_length3,
+                              int buffer_length, int offset_length, int copy_vectors1,
+                              ri_stream_t stream);
+
+/* Replaces gather_copy_and_scatter (gather_copy.cu:216-283, kernel copy_kernel.cuh:379-420):
+ * cache[g, dst_block[g,j], 0:sizes[g,j]] = src[g, s_copy_start + src_off[g,j] : +sizes]. */
+int ri_gather_copy_and_scatter(const void* ksrc, void* kcache, const void* vsrc, void* vcache,
+                               const int32_t* src_off, const int32_t* sizes,
+                               const int32_t* dst_block, const int32_t* num, int groups,
+                               int data_length, int buffer_length, int offset_length,
+                               int s_copy_start, ri_stream_t stream);
+
+/* ------------------------------------------------------------------------------------
+ * (1) Prefill k-means
+ * ---------------------------------------------------------------------------------- */
+
+/* Assignment step of _triton_k_means_train (cache_hub/kmeans.py:6-49, launch :101-111):
+ * assign[p, n] = argmax_c <data[p,n,:], centroids[p,c,:]> with fp32 accumulation and the
+ * smallest c on ties.  centroids [P, nc, 128] bf16 (nc % 32 == 0, kmeans.py:99), assign
+ * [P, N] int32.  Problem p reads N data rows starting at row
+ * (p / seg) * head_rows + (p % seg) * N of `data` (bf16, 128 wide): seg consecutive
+ * segments per head, heads head_rows apart — the reshape of kmeans.py:242 without a copy;
+ * seg = 1, head_rows = N for one problem per head.  (The reference's atomic sum/count side
+ * effects are produced by ri_kmeans_update instead, in a fixed summation order.) */
+int ri_kmeans_assign(const void* data, const void* centroids, int32_t* assign, int P, int N,
+                     int nc, int seg, int64_t head_rows, ri_stream_t stream);
+
+/* Inverted lists: replaces triton_reverse_index (cache_hub/kmeans.py:128-173) in CSR form.
+ * counts [P, nc] int32, offsets [P, nc+1] int32 (exclusive prefix), members [P, N] int32 =
+ * token ids grouped by cluster, ascending inside each cluster.
+ * workspace: ri_kmeans_workspace_bytes(P, N, nc). */
+size_t ri_kmeans_workspace_bytes(int P, int N, int nc);
+int ri_kmeans_build_lists(const int32_t* assign, int32_t* counts, int32_t* offsets,
+                          int32_t* members, int P, int N, int nc, void* workspace,
+                          size_t workspace_bytes, ri_stream_t stream);
+
+/* Centroid update: replaces the atomic accumulation of _triton_assign_kernel
+ * (kmeans.py:48-49) plus _triton_update_kernel (kmeans.py:52-80).  For every cluster with
+ * counts > 0: mean = (Σ member rows, fp32, ascending token order) / count; if normalize,
+ * mean /= ||mean||₂; centroids[p,c,:] = bf16(mean).  Empty clusters keep their centroid. */
+int ri_kmeans_update(const void* data, const int32_t* counts, const int32_t* offsets,
+                     const int32_t* members, void* centroids, int P, int N, int nc, int seg,
+                     int64_t head_rows, int normalize, ri_stream_t stream);
+
+/* Per-cluster value sums: replaces triton_index_add (cache_hub/kmeans.py:176-221).
+ * value_sum[p,c,:] = bf16(Σ member value rows, fp32, ascending token order). */
+int ri_kmeans_value_sum(const void* values, const int32_t* counts, const int32_t* offsets,
+                        const int32_t* members, void* value_sum, int P, int N, int nc,
+                        ri_stream_t stream);
+
+/* Device-side replacement of WaveBufferCPU::organize_kv (wave_buffer_cpu.cpp:545-567):
+ * out[p, i, :] = in[p, members[p, i], :] — K/V rows permuted into cluster-contiguous order. */
+int ri_permute_rows(const void* in, const int32_t* members, void* out, int P, int N,
+                    int64_t in_stride_rows, int64_t out_stride_rows, ri_stream_t stream);
+
+/* ------------------------------------------------------------------------------------
+ * Host wave buffer (LRU block cache manager + K/V re-organisation) and its thread pool
+ * ---------------------------------------------------------------------------------- */
+
+typedef struct ri_threadpool ri_threadpool;
+typedef struct ri_wavebuf ri_wavebuf;
+
+/* Replaces ThreadPool / MyThreadPool (wave_buffer_cpu.cpp:17-35, thread_pool.hpp:27-141). */
+ri_threadpool* ri_threadpool_create(int num_threads);
+void ri_threadpool_destroy(ri_threadpool* pool);
+
+/* Replaces WaveBufferCPU (wave_buffer_cpu.cpp:328-383 ctor; pybind surface :822-849). */
+ri_wavebuf* ri_wavebuf_create(int batch_size, int group_num, int dim, int nprobe,
+                              int block_size, int n_centroids, int final_n_centroids,
+                              int buffer_size, int capacity, int threads, ri_threadpool* pool);
+void ri_wavebuf_destroy(ri_wavebuf* wb);
+/* set_indices (wave_buffer_cpu.cpp:442-486): 12 host int32 arrays + searched ids (int64). */
+int ri_wavebuf_set_indices(ri_wavebuf* wb, int32_t* hit_ids, int32_t* hit_sizes,
+                           int32_t* hit_cumsum, int32_t* hit_nums, int32_t* miss_ids,
+                           int32_t* miss_sizes, int32_t* miss_cumsum, int32_t* miss_nums,
+                           int32_t* update_buffer_indices, int32_t* update_sizes,
+                           int32_t* update_cache_indices, int32_t* update_nums,
+                           int64_t* searched_clusters);
+/* set_kv (wave_buffer_cpu.cpp:488-507): host arrays, 2-byte elements. */
+int ri_wavebuf_set_kv(ri_wavebuf* wb, void* ivf_keys, void* ivf_values,
+                      int64_t output_seq_length, void* input_keys, void* input_values,
+                      int64_t input_seq_length);
+/* async_construction / construction_sync (wave_buffer_cpu.cpp:592-630). */
+int ri_wavebuf_async_construction(ri_wavebuf* wb, const int32_t* clusters,
+                                  const int32_t* cluster_size, int64_t max_cluster_size,
+                                  int batch_idx);
+int ri_wavebuf_construction_sync(ri_wavebuf* wb);
+/* update_kv (wave_buffer_cpu.cpp:688-720). */
+int ri_wavebuf_update_kv(ri_wavebuf* wb, void* update_keys, void* update_values,
+                         int64_t update_seq_length, const int32_t* clusters,
+                         const int32_t* cluster_size, int update_n_centroids,
+                         int64_t max_cluster_size);
+/* batch_access = para_batch_access (wave_buffer_cpu.cpp:789-809); sync (:811-814). */
+int ri_wavebuf_batch_access(ri_wavebuf* wb);
+int ri_wavebuf_sync(ri_wavebuf* wb);
+/* Number of clusters skipped so far because a group's pages exceeded buffer_size (the
+ * reference prints a warning per event, wave_buffer_cpu.cpp:212-216). */
+int64_t ri_wavebuf_overflow_events(const ri_wavebuf* wb);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* RETRO_MI355_H */

@@ -1,0 +1,29 @@
+"""CPU restatement of RetroInfer's wave-index path (reference: wennitao/RetrievalAttention).
+
+TEST INFRASTRUCTURE ONLY.  Nothing under this package is part of the product: it is the
+checker that tests/, __graft_entry__.smoke() and the cpu_baseline leg of bench.py compare the
+HIP kernels against.  The product (retrievalattention_amd/) never imports it.
+
+Every function cites the reference file:line it follows.  How each one is pinned:
+
+  scoring.batch_gemm_softmax      the reference's own test oracle bmm -> /sqrt(d) -> softmax
+                                  (library/retroinfer/test/test_batch_gemm_softmax.py:9-18, atol 1e-3)
+  scoring.select                  torch.sum / masked_fill_ / topk are library routines; checked
+                                  against torch.topk value-for-value and against brute force
+  copies.*                        the loop oracles of library/retroinfer/test/test_gather_copy.py
+                                  (:110-127, :190-194, :233-237), bit-exact
+  wavebuf.LruModel                brute-force list model + invariants (hit <=> resident, capacity,
+                                  unique block ids, least-recently-touched eviction)
+  kmeans.*                        brute force on tiny inputs in fp64, plus invariants (partition of
+                                  the tokens, centroid*size = sum of keys, empty cluster keeps its
+                                  centroid, float32 init formula, remainder tokens)
+  attention.weighted_flash_decoding   PARITY UNPINNED against the reference: the callee
+                                  (github.com/Starmys/flash-attention, branch "weighted") is not in
+                                  the reference tree and has no test there.  Semantics are inferred
+                                  from the call sites (cache_hub/retroinfer_cache.py:611-617,
+                                  :666-674) and pinned only by closed forms: w = 1 reduces to
+                                  softmax attention (torch SDPA); merging with a previous partial
+                                  equals attention over the concatenated keys; one token per
+                                  cluster makes the estimate exact; identical keys in a cluster
+                                  make the estimate exact for any sizes.
+"""

@@ -1,0 +1,377 @@
+// Prefill k-means kernels (gfx950): inner-product assignment on bf16 MFMA, deterministic
+// inverted lists, and list-ordered segmented reductions for centroid and value sums.
+// Restates cache_hub/kmeans.py (assign :6-49, update :52-80, reverse index :128-173,
+// index add :176-221) with a fixed summation order instead of fp32 atomics.
+#include "ri_common.h"
+
+typedef float f32x16_t __attribute__((ext_vector_type(16)));
+
+#define KM_CT 32          // centroids per LDS tile
+#define KM_ROW_U16 136    // padded LDS row (272 bytes) to spread ds_read_b128 over the banks
+
+// first data row of problem p: problems are `seg` consecutive N-row slices of each head
+__device__ __forceinline__ size_t km_row0(int p, int seg, int64_t head_rows, int N) {
+  return (size_t)(p / seg) * (size_t)head_rows + (size_t)(p % seg) * (size_t)N;
+}
+
+// ------------------------------------------------------------------------------------
+// assign: grid (ceil(N/256), P), 256 threads; wave = 64 tokens (two 32-token MFMA columns),
+// centroid tiles of 32 rows staged in LDS and shared by the four waves.
+// MFMA 32x32x16: A = centroid rows, B = token columns; accumulator i of lane l is
+// row (i/4)*8 + (l/32)*4 + i%4, column l%32.
+// ------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void km_assign_kernel(const uint16_t* __restrict__ data,
+                                                        const uint16_t* __restrict__ cent,
+                                                        int32_t* __restrict__ assign, int N, int nc, int seg,
+                                                        int64_t head_rows) {
+  __shared__ __attribute__((aligned(16))) uint16_t sh_c[KM_CT][KM_ROW_U16];
+  const int p = blockIdx.y;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int r = lane & 31, hh = lane >> 5;
+  const int t0 = blockIdx.x * 256 + wave * 64;
+  const uint16_t* dp = data + km_row0(p, seg, head_rows, N) * RI_DIM;
+  const uint16_t* cp = cent + (size_t)p * nc * RI_DIM;
+
+  uint4 b[2][8];
+#pragma unroll
+  for (int tt = 0; tt < 2; ++tt) {
+    const int tok = t0 + tt * 32 + r;
+    const uint16_t* q = dp + (size_t)tok * RI_DIM + hh * 8;
+#pragma unroll
+    for (int kk = 0; kk < 8; ++kk) b[tt][kk] = (tok < N) ? ri_ld16(q + kk * 16) : ri_zero16();
+  }
+  float best[2] = {-INFINITY, -INFINITY};
+  int bidx[2] = {0, 0};
+
+  for (int ct = 0; ct < nc; ct += KM_CT) {
+    __syncthreads();
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+      const int idx = threadIdx.x + 256 * u;
+      const int row = idx >> 4, piece = idx & 15;
+      *reinterpret_cast<uint4*>(&sh_c[row][piece * 8]) = ri_ld16(cp + (size_t)(ct + row) * RI_DIM + piece * 8);
+    }
+    __syncthreads();
+    f32x16_t acc[2];
+#pragma unroll
+    for (int tt = 0; tt < 2; ++tt)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) acc[tt][i] = 0.f;
+#pragma unroll
+    for (int kk = 0; kk < 8; ++kk) {
+      const uint4 a = *reinterpret_cast<const uint4*>(&sh_c[r][kk * 16 + hh * 8]);
+#pragma unroll
+      for (int tt = 0; tt < 2; ++tt)
+        acc[tt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ri_as_bf16x8(a), ri_as_bf16x8(b[tt][kk]), acc[tt], 0, 0, 0);
+    }
+#pragma unroll
+    for (int tt = 0; tt < 2; ++tt)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        const float v = acc[tt][i];
+        if (v > best[tt]) {
+          best[tt] = v;
+          bidx[tt] = ct + (i >> 2) * 8 + hh * 4 + (i & 3);
+        }
+      }
+  }
+#pragma unroll
+  for (int tt = 0; tt < 2; ++tt) {
+    const float ob = __shfl_xor(best[tt], 32);
+    const int oi = __shfl_xor(bidx[tt], 32);
+    if (ob > best[tt] || (ob == best[tt] && oi < bidx[tt])) {
+      best[tt] = ob;
+      bidx[tt] = oi;
+    }
+    const int tok = t0 + tt * 32 + r;
+    if (hh == 0 && tok < N) assign[(size_t)p * N + tok] = bidx[tt];
+  }
+}
+
+// ------------------------------------------------------------------------------------
+// inverted lists
+// ------------------------------------------------------------------------------------
+__global__ void km_zero_kernel(int32_t* a, size_t n) {
+  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) a[i] = 0;
+}
+
+__global__ __launch_bounds__(256) void km_count_kernel(const int32_t* __restrict__ assign,
+                                                       int32_t* __restrict__ counts, int N, int nc) {
+  const int p = blockIdx.y;
+  const int n = blockIdx.x * 256 + threadIdx.x;
+  if (n < N) atomicAdd(&counts[(size_t)p * nc + assign[(size_t)p * N + n]], 1);
+}
+
+// one workgroup per problem: offsets = exclusive prefix of counts; cursor = copy of offsets
+__global__ __launch_bounds__(1024) void km_scan_kernel(const int32_t* __restrict__ counts,
+                                                       int32_t* __restrict__ offsets,
+                                                       int32_t* __restrict__ cursor, int nc) {
+  __shared__ int32_t sh_w[16];
+  __shared__ int32_t sh_carry;
+  const int p = blockIdx.x;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  if (threadIdx.x == 0) sh_carry = 0;
+  __syncthreads();
+  for (int base = 0; base < nc; base += 1024) {
+    const int c = base + threadIdx.x;
+    const int32_t v = (c < nc) ? counts[(size_t)p * nc + c] : 0;
+    int32_t inc = v;
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+      const int32_t n = __shfl_up(inc, d);
+      if (lane >= d) inc += n;
+    }
+    if (lane == 63) sh_w[wave] = inc;
+    __syncthreads();
+    int32_t woff = 0, tot = 0;
+#pragma unroll
+    for (int w = 0; w < 16; ++w) {
+      const int32_t s = sh_w[w];
+      if (w < wave) woff += s;
+      tot += s;
+    }
+    const int32_t ex = sh_carry + woff + inc - v;
+    if (c < nc) {
+      offsets[(size_t)p * (nc + 1) + c] = ex;
+      cursor[(size_t)p * nc + c] = ex;
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) sh_carry += tot;
+    __syncthreads();
+  }
+  if (threadIdx.x == 0) offsets[(size_t)p * (nc + 1) + nc] = sh_carry;
+}
+
+__global__ __launch_bounds__(256) void km_scatter_kernel(const int32_t* __restrict__ assign,
+                                                         int32_t* __restrict__ cursor,
+                                                         int32_t* __restrict__ members, int N, int nc) {
+  const int p = blockIdx.y;
+  const int n = blockIdx.x * 256 + threadIdx.x;
+  if (n < N) {
+    const int pos = atomicAdd(&cursor[(size_t)p * nc + assign[(size_t)p * N + n]], 1);
+    members[(size_t)p * N + pos] = n;
+  }
+}
+
+// Ascending sort inside each list.  One wave per cluster for lists of <= 64 entries; longer
+// lists are queued and sorted by whole workgroups.
+__global__ __launch_bounds__(256) void km_sort_small_kernel(const int32_t* __restrict__ counts,
+                                                            const int32_t* __restrict__ offsets,
+                                                            int32_t* __restrict__ members,
+                                                            int32_t* __restrict__ big_list,
+                                                            int32_t* __restrict__ big_count, int N, int nc) {
+  const int p = blockIdx.y;
+  const int c = blockIdx.x * 4 + (threadIdx.x >> 6);
+  const int lane = threadIdx.x & 63;
+  if (c >= nc) return;
+  const int s = counts[(size_t)p * nc + c];
+  if (s <= 1) return;
+  if (s > 64) {
+    if (lane == 0) {
+      const int k = atomicAdd(&big_count[p], 1);
+      big_list[(size_t)p * nc + k] = c;
+    }
+    return;
+  }
+  int32_t* base = members + (size_t)p * N + offsets[(size_t)p * (nc + 1) + c];
+  const int32_t x = (lane < s) ? base[lane] : 0x7fffffff;
+  int rank = 0;
+  for (int k = 0; k < s; ++k) rank += (__shfl(x, k) < x);
+  if (lane < s) base[rank] = x;
+}
+
+#define KM_BIG_LDS 8192
+__global__ __launch_bounds__(1024) void km_sort_big_kernel(const int32_t* __restrict__ counts,
+                                                           const int32_t* __restrict__ offsets,
+                                                           int32_t* __restrict__ members,
+                                                           const int32_t* __restrict__ big_list,
+                                                           const int32_t* __restrict__ big_count, int N, int nc) {
+  __shared__ int32_t sh[KM_BIG_LDS];
+  const int p = blockIdx.y;
+  const int nbig = big_count[p];
+  for (int k = blockIdx.x; k < nbig; k += gridDim.x) {
+    const int c = big_list[(size_t)p * nc + k];
+    const int s = counts[(size_t)p * nc + c];
+    int32_t* g = members + (size_t)p * N + offsets[(size_t)p * (nc + 1) + c];
+    const bool in_lds = s <= KM_BIG_LDS;
+    int32_t* a = in_lds ? sh : g;
+    if (in_lds)
+      for (int i = threadIdx.x; i < s; i += 1024) sh[i] = g[i];
+    __syncthreads();
+    int P2 = 1;
+    while (P2 < s) P2 <<= 1;
+    // bitonic network with ascending comparators only, so entries past s act as +inf
+    for (int kk = 2; kk <= P2; kk <<= 1) {
+      for (int i = threadIdx.x; i < s; i += 1024) {
+        const int l = i ^ (kk - 1);
+        if (l > i && l < s) {
+          const int32_t x = a[i], y = a[l];
+          if (x > y) { a[i] = y; a[l] = x; }
+        }
+      }
+      __threadfence_block();
+      __syncthreads();
+      for (int j = kk >> 2; j > 0; j >>= 1) {
+        for (int i = threadIdx.x; i < s; i += 1024) {
+          const int l = i ^ j;
+          if (l > i && l < s) {
+            const int32_t x = a[i], y = a[l];
+            if (x > y) { a[i] = y; a[l] = x; }
+          }
+        }
+        __threadfence_block();
+        __syncthreads();
+      }
+    }
+    if (in_lds)
+      for (int i = threadIdx.x; i < s; i += 1024) g[i] = sh[i];
+    __syncthreads();
+  }
+}
+
+// ------------------------------------------------------------------------------------
+// list-ordered reductions: one wave per cluster, lane l owns dims 2l and 2l+1
+// ------------------------------------------------------------------------------------
+template <bool MEAN>
+__global__ __launch_bounds__(256) void km_reduce_kernel(const uint16_t* __restrict__ rows,
+                                                        const int32_t* __restrict__ counts,
+                                                        const int32_t* __restrict__ offsets,
+                                                        const int32_t* __restrict__ members,
+                                                        uint16_t* __restrict__ out, int N, int nc, int seg,
+                                                        int64_t head_rows, int normalize) {
+  const int p = blockIdx.y;
+  const int c = blockIdx.x * 4 + (threadIdx.x >> 6);
+  const int lane = threadIdx.x & 63;
+  if (c >= nc) return;
+  const int s = counts[(size_t)p * nc + c];
+  uint32_t* op = reinterpret_cast<uint32_t*>(out + ((size_t)p * nc + c) * RI_DIM) + lane;
+  if (s == 0) {
+    if (!MEAN) *op = 0u;  // empty cluster: zero value sum; the centroid is left untouched
+    return;
+  }
+  const int32_t* mem = members + (size_t)p * N + offsets[(size_t)p * (nc + 1) + c];
+  const uint32_t* rp = reinterpret_cast<const uint32_t*>(rows + km_row0(p, seg, head_rows, N) * RI_DIM) + lane;
+  float s0 = 0.f, s1 = 0.f;
+  for (int k = 0; k < s; ++k) {
+    const uint32_t v = rp[(size_t)mem[k] * (RI_DIM / 2)];
+    s0 += __uint_as_float(v << 16);
+    s1 += __uint_as_float(v & 0xffff0000u);
+  }
+  if (MEAN) {
+    const float cnt = (float)s;
+    s0 = s0 / cnt;
+    s1 = s1 / cnt;
+    if (normalize) {
+      float sq = s0 * s0 + s1 * s1;  // two roundings: built without fp contraction
+#pragma unroll
+      for (int o = 32; o > 0; o >>= 1) sq += __shfl_xor(sq, o);
+      const float nrm = sqrtf(sq);
+      s0 = s0 / nrm;
+      s1 = s1 / nrm;
+    }
+  }
+  *op = (uint32_t)ri_f32_to_bf16(s0) | ((uint32_t)ri_f32_to_bf16(s1) << 16);
+}
+
+// out[p, i, :] = in[p, members[p, i], :]; 16 lanes per row
+__global__ __launch_bounds__(256) void km_permute_kernel(const uint4* __restrict__ in,
+                                                         const int32_t* __restrict__ members,
+                                                         uint4* __restrict__ out, int N, int64_t in_stride,
+                                                         int64_t out_stride) {
+  const int p = blockIdx.y;
+  const int i = blockIdx.x * 16 + (threadIdx.x >> 4);
+  const int piece = threadIdx.x & 15;
+  if (i >= N) return;
+  const int32_t src = members[(size_t)p * N + i];
+  out[((size_t)p * out_stride + i) * 16 + piece] = in[((size_t)p * in_stride + src) * 16 + piece];
+}
+
+// ------------------------------------------------------------------------------------
+// C entry points
+// ------------------------------------------------------------------------------------
+static int km_check(int P, int N, int nc) {
+  if (P <= 0 || N <= 0 || nc <= 0 || P > 65535) return RI_ERR_ARG;
+  return RI_OK;
+}
+
+extern "C" int ri_kmeans_assign(const void* data, const void* centroids, int32_t* assign, int P, int N,
+                                int nc, int seg, int64_t head_rows, ri_stream_t stream) {
+  if (!data || !centroids || !assign) return RI_ERR_ARG;
+  int rc = km_check(P, N, nc);
+  if (rc) return rc;
+  if (nc % KM_CT != 0 || seg <= 0 || P % seg != 0) return RI_ERR_ARG;
+  km_assign_kernel<<<dim3((N + 255) / 256, P), 256, 0, (hipStream_t)stream>>>(
+      (const uint16_t*)data, (const uint16_t*)centroids, assign, N, nc, seg, head_rows);
+  RI_HIP_CHECK_LAUNCH();
+  return RI_OK;
+}
+
+extern "C" size_t ri_kmeans_workspace_bytes(int P, int N, int nc) {
+  if (P <= 0 || N <= 0 || nc <= 0) return 0;
+  // cursor [P, nc] + big_list [P, nc] + big_count [P]
+  return ((size_t)P * nc * 2 + (size_t)P) * sizeof(int32_t);
+}
+
+extern "C" int ri_kmeans_build_lists(const int32_t* assign, int32_t* counts, int32_t* offsets,
+                                     int32_t* members, int P, int N, int nc, void* workspace,
+                                     size_t workspace_bytes, ri_stream_t stream) {
+  if (!assign || !counts || !offsets || !members || !workspace) return RI_ERR_ARG;
+  int rc = km_check(P, N, nc);
+  if (rc) return rc;
+  if (workspace_bytes < ri_kmeans_workspace_bytes(P, N, nc)) return RI_ERR_WORKSPACE;
+  hipStream_t s = (hipStream_t)stream;
+  int32_t* cursor = (int32_t*)workspace;
+  int32_t* big_list = cursor + (size_t)P * nc;
+  int32_t* big_count = big_list + (size_t)P * nc;
+  km_zero_kernel<<<256, 256, 0, s>>>(counts, (size_t)P * nc);
+  RI_HIP_CHECK_LAUNCH();
+  km_zero_kernel<<<1, 256, 0, s>>>(big_count, (size_t)P);
+  RI_HIP_CHECK_LAUNCH();
+  const dim3 tok_grid((N + 255) / 256, P);
+  km_count_kernel<<<tok_grid, 256, 0, s>>>(assign, counts, N, nc);
+  RI_HIP_CHECK_LAUNCH();
+  km_scan_kernel<<<P, 1024, 0, s>>>(counts, offsets, cursor, nc);
+  RI_HIP_CHECK_LAUNCH();
+  km_scatter_kernel<<<tok_grid, 256, 0, s>>>(assign, cursor, members, N, nc);
+  RI_HIP_CHECK_LAUNCH();
+  km_sort_small_kernel<<<dim3((nc + 3) / 4, P), 256, 0, s>>>(counts, offsets, members, big_list, big_count, N, nc);
+  RI_HIP_CHECK_LAUNCH();
+  km_sort_big_kernel<<<dim3(16, P), 1024, 0, s>>>(counts, offsets, members, big_list, big_count, N, nc);
+  RI_HIP_CHECK_LAUNCH();
+  return RI_OK;
+}
+
+extern "C" int ri_kmeans_update(const void* data, const int32_t* counts, const int32_t* offsets,
+                                const int32_t* members, void* centroids, int P, int N, int nc, int seg,
+                                int64_t head_rows, int normalize, ri_stream_t stream) {
+  if (!data || !counts || !offsets || !members || !centroids) return RI_ERR_ARG;
+  int rc = km_check(P, N, nc);
+  if (rc) return rc;
+  if (seg <= 0 || P % seg != 0) return RI_ERR_ARG;
+  km_reduce_kernel<true><<<dim3((nc + 3) / 4, P), 256, 0, (hipStream_t)stream>>>(
+      (const uint16_t*)data, counts, offsets, members, (uint16_t*)centroids, N, nc, seg, head_rows, normalize);
+  RI_HIP_CHECK_LAUNCH();
+  return RI_OK;
+}
+
+extern "C" int ri_kmeans_value_sum(const void* values, const int32_t* counts, const int32_t* offsets,
+                                   const int32_t* members, void* value_sum, int P, int N, int nc,
+                                   ri_stream_t stream) {
+  if (!values || !counts || !offsets || !members || !value_sum) return RI_ERR_ARG;
+  int rc = km_check(P, N, nc);
+  if (rc) return rc;
+  km_reduce_kernel<false><<<dim3((nc + 3) / 4, P), 256, 0, (hipStream_t)stream>>>(
+      (const uint16_t*)values, counts, offsets, members, (uint16_t*)value_sum, N, nc, 1, (int64_t)N, 0);
+  RI_HIP_CHECK_LAUNCH();
+  return RI_OK;
+}
+
+extern "C" int ri_permute_rows(const void* in, const int32_t* members, void* out, int P, int N,
+                               int64_t in_stride_rows, int64_t out_stride_rows, ri_stream_t stream) {
+  if (!in || !members || !out || P <= 0 || N <= 0 || P > 65535 || in_stride_rows < N || out_stride_rows < N)
+    return RI_ERR_ARG;
+  km_permute_kernel<<<dim3((N + 15) / 16, P), 256, 0, (hipStream_t)stream>>>(
+      (const uint4*)in, members, (uint4*)out, N, in_stride_rows, out_stride_rows);
+  RI_HIP_CHECK_LAUNCH();
+  return RI_OK;
+}

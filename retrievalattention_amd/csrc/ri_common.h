@@ -1,0 +1,61 @@
+// Shared device/host helpers for the gfx950 wave-index kernels.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/retro_mi355.h"
+
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
+
+#define RI_DIM 128  // head dimension every kernel is specialised for
+
+// ---- bf16 <-> fp32 (round-to-nearest-even, NaN preserved as quiet NaN) ----
+__host__ __device__ __forceinline__ float ri_bf16_to_f32(uint16_t v) {
+  union { uint32_t u; float f; } x;
+  x.u = (uint32_t)v << 16;
+  return x.f;
+}
+__host__ __device__ __forceinline__ uint16_t ri_f32_to_bf16(float f) {
+  union { uint32_t u; float f; } x;
+  x.f = f;
+  if ((x.u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((x.u >> 16) | 0x40u);
+  uint32_t r = ((x.u >> 16) & 1u) + 0x7fffu;
+  return (uint16_t)((x.u + r) >> 16);
+}
+// fp32 value of the bf16 rounding of f
+__host__ __device__ __forceinline__ float ri_round_bf16(float f) {
+  return ri_bf16_to_f32(ri_f32_to_bf16(f));
+}
+
+__device__ __forceinline__ bf16x8_t ri_as_bf16x8(uint4 v) {
+  return __builtin_bit_cast(bf16x8_t, v);
+}
+__device__ __forceinline__ uint4 ri_ld16(const void* p) {
+  return *reinterpret_cast<const uint4*>(p);
+}
+__device__ __forceinline__ uint4 ri_zero16() { return make_uint4(0u, 0u, 0u, 0u); }
+
+// unpack 8 bf16 packed in a uint4 into fp32
+__device__ __forceinline__ void ri_unpack8(uint4 v, float* f) {
+  f[0] = __uint_as_float(v.x << 16); f[1] = __uint_as_float(v.x & 0xffff0000u);
+  f[2] = __uint_as_float(v.y << 16); f[3] = __uint_as_float(v.y & 0xffff0000u);
+  f[4] = __uint_as_float(v.z << 16); f[5] = __uint_as_float(v.z & 0xffff0000u);
+  f[6] = __uint_as_float(v.w << 16); f[7] = __uint_as_float(v.w & 0xffff0000u);
+}
+
+// bf16 bit pattern -> key whose unsigned order equals the float order
+__host__ __device__ __forceinline__ uint32_t ri_bf16_sort_key(uint16_t b) {
+  return (b & 0x8000u) ? (uint32_t)(~b & 0xffffu) : (uint32_t)(b | 0x8000u);
+}
+
+#define RI_HIP_CHECK_LAUNCH()                         \
+  do {                                                \
+    hipError_t e__ = hipGetLastError();               \
+    if (e__ != hipSuccess) {                          \
+      ri_set_last_hip_error((int)e__);                \
+      return RI_ERR_LAUNCH;                           \
+    }                                                 \
+  } while (0)
+
+void ri_set_last_hip_error(int e);

@@ -1,0 +1,283 @@
+"""Torch-facing wrappers of the C ABI.  The first block keeps the names and argument order of
+the reference's `retroinfer_kernels` extension and of `weighted_flash_decoding`
+(library/retroinfer/retroinfer_kernels/src/*.cu, *.cpp pybind sections), so code written
+against the reference runs unchanged; the second block exposes the fused MI355X entry points.
+
+Tensors only provide memory and the current stream; all arithmetic happens in the library.
+"""
+import math
+
+import torch
+
+from ._lib import lib, check
+
+_DT = (torch.bfloat16,)
+
+
+def _stream():
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _p(t):
+    return None if t is None else t.data_ptr()
+
+
+def _need(t, dtype, name, cuda=True):
+    if t.dtype != dtype:
+        raise TypeError(f"{name}: expected {dtype}, got {t.dtype}")
+    if cuda and not t.is_cuda:
+        raise ValueError(f"{name}: expected a device tensor")
+    if not t.is_contiguous():
+        raise ValueError(f"{name}: expected a contiguous tensor")
+
+
+_workspaces = {}
+
+
+def _workspace(nbytes, device, tag):
+    """Per-(device, tag) scratch tensor, grown on demand and reused across calls."""
+    key = (str(device), tag)
+    w = _workspaces.get(key)
+    if w is None or w.numel() < nbytes:
+        w = torch.empty(max(nbytes, 256), dtype=torch.uint8, device=device)
+        _workspaces[key] = w
+    return w
+
+
+# ----------------------------------------------------------------------------------------
+# retroinfer_kernels-compatible surface
+# ----------------------------------------------------------------------------------------
+def batch_gemm_softmax(A, B, D, Norm, Sum, Softmax, batch_count, m, n, k, alpha=1.0, beta=0.0):
+    """batch_gemm_softmax.cu:201-209.  A [bc, m, k], B [bc, n, k]; D/Softmax [bc, m, n]."""
+    if A.dtype not in _DT:
+        raise RuntimeError("Only BFloat16 is supported by the gfx950 kernels")
+    for t, nm in ((A, "A"), (B, "B"), (D, "D"), (Softmax, "Softmax")):
+        _need(t, torch.bfloat16, nm)
+    _need(Norm, torch.float32, "Norm"); _need(Sum, torch.float32, "Sum")
+    ntiles = (n + 255) // 256
+    if A.numel() < batch_count * m * k or B.numel() < batch_count * n * k or \
+            D.numel() < batch_count * m * n or Softmax.numel() < batch_count * m * n or \
+            Norm.numel() < batch_count * ntiles * m or Sum.numel() < batch_count * ntiles * m:
+        raise ValueError("batch_gemm_softmax: a buffer is smaller than its shape arguments")
+    check(lib().ri_batch_gemm_softmax(_p(A), _p(B), _p(D), _p(Norm), _p(Sum), _p(Softmax), batch_count, m, n, k,
+                                      float(alpha), float(beta), _stream()), "batch_gemm_softmax")
+
+
+def gather_copy_vectors(key_data, key_buffer, value_data, value_buffer, src_metadata, dst_metadata,
+                        data_offsets, groups, data_length, buffer_length, index_size, copy_start, copy_num):
+    """gather_copy.cu:288-292."""
+    for t, nm in ((key_data, "key_data"), (key_buffer, "key_buffer"), (value_data, "value_data"),
+                  (value_buffer, "value_buffer"), (src_metadata, "src_metadata"), (dst_metadata, "dst_metadata")):
+        _need(t, torch.bfloat16, nm)
+    _need(data_offsets, torch.int64, "data_offsets")
+    if key_data.numel() < groups * data_length * 128 or key_buffer.numel() < groups * buffer_length * 128 or \
+            data_offsets.numel() < groups * index_size or src_metadata.numel() < groups * data_length or \
+            dst_metadata.numel() < groups * buffer_length:
+        raise ValueError("gather_copy_vectors: a buffer is smaller than its shape arguments")
+    check(lib().ri_gather_copy_vectors(_p(key_data), _p(key_buffer), _p(value_data), _p(value_buffer),
+                                       _p(src_metadata), _p(dst_metadata), _p(data_offsets), groups, data_length,
+                                       buffer_length, index_size, copy_start, copy_num, _stream()),
+          "gather_copy_vectors")
+
+
+def gather_copy_and_concat(key_data1, key_data2, key_data3, key_buffer, value_data1, value_data2, value_data3,
+                           value_buffer, data_offsets2, data_copy_sizes2, buffer_offsets2, copy_chunks2,
+                           data_offsets3, data_copy_sizes3, buffer_offsets3, copy_chunks3, valid_lengths,
+                           groups, data_length1, data_length2, data_length3, buffer_length, offset_length,
+                           copy_vectors1):
+    """gather_copy.cu:294-300.  key_data2/value_data2 and the index tensors may be pinned host
+    tensors (read in place by the kernel), everything else lives on the device."""
+    for t in (data_offsets2, data_copy_sizes2, buffer_offsets2, copy_chunks2, data_offsets3, data_copy_sizes3,
+              buffer_offsets3, copy_chunks3, valid_lengths):
+        _need(t, torch.int32, "index tensor", cuda=False)
+        if not (t.is_cuda or t.is_pinned()):
+            raise ValueError("index tensors must be device or pinned host tensors")
+    for t in (key_data2, value_data2):
+        if not (t.is_cuda or t.is_pinned()):
+            raise ValueError("key_data2/value_data2 must be device or pinned host tensors")
+    check(lib().ri_gather_copy_and_concat(
+        _p(key_data1), _p(key_data2), _p(key_data3), _p(key_buffer), _p(value_data1), _p(value_data2),
+        _p(value_data3), _p(value_buffer), _p(data_offsets2), _p(data_copy_sizes2), _p(buffer_offsets2),
+        _p(copy_chunks2), _p(data_offsets3), _p(data_copy_sizes3), _p(buffer_offsets3), _p(copy_chunks3),
+        _p(valid_lengths), groups, data_length1, data_length2, data_length3, buffer_length, offset_length,
+        copy_vectors1, _stream()), "gather_copy_and_concat")
+
+
+def gather_copy_and_scatter(key_data, key_buffer, value_data, value_buffer, s_offsets, copy_sizes, d_offsets,
+                            copy_chunks, groups, data_length, buffer_length, offset_length, s_copy_start):
+    """gather_copy.cu:302-305."""
+    for t in (s_offsets, copy_sizes, d_offsets, copy_chunks):
+        _need(t, torch.int32, "index tensor", cuda=False)
+        if not (t.is_cuda or t.is_pinned()):
+            raise ValueError("index tensors must be device or pinned host tensors")
+    check(lib().ri_gather_copy_and_scatter(_p(key_data), _p(key_buffer), _p(value_data), _p(value_buffer),
+                                           _p(s_offsets), _p(copy_sizes), _p(d_offsets), _p(copy_chunks), groups,
+                                           data_length, buffer_length, offset_length, s_copy_start, _stream()),
+          "gather_copy_and_scatter")
+
+
+def weighted_flash_decoding(q, k, v, weight=None, previous_out=None, previous_lse=None, cache_seqlens=None,
+                            return_softmax_lse=False):
+    """Signature of the calls at cache_hub/retroinfer_cache.py:611-617 and :666-674.
+    q [BG, 1, gs, D]; k, v [BG, S, 1, D]; weight [BG, 1, 1, S]; previous_out [BG, 1, gs, D];
+    previous_lse [BG, gs] (any shape with BG*gs elements); cache_seqlens [BG] int32."""
+    BG, one, gs, D = q.shape
+    S = k.shape[1]
+    if one != 1 or D != 128 or k.shape[2] != 1:
+        raise ValueError("weighted_flash_decoding: expected q [BG,1,gs,128], k/v [BG,S,1,128]")
+    for t, nm in ((q, "q"), (k, "k"), (v, "v")):
+        _need(t, torch.bfloat16, nm)
+    if weight is not None:
+        _need(weight, torch.bfloat16, "weight")
+    if previous_out is not None:
+        _need(previous_out, torch.bfloat16, "previous_out")
+        _need(previous_lse, torch.float32, "previous_lse")
+    if cache_seqlens is not None:
+        _need(cache_seqlens, torch.int32, "cache_seqlens")
+    out = torch.empty_like(q)
+    lse = torch.empty((BG, gs), dtype=torch.float32, device=q.device) if return_softmax_lse else None
+    nb = lib().ri_flash_decoding_workspace_bytes(BG, gs)
+    ws = _workspace(nb, q.device, "attn")
+    check(lib().ri_weighted_flash_decoding(_p(q), _p(k), _p(v), _p(weight), _p(cache_seqlens), _p(previous_out),
+                                           _p(previous_lse), _p(out), _p(lse), BG, gs, S, S,
+                                           1.0 / math.sqrt(D), _p(ws), ws.numel(), _stream()),
+          "weighted_flash_decoding")
+    return (out, lse) if return_softmax_lse else out
+
+
+class ThreadPool:
+    """wave_buffer_cpu.cpp:17-35."""
+
+    def __init__(self, num_threads):
+        self._h = lib().ri_threadpool_create(int(num_threads))
+        if not self._h:
+            raise RuntimeError("ri_threadpool_create failed")
+
+    def get(self):
+        return self
+
+    def __del__(self):
+        h, self._h = getattr(self, "_h", None), None
+        if h:
+            lib().ri_threadpool_destroy(h)
+
+
+class WaveBufferCPU:
+    """wave_buffer_cpu.cpp:822-841.  Keeps references to every registered tensor, because the
+    native object stores their addresses."""
+
+    def __init__(self, batch_size, group_num, dim, nprobe, block_size, n_centroids, final_n_centroids,
+                 buffer_size, capacity, threads, pool):
+        self._pool = pool
+        self._keep = {}
+        self._h = lib().ri_wavebuf_create(batch_size, group_num, dim, nprobe, block_size, n_centroids,
+                                          final_n_centroids, buffer_size, capacity, threads, pool._h)
+        if not self._h:
+            raise ValueError("WaveBufferCPU: invalid construction arguments")
+
+    def __del__(self):
+        h, self._h = getattr(self, "_h", None), None
+        if h:
+            lib().ri_wavebuf_destroy(h)
+
+    def set_indices(self, hit_block_ids, hit_block_sizes, hit_block_sizes_cumsum, hit_block_nums,
+                    miss_block_ids, miss_block_sizes, miss_block_sizes_cumsum, miss_block_nums,
+                    update_buffer_indices, update_block_sizes, update_cache_indices, update_block_nums,
+                    searched_clusters):
+        ts = [hit_block_ids, hit_block_sizes, hit_block_sizes_cumsum, hit_block_nums, miss_block_ids,
+              miss_block_sizes, miss_block_sizes_cumsum, miss_block_nums, update_buffer_indices,
+              update_block_sizes, update_cache_indices, update_block_nums]
+        for t in ts:
+            _need(t, torch.int32, "index tensor", cuda=False)
+        _need(searched_clusters, torch.int64, "searched_clusters", cuda=False)
+        self._keep["indices"] = ts + [searched_clusters]
+        check(lib().ri_wavebuf_set_indices(self._h, *[_p(t) for t in ts], _p(searched_clusters)), "set_indices")
+
+    def set_kv(self, ivf_key, ivf_value, input_keys, input_values):
+        self._keep["kv"] = [ivf_key, ivf_value, input_keys, input_values]
+        check(lib().ri_wavebuf_set_kv(self._h, _p(ivf_key), _p(ivf_value), ivf_key.size(2), _p(input_keys),
+                                      _p(input_values), input_keys.size(1)), "set_kv")
+
+    def async_construction(self, clusters, cluster_size, batch_idx):
+        _need(clusters, torch.int32, "clusters", cuda=False)
+        _need(cluster_size, torch.int32, "cluster_size", cuda=False)
+        self._keep["construction"] = [clusters, cluster_size]
+        check(lib().ri_wavebuf_async_construction(self._h, _p(clusters), _p(cluster_size), clusters.size(2),
+                                                  int(batch_idx)), "async_construction")
+
+    def construction_sync(self):
+        check(lib().ri_wavebuf_construction_sync(self._h), "construction_sync")
+
+    def update_kv(self, update_keys, update_values, clusters, cluster_size):
+        _need(clusters, torch.int32, "clusters", cuda=False)
+        _need(cluster_size, torch.int32, "cluster_size", cuda=False)
+        check(lib().ri_wavebuf_update_kv(self._h, _p(update_keys), _p(update_values), update_keys.size(1),
+                                         _p(clusters), _p(cluster_size), clusters.size(1), clusters.size(2)),
+              "update_kv")
+
+    def batch_access(self):
+        check(lib().ri_wavebuf_batch_access(self._h), "batch_access")
+
+    def sync(self):
+        check(lib().ri_wavebuf_sync(self._h), "sync")
+
+    def overflow_events(self):
+        return int(lib().ri_wavebuf_overflow_events(self._h))
+
+
+# ----------------------------------------------------------------------------------------
+# fused MI355X entry points
+# ----------------------------------------------------------------------------------------
+def score_select(q, centroids, mask, cluster_size_i32, cluster_start, logits, dist, cI, ret_ids, est_ids,
+                 ret_tok_off, row_src, meta, nprobe, es, page, max_pages, scale):
+    """Centroid scoring + retrieval/estimation selection + token layout in two launches."""
+    BG, gs, D = q.shape
+    nc = centroids.shape[1]
+    nb = lib().ri_score_select_workspace_bytes(BG, gs, nc)
+    ws = _workspace(nb, q.device, "score")
+    check(lib().ri_score_select(_p(q), _p(centroids), _p(mask), _p(cluster_size_i32), _p(cluster_start),
+                                _p(logits), _p(dist), _p(cI), _p(ret_ids), _p(est_ids), _p(ret_tok_off),
+                                _p(row_src), 0 if row_src is None else row_src.shape[1], _p(meta), BG, gs, nc,
+                                nprobe, es, page, max_pages, float(scale), _p(ws), ws.numel(), _stream()),
+          "score_select")
+
+
+def wave_attention(q, steady_k, steady_v, static_len, store_k, store_v, row_src, meta, est_ids, logits,
+                   value_sum, cluster_size_bf16, out, valid_lengths, es, scale):
+    """Attention over steady zone + retrieved clusters (read in place) + estimation zone."""
+    BG, gs, D = q.shape
+    nc = value_sum.shape[1]
+    nb = lib().ri_wave_attention_workspace_bytes(BG, gs)
+    ws = _workspace(nb, q.device, "attn")
+    check(lib().ri_wave_attention(_p(q), _p(steady_k), _p(steady_v), steady_k.shape[-2], static_len, _p(store_k),
+                                  _p(store_v), store_k.shape[-2], _p(row_src), row_src.shape[1], _p(meta),
+                                  _p(est_ids), _p(logits), _p(value_sum), _p(cluster_size_bf16), _p(out),
+                                  _p(valid_lengths), BG, gs, nc, es, float(scale), _p(ws), ws.numel(), _stream()),
+          "wave_attention")
+
+
+def kmeans_assign(data, centroids, assign, P, N, nc, seg, head_rows):
+    check(lib().ri_kmeans_assign(_p(data), _p(centroids), _p(assign), P, N, nc, seg, head_rows, _stream()),
+          "kmeans_assign")
+
+
+def kmeans_build_lists(assign, counts, offsets, members, P, N, nc):
+    nb = lib().ri_kmeans_workspace_bytes(P, N, nc)
+    ws = _workspace(nb, assign.device, "kmeans")
+    check(lib().ri_kmeans_build_lists(_p(assign), _p(counts), _p(offsets), _p(members), P, N, nc, _p(ws),
+                                      ws.numel(), _stream()), "kmeans_build_lists")
+
+
+def kmeans_update(data, counts, offsets, members, centroids, P, N, nc, seg, head_rows, normalize):
+    check(lib().ri_kmeans_update(_p(data), _p(counts), _p(offsets), _p(members), _p(centroids), P, N, nc, seg,
+                                 head_rows, int(bool(normalize)), _stream()), "kmeans_update")
+
+
+def kmeans_value_sum(values, counts, offsets, members, value_sum, P, N, nc):
+    check(lib().ri_kmeans_value_sum(_p(values), _p(counts), _p(offsets), _p(members), _p(value_sum), P, N, nc,
+                                    _stream()), "kmeans_value_sum")
+
+
+def permute_rows(src, members, dst, P, N, in_stride_rows, out_stride_rows):
+    check(lib().ri_permute_rows(_p(src), _p(members), _p(dst), P, N, in_stride_rows, out_stride_rows, _stream()),
+          "permute_rows")

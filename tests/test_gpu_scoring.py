@@ -1,0 +1,158 @@
+"""Scoring and selection kernels against the oracle (GPU)."""
+import math
+
+import pytest
+import torch
+
+from oracle import scoring
+from oracle.numerics import bf16_ulp
+from tests.parity import check_zone_sets, check_rank_order, ulp_distance_bf16
+
+pytestmark = pytest.mark.gpu
+
+
+def _mixture(BG, gs, nc, seed, outliers=True):
+    g = torch.Generator().manual_seed(seed)
+    cent = torch.randn(BG, nc, 128, generator=g)
+    if outliers:
+        cent[:, :, :4] *= 8
+    q = torch.randn(BG, gs, 128, generator=g)
+    return q.to(torch.bfloat16), cent.to(torch.bfloat16)
+
+
+def test_batch_gemm_softmax_matches_reference_test(dev):
+    """Shape and tolerance of library/retroinfer/test/test_batch_gemm_softmax.py (atol 1e-3),
+    with 16 groups instead of 128 to keep the CPU side short."""
+    from retrievalattention_amd import kernels
+    BG, gs, n, d = 16, 4, 8200, 128
+    g = torch.Generator().manual_seed(0)
+    q = torch.randn(BG, gs, d, generator=g).to(torch.bfloat16)
+    c = torch.randn(BG, n, d, generator=g).to(torch.bfloat16)
+    nt = (n + 255) // 256
+    D = torch.zeros(BG, gs, n, dtype=torch.bfloat16, device=dev)
+    S = torch.zeros_like(D)
+    norm = torch.zeros(BG, gs, nt, dtype=torch.float32, device=dev)
+    ssum = torch.zeros_like(norm)
+    kernels.batch_gemm_softmax(q.to(dev), c.to(dev), D, norm, ssum, S, BG, gs, n, d, 1 / math.sqrt(d), 0)
+    torch.cuda.synchronize()
+    # the reference's oracle: bmm / sqrt(d) -> softmax, in bf16 tensors
+    ref = torch.softmax((torch.bmm(q.float(), c.float().transpose(1, 2)) / math.sqrt(d)), dim=-1)
+    assert torch.allclose(S.cpu().float(), ref, atol=1e-3)
+    # stage-wise: D is the bf16 rounding of the fp32 logits up to accumulation order
+    Dr, m, inv, Sr = scoring.batch_gemm_softmax(q, c)
+    dd = ulp_distance_bf16(D.cpu(), Dr)
+    near_zero = (D.cpu().float() - Dr.float()).abs() <= 1e-5   # ulps mean nothing next to 0
+    assert bool(((dd <= 1) | near_zero).all())
+    assert float((dd > 0).float().mean()) < 2e-3
+    # final row max / inverse sum sit in slot 0 of Norm / Sum
+    fm = norm.view(BG, -1)[:, :gs].cpu()
+    fi = ssum.view(BG, -1)[:, :gs].cpu()
+    assert torch.allclose(fm, m, rtol=0, atol=1e-5)
+    assert torch.allclose(fi, inv, rtol=1e-5)
+    # softmax given the kernel's own D and statistics: at most one bf16 ulp from the oracle's formula
+    Sg = (torch.exp(D.cpu().float() - fm[..., None]) * fi[..., None]).to(torch.bfloat16)
+    assert int(ulp_distance_bf16(S.cpu(), Sg).max()) <= 1
+
+
+@pytest.mark.parametrize("BG,gs,nc,nprobe,es,seed", [
+    (8, 4, 512, 9, 118, 0),       # config-1 shape
+    (4, 4, 8192, 147, 1900, 1),   # config-2 shape, fewer groups
+    (4, 7, 3840, 69, 890, 2),     # config-4 shape (gs = 7)
+    (2, 8, 16384, 294, 3801, 3),  # config-5 shape
+    (3, 1, 64, 1, 0, 4),          # smallest: one probe, no estimation zone
+    (2, 16, 1000, 20, 980, 5),    # nc not a multiple of 256, zones cover every cluster
+])
+def test_score_select(dev, BG, gs, nc, nprobe, es, seed):
+    from retrievalattention_amd import kernels
+    q, cent = _mixture(BG, gs, nc, seed)
+    g = torch.Generator().manual_seed(seed + 100)
+    mask = torch.rand(BG, nc, generator=g) < 0.02
+    size = torch.randint(1, 40, (BG, nc), generator=g, dtype=torch.int32)
+    size[mask] = 0
+    start = (torch.cumsum(size, 1) - size).to(torch.int32)
+    scale = 1 / math.sqrt(128)
+    page, max_pages = 8, max(4 * nprobe, 16) * 2
+    k2 = nprobe + es
+    o = dict(
+        logits=torch.empty(BG, gs, nc, dtype=torch.float32, device=dev),
+        dist=torch.empty(BG, nc, dtype=torch.bfloat16, device=dev),
+        cI=torch.empty(BG, k2, dtype=torch.int64, device=dev),
+        ret=torch.empty(BG, nprobe, dtype=torch.int32, device=dev),
+        est=torch.empty(BG, max(es, 1), dtype=torch.int32, device=dev),
+        off=torch.empty(BG, nprobe + 1, dtype=torch.int32, device=dev),
+        rows=torch.full((BG, max_pages * page), -1, dtype=torch.int32, device=dev),
+        meta=torch.empty(BG, 4, dtype=torch.int32, device=dev),
+    )
+    kernels.score_select(q.to(dev), cent.to(dev), mask.to(torch.uint8).to(dev), size.to(dev), start.to(dev),
+                         o["logits"], o["dist"], o["cI"], o["ret"], o["est"] if es else None, o["off"], o["rows"],
+                         o["meta"], nprobe, es, page, max_pages, scale)
+    torch.cuda.synchronize()
+    o = {k: v.cpu() for k, v in o.items()}
+    ret, est = o["ret"].long(), o["est"][:, :es].long()
+
+    # (1) logits: fp32 accumulation of exact products, any order
+    x_ref = scoring.logits_fp32(q, cent, scale)
+    assert torch.allclose(o["logits"], x_ref, rtol=2e-5, atol=2e-5)
+
+    # (2) score pipeline on the kernel's own logits: <= 1 bf16 ulp from the oracle
+    _, _, _, soft = scoring.softmax_from_logits(o["logits"])
+    dist_ref = scoring.dist_from_softmax(soft, mask)
+    dd = ulp_distance_bf16(o["dist"], dist_ref)
+    assert int(dd.max()) <= 1
+    assert float((dd > 0).float().mean()) < 0.02
+
+    # (3) selection is exact on the kernel's own scores (ties by ascending id)
+    ret_x, est_x = scoring.select(o["dist"], nprobe, es)
+    assert torch.equal(ret, ret_x)
+    assert torch.equal(est, est_x)
+    assert torch.equal(o["cI"][:, :nprobe], ret_x) and torch.equal(o["cI"][:, nprobe:], est_x)
+
+    # (4) end to end against the oracle's scores: identical up to boundary ties
+    _, _, _, soft_o = scoring.softmax_from_logits(x_ref)
+    dist_o = scoring.dist_from_softmax(soft_o, mask)
+    ret_o, est_o = scoring.select(dist_o, nprobe, es)
+    check_zone_sets(dist_o, ret, est, ret_o, est_o, nprobe, es, band=2.0)
+    check_rank_order(dist_o, ret, band=2.0)
+
+    # (5) token layout of the retrieved clusters
+    kept, offs = scoring.retrieval_layout(ret, size, page, max_pages)
+    assert torch.equal(o["meta"][:, 0].long(), kept)
+    assert torch.equal(o["off"].long(), offs)
+    assert torch.equal(o["meta"][:, 1].long(), offs[:, -1])
+    for gi in range(BG):
+        exp_rows = torch.cat([start[gi, c] + torch.arange(int(size[gi, c])) for c in ret[gi, :int(kept[gi])]]
+                             + [torch.zeros(0, dtype=torch.int64)])
+        assert torch.equal(o["rows"][gi, :exp_rows.numel()].long(), exp_rows.long())
+
+
+def test_score_select_page_cutoff(dev):
+    """A tiny execution buffer forces the reference's cut-off: clusters after the first one that
+    does not fit are dropped (wave_buffer_cpu.cpp:207-216)."""
+    from retrievalattention_amd import kernels
+    BG, gs, nc, nprobe, es = 2, 4, 256, 16, 32
+    q, cent = _mixture(BG, gs, nc, 7)
+    size = torch.full((BG, nc), 20, dtype=torch.int32)
+    start = (torch.cumsum(size, 1) - size).to(torch.int32)
+    page, max_pages = 8, 10  # 3 pages per cluster -> only 3 clusters fit
+    logits = torch.empty(BG, gs, nc, dtype=torch.float32, device=dev)
+    ret = torch.empty(BG, nprobe, dtype=torch.int32, device=dev)
+    est = torch.empty(BG, es, dtype=torch.int32, device=dev)
+    off = torch.empty(BG, nprobe + 1, dtype=torch.int32, device=dev)
+    rows = torch.full((BG, max_pages * page), -1, dtype=torch.int32, device=dev)
+    meta = torch.empty(BG, 4, dtype=torch.int32, device=dev)
+    kernels.score_select(q.to(dev), cent.to(dev), None, size.to(dev), start.to(dev), logits, None, None, ret, est,
+                         off, rows, meta, nprobe, es, page, max_pages, 1 / math.sqrt(128))
+    torch.cuda.synchronize()
+    assert meta.cpu()[:, 0].tolist() == [3, 3]
+    assert meta.cpu()[:, 1].tolist() == [60, 60]
+    assert meta.cpu()[:, 2].tolist() == [9, 9]
+
+
+def test_score_select_rejects_bad_shapes(dev):
+    from retrievalattention_amd import kernels
+    q, cent = _mixture(1, 4, 64, 0)
+    logits = torch.empty(1, 4, 64, dtype=torch.float32, device=dev)
+    ret = torch.empty(1, 80, dtype=torch.int32, device=dev)
+    with pytest.raises(RuntimeError, match="invalid argument"):
+        kernels.score_select(q.to(dev), cent.to(dev), None, None, None, logits, None, None, ret, None, None, None,
+                             None, 80, 0, 8, 16, 1.0)   # nprobe > nc
