@@ -1,0 +1,82 @@
+"""segment_k_means with the reference's signature and return values
+(cache_hub/kmeans.py:224-259 of the reference), driven by the gfx950 kernels.
+
+Differences that a caller can observe, both within what the reference leaves open:
+  * cluster sums are accumulated in ascending token order (fp32) instead of by atomics, so
+    the result is reproducible run to run;
+  * tokens inside a cluster list are ascending (the reference's order is whatever its atomics
+    produced).
+"""
+import torch
+
+from .. import kernels
+
+
+def init_centroid_indices(num_tokens, num_centroids, device):
+    """kmeans.py:234-236: float32 arithmetic, truncated to int64."""
+    idx = torch.arange(num_centroids, dtype=torch.float32, device=device) * (num_tokens / num_centroids)
+    idx += num_tokens / num_centroids / 2
+    return idx.to(torch.int64)
+
+
+class KMeansResult:
+    """CSR form of the clustering, kept on the device."""
+    __slots__ = ("centroids", "value_sum", "assign", "counts", "offsets", "members")
+
+
+def segment_k_means_csr(key, value, num_centroids, num_iters=10, num_segments=1, init_indices=None):
+    """Runs the clustering and returns a KMeansResult (no dense cluster lists, no host copy).
+    key/value [G, N, 128] bf16 contiguous device tensors."""
+    G, N, D = key.shape
+    if D != 128 or key.dtype != torch.bfloat16 or not key.is_contiguous():
+        raise ValueError("segment_k_means: expected contiguous bf16 [G, N, 128] keys")
+    if num_centroids % num_segments != 0:
+        raise AssertionError("num_centroids must be divisible by num_segments")
+    dev = key.device
+    nc, S = num_centroids, num_segments
+    if init_indices is None:
+        init_indices = init_centroid_indices(N, nc, dev)
+    centroids = torch.index_select(key, 1, init_indices).contiguous()
+    nseg, ncs = N // S, nc // S
+    if ncs % 32 != 0 or nc % 32 != 0:
+        raise AssertionError("centroids per segment must be a multiple of 32")  # kmeans.py:99
+    P = G * S
+    assign = torch.empty((P, max(nseg, 1)), dtype=torch.int32, device=dev)
+    counts = torch.empty((P, ncs), dtype=torch.int32, device=dev)
+    offsets = torch.empty((P, ncs + 1), dtype=torch.int32, device=dev)
+    members = torch.empty((P, max(nseg, 1)), dtype=torch.int32, device=dev)
+    if nseg > 0:
+        for _ in range(num_iters - 1):
+            kernels.kmeans_assign(key, centroids, assign, P, nseg, ncs, S, N)
+            kernels.kmeans_build_lists(assign, counts, offsets, members, P, nseg, ncs)
+            kernels.kmeans_update(key, counts, offsets, members, centroids, P, nseg, ncs, S, N, True)
+    r = KMeansResult()
+    r.assign = torch.empty((G, N), dtype=torch.int32, device=dev)
+    r.counts = torch.empty((G, nc), dtype=torch.int32, device=dev)
+    r.offsets = torch.empty((G, nc + 1), dtype=torch.int32, device=dev)
+    r.members = torch.empty((G, N), dtype=torch.int32, device=dev)
+    kernels.kmeans_assign(key, centroids, r.assign, G, N, nc, 1, N)
+    kernels.kmeans_build_lists(r.assign, r.counts, r.offsets, r.members, G, N, nc)
+    kernels.kmeans_update(key, r.counts, r.offsets, r.members, centroids, G, N, nc, 1, N, False)
+    r.centroids = centroids
+    r.value_sum = torch.empty((G, nc, D), dtype=value.dtype, device=dev)
+    kernels.kmeans_value_sum(value.contiguous(), r.counts, r.offsets, r.members, r.value_sum, G, N, nc)
+    return r
+
+
+def csr_to_dense(counts, offsets, members):
+    """[G, nc, max_cluster_size] zero-padded lists as triton_reverse_index returns them
+    (kmeans.py:155-173)."""
+    G, nc = counts.shape
+    mx = max(int(counts.max().item()), 1)
+    col = torch.arange(mx, device=counts.device)[None, None, :]
+    valid = col < counts[:, :, None]
+    src = (offsets[:, :nc, None].long() + col).clamp_max(members.shape[1] - 1)
+    dense = torch.gather(members.long()[:, None, :].expand(G, nc, -1), 2, src)
+    return torch.where(valid, dense, torch.zeros_like(dense)).to(torch.int32)
+
+
+def segment_k_means(key, value, num_centroids, num_iters=10, num_segments=1):
+    """Reference signature: returns (centroids, value_sum, clusters, cluster_size)."""
+    r = segment_k_means_csr(key.contiguous(), value, num_centroids, num_iters, num_segments)
+    return r.centroids, r.value_sum, csr_to_dense(r.counts, r.offsets, r.members), r.counts
