@@ -1,0 +1,431 @@
+"""retroinfer_cache: the wave-index KV cache with the reference's constructor, methods and
+attributes (cache_hub/retroinfer_cache.py of the reference), running on the gfx950 library.
+
+Two residencies of the clustered K/V:
+
+  "device"  every cluster's K/V stays in HBM in cluster-contiguous order.  A decode step is
+            two fused calls: score_select (scores, zones, row table) and wave_attention
+            (steady zone + retrieved clusters read in place + estimation zone).  No host
+            round trip, no execution buffer, no block cache.
+  "host"    the reference's arrangement: clustered K/V in pinned host memory, an LRU block
+            cache in HBM managed by the host wave buffer, misses read by the gather kernel
+            straight from host memory, admission after the attention.
+
+"auto" picks "device" when the store fits the memory the base class estimates to be free.
+Buffer names follow the reference so that code poking at them keeps working.
+"""
+import math
+
+import torch
+
+from .. import kernels
+from .cache import KV_Cache
+from .kmeans import segment_k_means_csr, csr_to_dense
+
+# generated tokens are folded into the index every THRESHOLD_LENGTH steps
+THRESHOLD_LENGTH = 1024
+
+
+def _pinned(shape, dtype, fill=None):
+    t = torch.empty(shape, dtype=dtype, pin_memory=True)
+    if fill is not None:
+        t.fill_(fill)
+    return t
+
+
+class retroinfer_cache(KV_Cache):
+    def __init__(self, valid_start, layer_num, batch_size, max_length, num_key_value_heads, num_heads,
+                 head_dim, dtype, layer_mapping, max_new_length, static_pattern_start, static_pattern_end, core,
+                 n_centroids, n_segment, nprobe, max_compute_cluster_num, cache_unit_size, cache_cluster_num,
+                 num_gpus, model_size, use_cluster_estimation=False, kv_residency="auto"):
+        super().__init__(layer_num, batch_size, max_length, num_key_value_heads, num_heads, head_dim, dtype,
+                         layer_mapping, num_gpus, model_size)
+        if head_dim != 128 or dtype != torch.bfloat16:
+            raise ValueError("the gfx950 kernels are built for head_dim 128 and bfloat16")
+        if cache_unit_size != 8:
+            raise ValueError("cache_unit_size must be 8 (block size of the copy kernels)")
+        self.valid_start = valid_start
+        self.static_pattern_start = static_pattern_start
+        self.static_pattern_end = static_pattern_end
+        self.static_pattern_total = static_pattern_start + static_pattern_end
+        self.group_size = self.num_heads // self.kv_head
+        self.batch_groups = self.batch_size * self.kv_head
+        self.page_size = cache_unit_size
+        self.core = core
+        self.use_cluster_estimation = use_cluster_estimation
+
+        self.input_length = self.max_length - max_new_length
+        self.max_new_length = min(max_new_length - 1, THRESHOLD_LENGTH)  # one token comes out of prefill
+        self.input_length_new = ((max_new_length - 2) // THRESHOLD_LENGTH) * THRESHOLD_LENGTH
+        self.n_centroids_per_update_segment = ((THRESHOLD_LENGTH // 16) // 32) * 32
+        self.n_centroids_new = ((max_new_length - 2) // THRESHOLD_LENGTH) * self.n_centroids_per_update_segment
+        self.RSQRT_DIM = 1.0 / math.sqrt(self.head_dim)
+        self.DTYPE_MIN = torch.finfo(self.dtype).min
+
+        self.n_centroids = n_centroids
+        self.n_segment = n_segment
+        self.nprobe = nprobe
+        self.max_compute_cluster_num = max_compute_cluster_num
+        self.es_cluster_num = max_compute_cluster_num - nprobe
+
+        avg_cluster_size = (self.input_length - self.static_pattern_total) // self.n_centroids
+        pages_per_cluster = max(1, math.ceil(avg_cluster_size / self.page_size))
+        self.cache_size = cache_cluster_num * pages_per_cluster
+        self.buffer_size = max(int(self.nprobe * 4), 16) * pages_per_cluster
+        self.static_stride = self.static_pattern_total + self.max_new_length
+        self.list_stride = self.input_length - self.static_pattern_total + self.input_length_new
+        self.execution_stride = self.buffer_size * self.page_size + self.static_stride
+        self.cache_stride = self.cache_size
+
+        if kv_residency not in ("auto", "device", "host"):
+            raise ValueError("kv_residency must be 'auto', 'device' or 'host'")
+        if kv_residency == "auto":
+            store_gib = 2 * layer_num * self.batch_groups * self.list_stride * head_dim * 2 / 1024 ** 3
+            kv_residency = "device" if store_gib * 1.25 < self.free_memory else "host"
+        self.kv_residency = kv_residency
+        self.allocated = True  # the GPU side is always allocated up front on a 288 GB part
+
+        dev = lambda ldx: self.layer_mapping[str(ldx)]
+        BG, D = self.batch_groups, self.head_dim
+        zeros = lambda shape, dt, d: torch.zeros(shape, dtype=dt, device=d)
+        L = range(self.layer_num)
+        self.steady_zone_keys = [zeros((batch_size, self.kv_head, self.static_stride, D), dtype, dev(l)) for l in L]
+        self.steady_zone_values = [zeros((batch_size, self.kv_head, self.static_stride, D), dtype, dev(l)) for l in L]
+        # meta index
+        self.centroids = [zeros((BG, n_centroids, D), dtype, dev(l)) for l in L]
+        self.value_sum = [zeros((BG, n_centroids, D), dtype, dev(l)) for l in L]
+        self.centroids_mask = [zeros((BG, n_centroids), torch.bool, dev(l)) for l in L]
+        self.cluster_size = [zeros((BG, n_centroids), dtype, dev(l)) for l in L]
+        if self.input_length_new > 0 and self.kv_residency == "host":
+            self.offload_update_keys = _pinned((BG, THRESHOLD_LENGTH, D), dtype)
+            self.offload_update_values = _pinned((BG, THRESHOLD_LENGTH, D), dtype)
+
+        if self.kv_residency == "device":
+            self._init_device_store()
+        else:
+            self._init_wave_buffer()
+        self.allocate_computation_buffer()
+
+        self.copystream = torch.cuda.Stream()
+        self.mainevents, self.copyevents = {}, {}
+        for d in sorted(set(self.layer_mapping.values()), key=lambda x: int(str(x).split(":")[-1])):
+            with torch.cuda.device(d):
+                self.mainevents[d] = torch.cuda.Event()
+                self.copyevents[d] = torch.cuda.Event()
+
+    # ------------------------------------------------------------------ allocation
+    def _init_device_store(self):
+        dev = lambda ldx: self.layer_mapping[str(ldx)]
+        BG, D = self.batch_groups, self.head_dim
+        L = range(self.layer_num)
+        shape = (self.batch_size, self.kv_head, self.list_stride, D)
+        self.list_keys = [torch.zeros(shape, dtype=self.dtype, device=dev(l)) for l in L]
+        self.list_values = [torch.zeros(shape, dtype=self.dtype, device=dev(l)) for l in L]
+        # per cluster: first row in the store and token count
+        self.cluster_start = [torch.zeros((BG, self.n_centroids), dtype=torch.int32, device=dev(l)) for l in L]
+        self.cluster_size_i32 = [torch.zeros((BG, self.n_centroids), dtype=torch.int32, device=dev(l)) for l in L]
+        self.store_rows = [[0] * BG for _ in L]  # rows of the store in use, per group
+
+    def _init_wave_buffer(self):
+        dev = lambda ldx: self.layer_mapping[str(ldx)]
+        BG, D = self.batch_groups, self.head_dim
+        L = range(self.layer_num)
+        self.thread_pool = kernels.ThreadPool(self.core)
+        pool = self.thread_pool.get()
+        self.wave_buffer = [kernels.WaveBufferCPU(
+            self.batch_size, self.kv_head, D, self.nprobe, self.page_size, self.n_centroids,
+            self.n_centroids + self.n_centroids_new, self.buffer_size, self.cache_size, self.core, pool) for _ in L]
+        names = ["hit_unit_idices", "hit_unit_sizes", "hit_unit_sizes_cumsum", "miss_unit_idices", "miss_unit_sizes",
+                 "miss_unit_sizes_cumsum", "update_buffer_indices", "update_unit_sizes", "update_cache_indices"]
+        for nm in names:
+            setattr(self, nm, [_pinned((BG, self.buffer_size), torch.int32, 0) for _ in L])
+        for nm in ("hit_num_units", "miss_num_units", "update_num_units"):
+            setattr(self, nm, [_pinned((BG,), torch.int32, 0) for _ in L])
+        self.cluster_ids = [_pinned((BG, self.nprobe), torch.int64, 0) for _ in range(2)]
+        for l in L:
+            self.wave_buffer[l].set_indices(
+                self.hit_unit_idices[l], self.hit_unit_sizes[l], self.hit_unit_sizes_cumsum[l], self.hit_num_units[l],
+                self.miss_unit_idices[l], self.miss_unit_sizes[l], self.miss_unit_sizes_cumsum[l],
+                self.miss_num_units[l], self.update_buffer_indices[l], self.update_unit_sizes[l],
+                self.update_cache_indices[l], self.update_num_units[l], self.cluster_ids[l % 2])
+        self.cache_keys = [torch.zeros((self.batch_size, self.kv_head, self.cache_size, self.page_size, D),
+                                       dtype=self.dtype, device=dev(l)) for l in L]
+        self.cache_values = [torch.zeros_like(self.cache_keys[l]) for l in L]
+        n_in = self.input_length - self.static_pattern_total
+        self.offload_keys = _pinned((self.kv_head, n_in, D), self.dtype)
+        self.offload_values = _pinned((self.kv_head, n_in, D), self.dtype)
+        self.list_keys = [_pinned((self.batch_size, self.kv_head, self.list_stride, D), self.dtype) for _ in L]
+        self.list_values = [_pinned((self.batch_size, self.kv_head, self.list_stride, D), self.dtype) for _ in L]
+        for l in L:
+            self.wave_buffer[l].set_kv(self.list_keys[l], self.list_values[l], self.offload_keys, self.offload_values)
+
+    def allocate_computation_buffer(self):
+        """Layer-shared scratch (reference: retroinfer_cache.py:302-334)."""
+        d0 = self.layer_mapping[str(0)]
+        BG, D, gs = self.batch_groups, self.head_dim, self.group_size
+        i32 = lambda *s: torch.zeros(s, dtype=torch.int32, device=d0)
+        self.logits = torch.zeros((BG, gs, self.n_centroids), dtype=torch.float32, device=d0)
+        self.cI = [torch.zeros((BG, self.max_compute_cluster_num), dtype=torch.int64, device=d0) for _ in range(2)]
+        self.ret_ids = [i32(BG, self.nprobe) for _ in range(2)]
+        self.est_ids = [i32(BG, max(self.es_cluster_num, 1)) for _ in range(2)]
+        self.valid_lengths = [i32(BG) for _ in range(2)]
+        if self.kv_residency == "device":
+            self.ret_tok_off = i32(BG, self.nprobe + 1)
+            self.row_src = i32(BG, self.buffer_size * self.page_size)
+            self.meta = i32(BG, 4)
+        else:
+            shape = (BG, self.execution_stride, 1, D)
+            self.execution_buffer_keys = [torch.zeros(shape, dtype=self.dtype, device=d0) for _ in range(2)]
+            self.execution_buffer_values = [torch.zeros(shape, dtype=self.dtype, device=d0) for _ in range(2)]
+            es = max(self.es_cluster_num, 1)
+            self.es_centroids = torch.zeros((BG, es, 1, D), dtype=self.dtype, device=d0)
+            self.es_value_sum = torch.zeros((BG, es, 1, D), dtype=self.dtype, device=d0)
+            self.es_cluster_size = torch.zeros((BG, 1, 1, es), dtype=self.dtype, device=d0)
+
+    def pre_allocate_decision(self):
+        """Kept for callers of the reference API; this build always pre-allocates."""
+        return True
+
+    def prepare_cache(self):
+        """End of prefill (reference: retroinfer_cache.py:336-365)."""
+        torch.cuda.synchronize()
+        if self.kv_residency == "host":
+            self.wave_buffer[self.layer_num - 1].construction_sync()
+        self.clusters_cpu = self.cluster_size_cpu = None
+        self.temp_keys = self.temp_values = None
+
+    # ------------------------------------------------------------------ prefill
+    def prefill_update_kv_cache(self, query_states, key_states, value_states, layer_idx, batch_idx):
+        """Clusters one sequence of one layer (reference: retroinfer_cache.py:368-441).
+        key/value_states [1, seq_len, kv_heads, dim].  Returns the K/V past valid_start."""
+        bsz, seq_len, group_num, head_dim = key_states.shape
+        assert bsz == 1, "Multi-batch prefilling only support prefill single batch one by one."
+        assert seq_len <= self.input_length, f"seq_len({seq_len}) should less than input_length({self.input_length})"
+        vs = self.valid_start[batch_idx]
+        sps, spe, spt = self.static_pattern_start, self.static_pattern_end, self.static_pattern_total
+        valid_length = seq_len - spt - vs
+        H = self.kv_head
+        rows = slice(batch_idx * H, (batch_idx + 1) * H)
+        dkey = self.layer_mapping[str(layer_idx)]
+
+        if self.kv_residency == "host":
+            # the previous construction must have consumed the shared offload buffers
+            prev = layer_idx - 1 if layer_idx > 0 else (self.layer_num - 1 if batch_idx > 0 else None)
+            if prev is not None:
+                self.wave_buffer[prev].construction_sync()
+
+        self.temp_keys = key_states[0, vs + sps:seq_len - spe].transpose(0, 1).contiguous()      # [H, N, D]
+        self.temp_values = value_states[0, vs + sps:seq_len - spe].transpose(0, 1).contiguous()
+        if self.kv_residency == "host":
+            self.mainevents[dkey].record()
+            with torch.cuda.stream(self.copystream):
+                self.mainevents[dkey].wait()
+                self.offload_keys[:, :valid_length].copy_(self.temp_keys, non_blocking=True)
+                self.offload_values[:, :valid_length].copy_(self.temp_values, non_blocking=True)
+                self.copyevents[dkey].record()
+
+        for zone, src in ((self.steady_zone_keys, key_states), (self.steady_zone_values, value_states)):
+            zone[layer_idx][batch_idx, :, :sps] = src[0, vs:vs + sps].transpose(0, 1)
+            zone[layer_idx][batch_idx, :, sps:spt] = src[0, seq_len - spe:seq_len].transpose(0, 1)
+
+        mean_key = torch.mean(self.temp_keys, dim=1, keepdim=True)
+        km = segment_k_means_csr(self.temp_keys - mean_key, self.temp_values, self.n_centroids,
+                                 num_segments=self.n_segment)
+        self.centroids[layer_idx][rows].copy_(km.centroids + mean_key)
+        self.value_sum[layer_idx][rows].copy_(km.value_sum)
+        self.centroids_mask[layer_idx][rows].copy_(km.counts == 0)
+        self.cluster_size[layer_idx][rows].copy_(km.counts.to(self.dtype))
+
+        if self.kv_residency == "device":
+            # cluster-contiguous store built on the device (stands in for organize_kv on the host)
+            lk = self.list_keys[layer_idx][batch_idx]
+            lv = self.list_values[layer_idx][batch_idx]
+            kernels.permute_rows(self.temp_keys, km.members, lk, H, valid_length, valid_length, self.list_stride)
+            kernels.permute_rows(self.temp_values, km.members, lv, H, valid_length, valid_length, self.list_stride)
+            self.cluster_start[layer_idx][rows].copy_(km.offsets[:, :self.n_centroids])
+            self.cluster_size_i32[layer_idx][rows].copy_(km.counts)
+            for h in range(H):
+                self.store_rows[layer_idx][batch_idx * H + h] = valid_length
+        else:
+            self.cluster_size_cpu = km.counts.cpu().contiguous()
+            self.clusters_cpu = csr_to_dense(km.counts, km.offsets, km.members).cpu().contiguous()
+
+        if layer_idx == self.layer_num - 1 and batch_idx + bsz == self.batch_size:
+            self.context += seq_len
+        return key_states[:, vs:], value_states[:, vs:]
+
+    def sync(self, layer_idx, batch_idx):
+        """After the prefill attention of (layer, sequence): hand the offloaded K/V to the host
+        re-organisation (reference: retroinfer_cache.py:443-458).  Nothing to do on the device."""
+        if self.kv_residency == "host":
+            self.copyevents[self.layer_mapping[str(layer_idx)]].synchronize()
+            self.wave_buffer[layer_idx].async_construction(self.clusters_cpu, self.cluster_size_cpu, batch_idx)
+
+    # ------------------------------------------------------------------ decode-time index growth
+    def _update_kv_cache(self):
+        """Folds the last THRESHOLD_LENGTH generated tokens into the index
+        (reference: retroinfer_cache.py:462-524)."""
+        sps, spe = self.static_pattern_start, self.static_pattern_end
+        BG, D, ncu = self.batch_groups, self.head_dim, self.n_centroids_per_update_segment
+        lo, hi = sps, self.static_pattern_total - spe
+        for ldx in range(self.layer_num):
+            dkey = self.layer_mapping[str(ldx)]
+            torch.cuda.set_device(dkey)
+            uk = self.steady_zone_keys[ldx][:, :, lo:hi].clone().reshape(BG, THRESHOLD_LENGTH, D).contiguous()
+            uv = self.steady_zone_values[ldx][:, :, lo:hi].clone().reshape(BG, THRESHOLD_LENGTH, D).contiguous()
+            for zone in (self.steady_zone_keys, self.steady_zone_values):   # slide the local window
+                zone[ldx][:, :, sps:sps + spe] = zone[ldx][:, :, hi:hi + spe].clone()
+            if self.kv_residency == "host":
+                self.mainevents[dkey].record()
+                with torch.cuda.stream(self.copystream):
+                    self.mainevents[dkey].wait()
+                    self.offload_update_keys.copy_(uk, non_blocking=True)
+                    self.offload_update_values.copy_(uv, non_blocking=True)
+                    self.copyevents[dkey].record()
+            mean_key = torch.mean(uk, dim=1, keepdim=True)
+            km = segment_k_means_csr(uk - mean_key, uv, ncu, num_segments=1)
+            self.centroids[ldx] = torch.cat((self.centroids[ldx], km.centroids + mean_key), dim=1)
+            self.value_sum[ldx] = torch.cat((self.value_sum[ldx], km.value_sum), dim=1)
+            self.centroids_mask[ldx] = torch.cat((self.centroids_mask[ldx], km.counts == 0), dim=1)
+            self.cluster_size[ldx] = torch.cat((self.cluster_size[ldx], km.counts.to(self.dtype)), dim=1)
+            if self.kv_residency == "device":
+                base = self.store_rows[ldx][0]
+                assert base + THRESHOLD_LENGTH <= self.list_stride, "cluster store is full"
+                lk = self.list_keys[ldx].view(BG, self.list_stride, D)[:, base:]
+                lv = self.list_values[ldx].view(BG, self.list_stride, D)[:, base:]
+                kernels.permute_rows(uk, km.members, lk, BG, THRESHOLD_LENGTH, THRESHOLD_LENGTH, self.list_stride)
+                kernels.permute_rows(uv, km.members, lv, BG, THRESHOLD_LENGTH, THRESHOLD_LENGTH, self.list_stride)
+                self.cluster_start[ldx] = torch.cat((self.cluster_start[ldx], km.offsets[:, :ncu] + base), dim=1)
+                self.cluster_size_i32[ldx] = torch.cat((self.cluster_size_i32[ldx], km.counts), dim=1)
+                self.store_rows[ldx] = [base + THRESHOLD_LENGTH] * BG
+            else:
+                self.copyevents[dkey].synchronize()
+                self.wave_buffer[ldx].update_kv(self.offload_update_keys, self.offload_update_values,
+                                                csr_to_dense(km.counts, km.offsets, km.members).cpu().contiguous(),
+                                                km.counts.cpu().contiguous())
+        torch.cuda.set_device(self.layer_mapping[str(0)])
+        self.n_centroids += ncu
+        self.logits = torch.zeros((BG, self.group_size, self.n_centroids), dtype=torch.float32,
+                                  device=self.layer_mapping[str(0)])
+        self.static_pattern_total = sps + spe
+
+    def decode_update_kv_cache(self, key_states, value_states, layer_idx):
+        """Appends the new token's K/V to the steady zone (reference: retroinfer_cache.py:527-546)."""
+        if self.static_pattern_total == self.static_pattern_start + self.static_pattern_end + THRESHOLD_LENGTH:
+            self._update_kv_cache()
+        self.steady_zone_keys[layer_idx][:, :, self.static_pattern_total] = key_states[:, 0]
+        self.steady_zone_values[layer_idx][:, :, self.static_pattern_total] = value_states[:, 0]
+        if layer_idx == self.layer_num - 1:
+            self.context += 1
+            self.static_pattern_total += 1
+        return None, None
+
+    # ------------------------------------------------------------------ decode
+    def _select(self, queries, layer, buf, with_layout):
+        BG, gs, D = self.batch_groups, self.group_size, self.head_dim
+        q = queries.view(BG, gs, D)
+        es = self.es_cluster_num
+        dev_mode = with_layout and self.kv_residency == "device"
+        kernels.score_select(
+            q, self.centroids[layer], self.centroids_mask[layer],
+            self.cluster_size_i32[layer] if dev_mode else None, self.cluster_start[layer] if dev_mode else None,
+            self.logits, None, self.cI[buf], self.ret_ids[buf], self.est_ids[buf] if es > 0 else None,
+            self.ret_tok_off if dev_mode else None, self.row_src if dev_mode else None,
+            self.meta if dev_mode else None, self.nprobe, es, self.page_size, self.buffer_size, self.RSQRT_DIM)
+
+    def compute(self, queries, layer_idx, queries_next=None):
+        """Decode attention of one layer (reference: retroinfer_cache.py:549-697).
+        queries [batch, 1, heads, dim] on the device; returns the same shape."""
+        BG, gs, D = self.batch_groups, self.group_size, self.head_dim
+        last = layer_idx == self.layer_num - 1
+        static_len = self.static_pattern_total if last else self.static_pattern_total + 1
+        buf, nbuf = layer_idx % 2, (layer_idx + 1) % 2
+        search_here = layer_idx < 2 or not self.use_cluster_estimation
+        search_next = (self.use_cluster_estimation and 0 < layer_idx < self.layer_num - 1
+                       and queries_next is not None)
+        if self.kv_residency == "device" and not self.use_cluster_estimation:
+            return self._compute_device(queries, layer_idx, static_len, buf)
+        return self._compute_staged(queries, layer_idx, queries_next, static_len, buf, nbuf, search_here,
+                                    search_next)
+
+    def _compute_device(self, queries, layer_idx, static_len, buf):
+        BG, gs, D = self.batch_groups, self.group_size, self.head_dim
+        self._select(queries, layer_idx, buf, True)
+        out = torch.empty((BG, gs, D), dtype=self.dtype, device=queries.device)
+        es = self.es_cluster_num
+        kernels.wave_attention(
+            queries.view(BG, gs, D), self.steady_zone_keys[layer_idx], self.steady_zone_values[layer_idx],
+            static_len, self.list_keys[layer_idx], self.list_values[layer_idx], self.row_src, self.meta,
+            self.est_ids[buf] if es > 0 else None, self.logits if es > 0 else None, self.value_sum[layer_idx],
+            self.cluster_size[layer_idx], out, self.valid_lengths[buf], es, self.RSQRT_DIM)
+        return out.view(self.batch_size, 1, self.num_heads, D)
+
+    # staged path: the reference's sequence of operators, one call each
+    def _search(self, queries, layer, buf):
+        self._select(queries, layer, buf, False)
+        if self.kv_residency == "host":
+            self.cluster_ids[buf].copy_(self.cI[buf][:, :self.nprobe])  # blocking copy into pinned memory
+
+    def _assemble(self, layer, buf, static_len):
+        if self.kv_residency == "host":
+            kernels.gather_copy_and_concat(
+                self.steady_zone_keys[layer], self.list_keys[layer], self.cache_keys[layer],
+                self.execution_buffer_keys[buf], self.steady_zone_values[layer], self.list_values[layer],
+                self.cache_values[layer], self.execution_buffer_values[buf],
+                self.miss_unit_idices[layer], self.miss_unit_sizes[layer], self.miss_unit_sizes_cumsum[layer],
+                self.miss_num_units[layer], self.hit_unit_idices[layer], self.hit_unit_sizes[layer],
+                self.hit_unit_sizes_cumsum[layer], self.hit_num_units[layer], self.valid_lengths[buf],
+                self.batch_groups, self.static_stride, self.list_stride, self.cache_stride, self.execution_stride,
+                self.buffer_size, static_len)
+
+    def _compute_staged(self, queries, layer_idx, queries_next, static_len, buf, nbuf, search_here, search_next):
+        BG, gs, D = self.batch_groups, self.group_size, self.head_dim
+        q4 = queries.view(BG, 1, gs, D)
+        if self.kv_residency == "device":
+            return self._compute_device_estimated(queries, layer_idx, queries_next, static_len, buf, nbuf,
+                                                  search_here, search_next)
+        if search_here:
+            self._search(queries, layer_idx, buf)
+        if search_next:
+            self._search(queries_next, layer_idx + 1, nbuf)
+        if self.es_cluster_num > 0:
+            kernels.gather_copy_vectors(
+                self.centroids[layer_idx], self.es_centroids, self.value_sum[layer_idx], self.es_value_sum,
+                self.cluster_size[layer_idx], self.es_cluster_size, self.cI[buf], BG, self.n_centroids,
+                self.es_cluster_num, self.max_compute_cluster_num, self.nprobe, self.es_cluster_num)
+            es_out, es_lse = kernels.weighted_flash_decoding(q4, self.es_centroids, self.es_value_sum,
+                                                             self.es_cluster_size, return_softmax_lse=True)
+        else:
+            es_out = es_lse = None
+        if search_here:
+            self.wave_buffer[layer_idx].batch_access()
+        if search_next:
+            self.wave_buffer[layer_idx + 1].batch_access()
+        if search_here:
+            self._assemble(layer_idx, buf, static_len)
+        if search_next:
+            cur = torch.cuda.current_stream()
+            self.copystream.wait_stream(cur)
+            with torch.cuda.stream(self.copystream):
+                self._assemble(layer_idx + 1, nbuf, static_len)
+        if not search_here:
+            # this layer's buffer was assembled on the copy stream during the previous layer
+            torch.cuda.current_stream().wait_stream(self.copystream)
+        attn = kernels.weighted_flash_decoding(
+            q4, self.execution_buffer_keys[buf], self.execution_buffer_values[buf], previous_out=es_out,
+            previous_lse=es_lse, cache_seqlens=self.valid_lengths[buf])
+        self.wave_buffer[layer_idx].sync()
+        kernels.gather_copy_and_scatter(
+            self.execution_buffer_keys[buf], self.cache_keys[layer_idx], self.execution_buffer_values[buf],
+            self.cache_values[layer_idx], self.update_buffer_indices[layer_idx], self.update_unit_sizes[layer_idx],
+            self.update_cache_indices[layer_idx], self.update_num_units[layer_idx], BG, self.execution_stride,
+            self.cache_stride, self.buffer_size, static_len)
+        return attn.view(self.batch_size, 1, self.num_heads, D)
+
+    def _compute_device_estimated(self, queries, layer_idx, queries_next, static_len, buf, nbuf, search_here,
+                                  search_next):
+        """Device residency with next-layer cluster estimation: zones come from the query the
+        previous layer predicted, scores of the estimation zone from the true query."""
+        raise NotImplementedError(
+            "use_cluster_estimation with kv_residency='device' is not available: a device-resident "
+            "store has no transfer to hide; construct the cache with use_cluster_estimation=False")

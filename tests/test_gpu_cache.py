@@ -1,0 +1,163 @@
+"""retroinfer_cache end to end on the GPU: prefill clustering, decode steps, both residencies."""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import pipeline, scoring, attention
+from oracle import kmeans as okm
+from tests.parity import check_zone_sets
+
+pytestmark = pytest.mark.gpu
+MAX_ABS, MEAN_ABS = 2e-2, 2e-3
+
+
+def _close(got, ref):
+    d = (got.float() - ref.float()).abs()
+    assert float(d.max()) <= MAX_ABS and float(d.mean()) <= MEAN_ABS, (float(d.max()), float(d.mean()))
+
+
+def _make_cache(dev, residency, layers, B, Hkv, gs, ctx, n_centroids, n_segment, nprobe, es, new=8,
+                cache_cluster_num=None):
+    from retrievalattention_amd.cache_hub import retroinfer_cache
+    return retroinfer_cache(
+        valid_start=[0] * B, layer_num=layers, batch_size=B, max_length=ctx + new, num_key_value_heads=Hkv,
+        num_heads=Hkv * gs, head_dim=128, dtype=torch.bfloat16, layer_mapping={str(l): "cuda:0" for l in range(layers)},
+        max_new_length=new, static_pattern_start=4, static_pattern_end=64, core=4, n_centroids=n_centroids,
+        n_segment=n_segment, nprobe=nprobe, max_compute_cluster_num=nprobe + es, cache_unit_size=8,
+        cache_cluster_num=cache_cluster_num if cache_cluster_num is not None else 3 * nprobe, num_gpus=1,
+        model_size=8, kv_residency=residency)
+
+
+def _prefill(cache, K, V, layers, B):
+    """K, V [layers][B] tensors [1, ctx, Hkv, 128] on the device."""
+    for b in range(B):
+        for l in range(layers):
+            cache.prefill_update_kv_cache(None, K[l][b], V[l][b], l, b)
+            cache.sync(l, b)
+    cache.prepare_cache()
+
+
+def _gen(layers, B, Hkv, gs, ctx, nmix, dev, seed):
+    from retrievalattention_amd import synth
+    K, V = [], []
+    for l in range(layers):
+        k, v, _ = synth.make_batch(seed + l, B, Hkv, ctx, nmix, gs, outliers=True)
+        K.append([k[b].transpose(0, 1)[None].contiguous().to(dev) for b in range(B)])
+        V.append([v[b].transpose(0, 1)[None].contiguous().to(dev) for b in range(B)])
+    return K, V
+
+
+@pytest.mark.parametrize("residency", ["device", "host"])
+def test_decode_matches_oracle(dev, residency):
+    """Prefill + three decode steps; every compute() is compared with the oracle's decode step
+    run on the index the cache actually holds."""
+    layers, B, Hkv, gs, ctx = 2, 2, 2, 4, 4096 + 68
+    nc, S, nprobe, es = 256, 1, 8, 60
+    cache = _make_cache(dev, residency, layers, B, Hkv, gs, ctx, nc, S, nprobe, es)
+    K, V = _gen(layers, B, Hkv, gs, ctx, 256, dev, 0)
+    _prefill(cache, K, V, layers, B)
+    assert cache.context == ctx
+    BG = B * Hkv
+    g = torch.Generator().manual_seed(9)
+    # the oracle needs the cluster-contiguous store: rebuild it on the CPU from the cache's assignment
+    stores = []
+    for l in range(layers):
+        sk, sv, st = [], [], []
+        for b in range(B):
+            for h in range(Hkv):
+                keys = K[l][b][0, 4:ctx - 64, h].cpu(); vals = V[l][b][0, 4:ctx - 64, h].cpu()
+                mean = torch.mean(keys[None], dim=1, keepdim=True)
+                a, _, _ = okm.assign(keys - mean[0], (cache.centroids[l][b * Hkv + h].cpu() - mean[0]))
+                # use the sizes the cache reports; order inside a cluster = ascending token id
+                size = cache.cluster_size[l][b * Hkv + h].cpu().float().to(torch.int64)
+                if residency == "device":
+                    gi = b * Hkv + h
+                    rows = int(cache.store_rows[l][gi])
+                    sk.append(cache.list_keys[l].view(BG, -1, 128)[gi, :rows].cpu())
+                    sv.append(cache.list_values[l].view(BG, -1, 128)[gi, :rows].cpu())
+                else:
+                    gi = b * Hkv + h
+                    rows = int(size.sum())
+                    sk.append(cache.list_keys[l].view(BG, -1, 128)[gi, :rows].clone())
+                    sv.append(cache.list_values[l].view(BG, -1, 128)[gi, :rows].clone())
+                st.append(torch.cumsum(size, 0) - size)
+                # the store is a permutation of the clustered tokens
+                assert torch.equal(torch.sort(sk[-1].float().sum(1)).values, torch.sort(keys.float().sum(1)).values)
+        stores.append((sk, sv, torch.stack(st)))
+    for step in range(3):
+        for l in range(layers):
+            k_new = torch.randn(B, 1, Hkv, 128, generator=g).to(torch.bfloat16)
+            v_new = torch.randn(B, 1, Hkv, 128, generator=g).to(torch.bfloat16)
+            q = torch.randn(B, 1, Hkv * gs, 128, generator=g).to(torch.bfloat16)
+            cache.decode_update_kv_cache(k_new.to(dev), v_new.to(dev), l)
+            out = cache.compute(q.to(dev), l)
+            torch.cuda.synchronize()
+            static_len = cache.static_pattern_total if l == layers - 1 else cache.static_pattern_total + 1
+            if l == layers - 1:
+                static_len = cache.static_pattern_total  # already advanced by decode_update_kv_cache
+            size_bf = cache.cluster_size[l].cpu()
+            size_i = size_bf.float().to(torch.int32)
+            ref, aux = pipeline.decode_step(
+                q.view(BG, gs, 128), cache.steady_zone_keys[l].view(BG, -1, 128).cpu(),
+                cache.steady_zone_values[l].view(BG, -1, 128).cpu(), static_len, cache.centroids[l].cpu(),
+                cache.value_sum[l].cpu(), cache.centroids_mask[l].cpu(), size_i, size_bf, stores[l][0], stores[l][1],
+                stores[l][2], nprobe, es, 8, cache.buffer_size, logits=cache.logits.cpu())
+            _close(out.cpu().view(BG, gs, 128), ref)
+            buf = l % 2
+            assert torch.equal(cache.cI[buf][:, :nprobe].cpu(), aux["ret"])
+            assert torch.equal(cache.cI[buf][:, nprobe:].cpu(), aux["est"])
+            assert torch.equal(cache.valid_lengths[buf].cpu().long(), static_len + aux["offs"][:, -1])
+    assert cache.context == ctx + 3
+
+
+def test_full_retrieval_equals_dense_attention(dev):
+    """Property (v): probing every cluster with no estimation zone is dense attention over
+    steady zone + all clustered tokens, whatever the partition."""
+    layers, B, Hkv, gs, ctx = 1, 1, 2, 4, 2048 + 68
+    nc = 128
+    cache = _make_cache(dev, "device", layers, B, Hkv, gs, ctx, nc, 1, nc, 0)
+    cache.buffer_size = 10 ** 6 // 8   # no page cut-off
+    cache.allocate_computation_buffer()
+    K, V = _gen(layers, B, Hkv, gs, ctx, 100, dev, 3)
+    _prefill(cache, K, V, layers, B)
+    g = torch.Generator().manual_seed(1)
+    q = torch.randn(B, 1, Hkv * gs, 128, generator=g).to(torch.bfloat16)
+    kn = torch.randn(B, 1, Hkv, 128, generator=g).to(torch.bfloat16)
+    vn = torch.randn(B, 1, Hkv, 128, generator=g).to(torch.bfloat16)
+    cache.decode_update_kv_cache(kn.to(dev), vn.to(dev), 0)
+    out = cache.compute(q.to(dev), 0).cpu()
+    kk = torch.cat([K[0][0][0].cpu(), kn[0]], 0).transpose(0, 1)   # [Hkv, ctx+1, D]
+    vv = torch.cat([V[0][0][0].cpu(), vn[0]], 0).transpose(0, 1)
+    ref = torch.nn.functional.scaled_dot_product_attention(
+        q.view(Hkv, gs, 128).float(), kk.float(), vv.float())
+    _close(out.view(Hkv, gs, 128), ref)
+
+
+def test_host_and_device_residency_agree_and_cache_warms(dev):
+    """Same inputs through both residencies: identical selections, outputs within tolerance;
+    repeated queries turn misses into hits in the LRU block cache."""
+    layers, B, Hkv, gs, ctx = 1, 2, 2, 7, 3072 + 68
+    nc, nprobe, es = 192, 6, 40
+    K, V = _gen(layers, B, Hkv, gs, ctx, 192, dev, 5)
+    cd = _make_cache(dev, "device", layers, B, Hkv, gs, ctx, nc, 1, nprobe, es)
+    ch = _make_cache(dev, "host", layers, B, Hkv, gs, ctx, nc, 1, nprobe, es)
+    _prefill(cd, K, V, layers, B)
+    _prefill(ch, K, V, layers, B)
+    assert torch.equal(cd.centroids[0], ch.centroids[0])
+    g = torch.Generator().manual_seed(2)
+    q = torch.randn(B, 1, Hkv * gs, 128, generator=g).to(torch.bfloat16).to(dev)
+    kn = torch.randn(B, 1, Hkv, 128, generator=g).to(torch.bfloat16).to(dev)
+    vn = torch.randn(B, 1, Hkv, 128, generator=g).to(torch.bfloat16).to(dev)
+    hits = []
+    for step in range(3):
+        for c in (cd, ch):
+            c.decode_update_kv_cache(kn, vn, 0)
+        od, oh = cd.compute(q, 0), ch.compute(q, 0)
+        torch.cuda.synchronize()
+        _close(oh.cpu(), od.cpu())
+        assert torch.equal(cd.cI[0].cpu(), ch.cI[0].cpu())
+        assert torch.equal(cd.valid_lengths[0].cpu(), ch.valid_lengths[0].cpu())
+        hits.append(int(ch.hit_num_units[0].sum()))
+    assert hits[0] == 0 and hits[1] > 0 and hits[2] >= hits[1]
