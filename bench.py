@@ -1,0 +1,261 @@
+"""Benchmark of the wave-index decode attention step on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config c2|c1|c4|c5] [--layers L]
+
+A step is one layer's decode attention (retroinfer_cache.compute) for the whole batch: centroid
+scoring, zone selection, estimation zone and attention over steady zone + retrieved clusters,
+with the index and all K/V resident in HBM before the timed region.  Step i runs layer
+i mod L; every layer has its own seeded synthetic K/V and index, built by the library's own
+prefill k-means.  Prints one JSON line (see the keys at the bottom).
+"""
+import argparse
+import json
+import math
+import os
+import sys
+import time
+
+import torch
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK = 8.0e12  # bytes/s, MI355X
+
+CONFIGS = {
+    # name: batch, kv heads, group size, clustered tokens, mixture centres, centroids, segments, outliers, layers
+    "c1": dict(B=1, Hkv=8, gs=4, N=8192, K=512, nc=512, S=1, outliers=False, L=1,
+               desc="Llama-3-8B shape, batch 1, 8192 tokens, 512 centroids"),
+    "c2": dict(B=4, Hkv=8, gs=4, N=131072, K=8192, nc=8192, S=16, outliers=True, L=32,
+               desc="Llama-3-8B shape (32 q / 8 kv heads, dim 128), batch 4, 131072 tokens, 8192 centroids"),
+    "c4": dict(B=16, Hkv=4, gs=7, N=61440, K=3840, nc=3840, S=8, outliers=False, L=28,
+               desc="Qwen2.5-7B shape, batch 16, 61440 tokens, 3840 centroids (device-resident variant)"),
+    "c5": dict(B=8, Hkv=8, gs=8, N=262144, K=16384, nc=16384, S=32, outliers=True, L=1,
+               desc="Qwen2.5-72B single layer, batch 8, 262144 tokens, 16384 centroids"),
+}
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def build_cache(cfg, L, dev):
+    from retrievalattention_amd import synth
+    from retrievalattention_amd.cache_hub import retroinfer_cache
+    B, Hkv, gs, N = cfg["B"], cfg["Hkv"], cfg["gs"], cfg["N"]
+    nprobe = max(1, int(cfg["nc"] * 0.018))
+    es = int(cfg["nc"] * 0.232)
+    ctx = N + synth.STEADY_START + synth.STEADY_END
+    new = 2
+    cache = retroinfer_cache(
+        valid_start=[0] * B, layer_num=L, batch_size=B, max_length=ctx + new, num_key_value_heads=Hkv,
+        num_heads=Hkv * gs, head_dim=128, dtype=torch.bfloat16, layer_mapping={str(l): "cuda:0" for l in range(L)},
+        max_new_length=new, static_pattern_start=synth.STEADY_START, static_pattern_end=synth.STEADY_END, core=8,
+        n_centroids=cfg["nc"], n_segment=cfg["S"], nprobe=nprobe, max_compute_cluster_num=nprobe + es,
+        cache_unit_size=8, cache_cluster_num=3 * nprobe, num_gpus=1, model_size=0, kv_residency="device")
+    queries = []
+    t0 = time.time()
+    for l in range(L):
+        qs = []
+        for b in range(B):
+            ks, vs = [], []
+            for h in range(Hkv):
+                k, v, q = synth.make_group(l, b, h, N, cfg["K"], gs, outliers=cfg["outliers"],
+                                           n_extra=synth.STEADY_START + synth.STEADY_END, device=dev)
+                # steady zone = the extra tokens: 4 first, 64 last
+                k = torch.cat([k[N:N + 4], k[:N], k[N + 4:]]).to(torch.bfloat16)
+                v = torch.cat([v[N:N + 4], v[:N], v[N + 4:]]).to(torch.bfloat16)
+                ks.append(k); vs.append(v); qs.append(q.to(torch.bfloat16))
+            K = torch.stack(ks, 1)[None].contiguous()   # [1, ctx, Hkv, D]
+            V = torch.stack(vs, 1)[None].contiguous()
+            cache.prefill_update_kv_cache(None, K, V, l, b)
+            cache.sync(l, b)
+            del K, V, ks, vs
+        queries.append(torch.cat(qs).view(B, 1, Hkv * gs, 128).contiguous())
+        if l == 0 or (l + 1) % 8 == 0:
+            torch.cuda.synchronize()
+            log(f"[bench] built layer {l + 1}/{L} ({time.time() - t0:.1f}s)")
+    cache.prepare_cache()
+    cache.temp_keys = cache.temp_values = None
+    torch.cuda.empty_cache()
+    # one generated token per layer so that the steady zone has its 69th entry
+    g = torch.Generator(device=dev).manual_seed(12345)
+    for l in range(L):
+        kn = torch.randn(B, 1, Hkv, 128, generator=g, device=dev).to(torch.bfloat16)
+        vn = torch.randn(B, 1, Hkv, 128, generator=g, device=dev).to(torch.bfloat16)
+        cache.decode_update_kv_cache(kn, vn, l)
+    return cache, queries, nprobe, es
+
+
+def algorithmic_bytes(cache, cfg, nprobe, es, layer, static_len):
+    """HBM bytes one decode layer-step has to touch: centroids once, queries, mask, value-sum rows
+    and sizes of the estimation zone, K and V of retrieved + steady tokens once, output."""
+    BG, gs, nc, D, e = cfg["B"] * cfg["Hkv"], cfg["gs"], cfg["nc"], 128, 2
+    t_ret = cache.meta[:, 1].sum().item()
+    parts = {
+        "centroids": BG * nc * D * e + BG * gs * D * e + BG * nc,
+        "estimation": BG * es * (D * e + e),
+        "kv": 2 * e * D * (t_ret + BG * static_len),
+        "out": BG * gs * D * e,
+    }
+    return parts, t_ret
+
+
+def time_region(fn, iters):
+    torch.cuda.synchronize()
+    s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    s.record()
+    for _ in range(iters):
+        fn()
+    e.record()
+    torch.cuda.synchronize()
+    return s.elapsed_time(e) * 1e-3 / iters
+
+
+def cpu_baseline(cache, cfg, queries, nprobe, es, static_len, max_seconds=30.0):
+    """The CPU restatement (oracle/) of the same decode step, layer 0, on the host cores."""
+    from oracle import pipeline
+    BG, gs = cfg["B"] * cfg["Hkv"], cfg["gs"]
+    torch.set_num_threads(os.cpu_count() or 1)
+    l = 0
+    rows = cache.store_rows[l]
+    sk = [cache.list_keys[l].view(BG, -1, 128)[g, :rows[g]].cpu() for g in range(BG)]
+    sv = [cache.list_values[l].view(BG, -1, 128)[g, :rows[g]].cpu() for g in range(BG)]
+    args = (queries[l].view(BG, gs, 128).cpu(), cache.steady_zone_keys[l].view(BG, -1, 128).cpu(),
+            cache.steady_zone_values[l].view(BG, -1, 128).cpu(), static_len, cache.centroids[l].cpu(),
+            cache.value_sum[l].cpu(), cache.centroids_mask[l].cpu(), cache.cluster_size_i32[l].cpu(),
+            cache.cluster_size[l].cpu(), sk, sv, cache.cluster_start[l].cpu().long(), nprobe, es, 8,
+            cache.buffer_size)
+    pipeline.decode_step(*args)  # warm-up
+    times = []
+    t_all = time.time()
+    while len(times) < 5 and time.time() - t_all < max_seconds:
+        t0 = time.time()
+        ref, _ = pipeline.decode_step(*args)
+        times.append(time.time() - t0)
+    times.sort()
+    return times[len(times) // 2], len(times), ref
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=640)
+    ap.add_argument("--warmup", type=int, default=64)
+    ap.add_argument("--config", default="c2", choices=sorted(CONFIGS))
+    ap.add_argument("--layers", type=int, default=0, help="distinct layers (default: the config's)")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-graph", action="store_true", help="time eager launches instead of HIP graph replays")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py measures one GPU: the wave-index path has no cross-GPU exchange (run with --gpus 1)")
+    if not torch.cuda.is_available():
+        sys.exit("bench.py needs a GPU")
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    cfg = CONFIGS[args.config]
+    L = args.layers or cfg["L"]
+    B, Hkv, gs = cfg["B"], cfg["Hkv"], cfg["gs"]
+    BG = B * Hkv
+    cache, queries, nprobe, es = build_cache(cfg, L, dev)
+    static_len = cache.static_pattern_total  # 4 + 64 + the token being decoded (already counted)
+
+    # every layer-step is "not the last layer" for timing purposes: same static_len everywhere
+    def step(l):
+        return cache._compute_device(queries[l], l, static_len, l % 2)
+
+    outs = [step(l) for l in range(L)]
+    torch.cuda.synchronize()
+
+    graphs = None
+    if not args.no_graph:
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            for l in range(L):
+                step(l)
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        graphs = []
+        for l in range(L):
+            gr = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(gr):
+                o = step(l)
+            graphs.append((gr, o))
+        torch.cuda.synchronize()
+        # replays must reproduce the eager result
+        for l in range(L):
+            graphs[l][0].replay()
+        torch.cuda.synchronize()
+        for l in range(L):
+            if not torch.equal(graphs[l][1], outs[l]):
+                sys.exit(f"graph replay of layer {l} differs from the eager result")
+
+    def run(i):
+        l = i % L
+        if graphs is not None:
+            graphs[l][0].replay()
+        else:
+            step(l)
+
+    for i in range(args.warmup):
+        run(i)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(args.steps):
+        run(i)
+    torch.cuda.synchronize()
+    t_step = (time.perf_counter() - t0) / args.steps
+
+    # per-kernel timings with events on the launch stream, each stage alone
+    from retrievalattention_amd import kernels
+    l0 = 0
+    t_select = time_region(lambda: cache._select(queries[l0], l0, 0, True), 200)
+    out_tmp = torch.empty((BG, gs, 128), dtype=torch.bfloat16, device=dev)
+    t_attn = time_region(lambda: kernels.wave_attention(
+        queries[l0].view(BG, gs, 128), cache.steady_zone_keys[l0], cache.steady_zone_values[l0], static_len,
+        cache.list_keys[l0], cache.list_values[l0], cache.row_src, cache.meta, cache.est_ids[0], cache.logits,
+        cache.value_sum[l0], cache.cluster_size[l0], out_tmp, cache.valid_lengths[0], es, cache.RSQRT_DIM), 200)
+    cache._select(queries[l0], l0, 0, True)
+    torch.cuda.synchronize()
+    parts, t_ret = algorithmic_bytes(cache, cfg, nprobe, es, l0, static_len)
+    total_bytes = sum(parts.values())
+    score_bytes = parts["centroids"]
+    attn_bytes = parts["estimation"] + parts["kv"] + parts["out"]
+
+    Lmodel = cfg["L"]
+    tokens_per_s = B / (Lmodel * t_step)
+    result = {
+        "metric": "decode tokens/s at 128K ctx (attention only, B / (L * t_layer_step)); us/layer-step and % HBM roofline alongside",
+        "value": tokens_per_s, "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": t_step * 1e3, "us_per_layer_step": t_step * 1e6, "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": f"{args.config}: {cfg['desc']}; nprobe {nprobe}, estimation zone {es}, "
+                               f"steady zone {static_len}, {L} layers with independent seeds, "
+                               f"{'HIP graph replay' if graphs is not None else 'eager launches'}",
+                   "batch": B, "context_tokens": cfg["N"], "layers_for_tokens_per_s": Lmodel,
+                   "retrieved_tokens_per_group": t_ret / BG},
+        "step_roofline": {"bound": "hbm", "algorithmic_bytes": total_bytes, "achieved": total_bytes / t_step / 1e9,
+                          "peak": HBM_PEAK / 1e9, "unit": "GB/s", "frac": total_bytes / t_step / HBM_PEAK},
+        "stages": {
+            "score_select": {"us": t_select * 1e6, "algorithmic_bytes": score_bytes,
+                             "GBps": score_bytes / t_select / 1e9},
+            "wave_attention": {"us": t_attn * 1e6, "algorithmic_bytes": attn_bytes,
+                               "GBps": attn_bytes / t_attn / 1e9},
+        },
+    }
+    dom = max(result["stages"].items(), key=lambda kv: kv[1]["us"])
+    result["roofline"] = {"bound": "hbm", "kernel": dom[0], "achieved": dom[1]["GBps"], "peak": HBM_PEAK / 1e9,
+                          "unit": "GB/s", "frac": dom[1]["GBps"] * 1e9 / HBM_PEAK, "traffic": None}
+    if not args.no_cpu_baseline:
+        t_cpu, n, ref = cpu_baseline(cache, cfg, queries, nprobe, es, static_len)
+        d = (outs[0].view(BG, gs, 128).cpu().float() - ref.float()).abs()
+        result["cpu_baseline"] = {"value": B / (Lmodel * t_cpu), "unit": "tokens/s", "us_per_layer_step": t_cpu * 1e6,
+                                  "cores": torch.get_num_threads(), "kind": "port",
+                                  "sample": f"median of {n} full-shape decode layer-steps of layer 0 (oracle/pipeline.py)",
+                                  "max_abs_vs_gpu": float(d.max()), "mean_abs_vs_gpu": float(d.mean())}
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

@@ -103,7 +103,11 @@ int ri_score_select(const void* q, const void* centroids, const uint8_t* mask,
  *   rows), prev_out [BG, gs, 128] bf16 + prev_lse [BG, gs] fp32 or both NULL,
  *   out [BG, gs, 128] bf16, lse_out [BG, gs] fp32 or NULL.
  *   out = (e^{prev_lse}·prev_out + Σ_r e^{s_r} v_r) / (e^{prev_lse} + Σ_r w_r e^{s_r}),
- *   s_r = scale·q·k_r;  lse_out = log of that denominator. */
+ *   s_r = scale·q·k_r;  lse_out = log of that denominator.
+ *   workspace: ri_flash_decoding_workspace_bytes(BG, gs) bytes of device memory that the
+ *   caller zeroes once after allocating it (its head holds per-group arrival counters which
+ *   every call leaves at zero again); calls sharing a workspace must not overlap in time.
+ *   BG <= 4096. */
 size_t ri_flash_decoding_workspace_bytes(int BG, int gs);
 int ri_weighted_flash_decoding(const void* q, const void* k, const void* v, const void* weight,
                                const int32_t* cache_seqlens, const void* prev_out,
@@ -121,7 +125,8 @@ int ri_weighted_flash_decoding(const void* q, const void* k, const void* v, cons
  *   row_src, meta, est_ids, logits: as written by ri_score_select
  *   value_sum [BG, nc, 128] bf16, cluster_size_bf16 [BG, nc] bf16 (estimation weights)
  *   es may be 0 (no estimation zone).  out [BG, gs, 128] bf16; valid_lengths [BG] int32 or
- *   NULL receives static_len + retrieved tokens (what gather_copy_and_concat reports). */
+ *   NULL receives static_len + retrieved tokens (what gather_copy_and_concat reports).
+ *   workspace: same rules as ri_weighted_flash_decoding (zeroed once by the caller). */
 size_t ri_wave_attention_workspace_bytes(int BG, int gs);
 int ri_wave_attention(const void* q, const void* steady_k, const void* steady_v,
                       int64_t steady_stride, int static_len, const void* store_k,

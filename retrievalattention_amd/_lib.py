@@ -50,6 +50,9 @@ def lib():
     """Loads the shared library once and declares every entry point."""
     global _lib
     if _lib is None:
+        # torch ships its own HIP runtime; it has to be in the process first so that the library
+        # binds to that one instead of bringing a second runtime with no device context
+        import torch  # noqa: F401
         if not os.path.exists(LIB_PATH):
             raise RuntimeError(
                 f"{LIB_PATH} is missing: build it with `python -m retrievalattention_amd.build` "

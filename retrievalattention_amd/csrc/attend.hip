@@ -1,7 +1,10 @@
 // Weighted flash decoding for the wave index (gfx950).
 //
 // One kernel serves every attention call of the decode step.  A workgroup (4 waves) takes
-// one split of one group's rows; a wave walks its rows in chunks of 16:
+// one split of one group's rows; a wave owns a contiguous run of rows and walks it in batches
+// of 64 rows = 4 chunks of 16.  For a batch it first fetches one row descriptor per lane
+// (where the row lives), then issues every K and V load of the batch before it computes, so
+// that a short kernel keeps enough bytes in flight to load HBM:
 //   * key/value rows ("KV" splits): scores = scale * q·k on bf16 MFMA 16x16x32 with the
 //     query heads as the A rows and 16 key rows as the B columns, so each lane ends up with
 //     the scores of one key row for four heads;
@@ -9,13 +12,18 @@
 //     by the scoring kernel, the "value" row is the cluster's value sum and the softmax
 //     denominator is weighted by the cluster size.
 // P·V runs on the vector ALU in fp32: lane (c, h) accumulates dims 8c..8c+7 over rows
-// h, h+4, h+8, h+12 of each chunk, for all heads.  Splits write (max, denominator,
-// numerator) partials; combine_kernel merges them (and an optional previous result) with the
-// usual log-sum-exp rule.
+// h, h+4, h+8, h+12 of each chunk, for all heads.  Every workgroup writes a
+// (max, denominator, numerator) partial; the workgroup that finishes last for a group merges
+// the partials (and an optional previous result) with the log-sum-exp rule and writes the
+// output, so the whole call is one launch.
 //
 // Semantics follow the weighted_flash_decoding call sites at
 // cache_hub/retroinfer_cache.py:611-617 and :666-674.
+#include <stdlib.h>
+
 #include "ri_common.h"
+
+#define ATT_FLAG_A 0x40000000  // descriptor bit: row lives in region A
 
 struct AttendParams {
   const uint16_t* q;  // [BG, gs, 128]
@@ -37,19 +45,27 @@ struct AttendParams {
   const uint16_t* weightB;  // [BG, weight_stride] bf16 per region-B row, or null
   int weight_stride;
   // estimation rows
-  const int32_t* est_ids;  // [BG, es]
-  const float* logits;     // [BG, gs, nc]
+  const int32_t* est_ids;     // [BG, es]
+  const float* logits;        // [BG, gs, nc]
   const uint16_t* value_sum;  // [BG, nc, 128]
   const uint16_t* csize;      // [BG, nc] bf16
   int nc;
   int es;
-  // partials
+  // partials and the per-group arrival counters (zero between launches)
   float* part_ml;   // [BG, S, GS_PAD, 2]
   float* part_acc;  // [BG, S, GS_PAD, 128]
+  int* counters;    // [BG]
   int S_kv;
   int S_es;
   int gs;
+  int fuse;  // 1: the last workgroup of a group merges; 0: a separate combine launch does
   float scale;
+  // epilogue
+  const uint16_t* prev_out;  // [BG, gs, 128] or null
+  const float* prev_lse;     // [BG, gs] or null
+  uint16_t* out;             // [BG, gs, 128]
+  float* lse_out;            // [BG, gs] or null
+  int32_t* valid_lengths;    // [BG] or null: lenA + lenB(g)
 };
 
 template <int GS_PAD>
@@ -122,13 +138,61 @@ __device__ __forceinline__ void chunk_update(WaveState<GS_PAD>& st, const float 
   __builtin_amdgcn_wave_barrier();  // p_sh is rewritten by the next chunk
 }
 
+// rows of a wave: the group's `total` rows are cut into `nwaves` runs of a multiple of 16 rows
+__device__ __forceinline__ void wave_rows(int total, int nwaves, int wid, int* r0, int* r1) {
+  int rpw = (total + nwaves - 1) / nwaves;
+  rpw = (rpw + 15) & ~15;
+  *r0 = min(total, wid * rpw);
+  *r1 = min(total, *r0 + rpw);
+}
+
+// Merges the S split partials of group g (and the optional previous result) and writes the
+// output; called by all 256 threads of one workgroup.
 template <int GS_PAD>
-__global__ __launch_bounds__(256) void attend_kernel(AttendParams P) {
+__device__ __forceinline__ void combine_group(const AttendParams& P, int g, int S, int lenB) {
+  const int gs = P.gs;
+  for (int idx = threadIdx.x; idx < gs * (RI_DIM / 2); idx += 256) {
+    const int j = idx / (RI_DIM / 2), d2 = (idx % (RI_DIM / 2)) * 2;
+    const float* ml = P.part_ml + ((size_t)g * S * GS_PAD + j) * 2;
+    const float* pa = P.part_acc + ((size_t)g * S * GS_PAD + j) * RI_DIM + d2;
+    float M = P.prev_lse ? P.prev_lse[(size_t)g * gs + j] : -INFINITY;
+#pragma unroll 8
+    for (int s = 0; s < S; ++s) M = fmaxf(M, ml[(size_t)s * GS_PAD * 2]);
+    float L = 0.f, A0 = 0.f, A1 = 0.f;
+    if (P.prev_lse) {
+      const float pl = P.prev_lse[(size_t)g * gs + j];
+      const float f = (pl == -INFINITY) ? 0.f : __expf(pl - M);
+      const uint32_t po = *reinterpret_cast<const uint32_t*>(P.prev_out + ((size_t)g * gs + j) * RI_DIM + d2);
+      L = f;
+      A0 = f * __uint_as_float(po << 16);
+      A1 = f * __uint_as_float(po & 0xffff0000u);
+    }
+#pragma unroll 8
+    for (int s = 0; s < S; ++s) {
+      const float m = ml[(size_t)s * GS_PAD * 2];
+      const float f = (m == -INFINITY) ? 0.f : __expf(m - M);
+      const float2 a2 = *reinterpret_cast<const float2*>(pa + (size_t)s * GS_PAD * RI_DIM);
+      L += ml[(size_t)s * GS_PAD * 2 + 1] * f;
+      A0 += a2.x * f;
+      A1 += a2.y * f;
+    }
+    const uint32_t o = (uint32_t)ri_f32_to_bf16(A0 / L) | ((uint32_t)ri_f32_to_bf16(A1 / L) << 16);
+    *reinterpret_cast<uint32_t*>(P.out + ((size_t)g * gs + j) * RI_DIM + d2) = o;
+    if (d2 == 0 && P.lse_out) P.lse_out[(size_t)g * gs + j] = M + __logf(L);
+  }
+  if (threadIdx.x == 0 && P.valid_lengths) P.valid_lengths[g] = P.lenA + lenB;
+}
+
+// CH = chunks (of 16 rows) a wave loads ahead of computing
+template <int GS_PAD, int CH>
+__global__ __launch_bounds__(256, 2) void attend_kernel(AttendParams P) {
   __shared__ float sh_p[4][16 * GS_PAD];
   __shared__ float sh_al[4][GS_PAD];
   __shared__ float sh_m[4][GS_PAD];
   __shared__ float sh_l[4][GS_PAD];
   __shared__ float sh_acc[4][GS_PAD][RI_DIM];
+  __shared__ __attribute__((aligned(16))) uint16_t sh_q[GS_PAD][RI_DIM];
+  __shared__ int sh_last;
 
   const int g = blockIdx.y;
   const int split = blockIdx.x;
@@ -136,6 +200,7 @@ __global__ __launch_bounds__(256) void attend_kernel(AttendParams P) {
   const int wave = threadIdx.x >> 6;
   const int n = lane & 15, h = lane >> 4;
   const int gs = P.gs;
+  constexpr int ND = (CH * 16 + 63) / 64;  // descriptor registers per batch
 
   WaveState<GS_PAD> st;
 #pragma unroll
@@ -147,26 +212,23 @@ __global__ __launch_bounds__(256) void attend_kernel(AttendParams P) {
 
   float* p_sh = sh_p[wave];
   float* al_sh = sh_al[wave];
+  const int lenB = P.lenB_ptr ? P.lenB_ptr[(size_t)g * P.lenB_ptr_stride] : P.lenB_const;
 
   if (split < P.S_kv) {
     // ---------------- key/value rows ----------------
-    const int lenB = P.lenB_ptr ? P.lenB_ptr[(size_t)g * P.lenB_ptr_stride] : P.lenB_const;
     const int total = P.lenA + lenB;
-    const int chunks = (total + 15) >> 4;
-    const int nwaves = P.S_kv * 4;
-    const int cpw = (chunks + nwaves - 1) / nwaves;
-    const int wid = split * 4 + wave;
-    const int cb = wid * cpw;
-    const int ce = min(chunks, cb + cpw);
+    int r0, r1;
+    wave_rows(total, P.S_kv * 4, split * 4 + wave, &r0, &r1);
 
-    // A operand: query heads; row m of the MFMA holds head m % GS_PAD (zero if >= gs)
-    uint4 aq[4];
-    {
-      const int head = n % GS_PAD;
-      const uint16_t* qp = P.q + ((size_t)g * gs + head) * RI_DIM + h * 8;
-#pragma unroll
-      for (int kk = 0; kk < 4; ++kk) aq[kk] = (head < gs) ? ri_ld16(qp + kk * 32) : ri_zero16();
+    // A operand: query heads through LDS (read again per chunk: registers go to the loads);
+    // row m of the MFMA holds head m % GS_PAD, zero if >= gs
+    for (int i = threadIdx.x; i < GS_PAD * (RI_DIM / 8); i += 256) {
+      const int head = i / (RI_DIM / 8), piece = i % (RI_DIM / 8);
+      *reinterpret_cast<uint4*>(&sh_q[head][piece * 8]) =
+          (head < gs) ? ri_ld16(P.q + ((size_t)g * gs + head) * RI_DIM + piece * 8) : ri_zero16();
     }
+    __syncthreads();
+    const uint16_t* qrow = &sh_q[n % GS_PAD][h * 8];
     const uint16_t* kA = P.kA + (size_t)g * P.strideA * RI_DIM;
     const uint16_t* vA = P.vA + (size_t)g * P.strideA * RI_DIM;
     const uint16_t* kB = P.kB + (size_t)g * P.strideB * RI_DIM;
@@ -174,84 +236,107 @@ __global__ __launch_bounds__(256) void attend_kernel(AttendParams P) {
     const int32_t* rs = P.row_src ? P.row_src + (size_t)g * P.rs_stride : nullptr;
     const uint16_t* wB = P.weightB ? P.weightB + (size_t)g * P.weight_stride : nullptr;
 
-    for (int c = cb; c < ce; ++c) {
-      // key row of this lane
-      const int row = c * 16 + n;
-      const bool valid = row < total;
-      const uint16_t* kp = nullptr;
-      float w = 1.f;
-      if (valid) {
-        if (row < P.lenA) {
-          kp = kA + (size_t)row * RI_DIM;
-        } else {
-          const int rb = row - P.lenA;
-          const int src = rs ? rs[rb] : rb;
-          kp = kB + (size_t)src * RI_DIM;
-          if (wB) w = ri_bf16_to_f32(wB[rb]);
-        }
-      }
-      uint4 bk[4];
+    for (int b0 = r0; b0 < r1; b0 += 16 * CH) {
+      // descriptors, one row per lane and register: where row b0 + 64*k + lane lives (-1 = past the end)
+      int desc[ND];
+      float wd[ND];
 #pragma unroll
-      for (int kk = 0; kk < 4; ++kk) bk[kk] = valid ? ri_ld16(kp + kk * 32 + h * 8) : ri_zero16();
-      // value rows of this lane: rows h, h+4, h+8, h+12 of the chunk, dims 8n..8n+7
-      uint4 v[4];
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const int vr = c * 16 + h + 4 * i;
-        if (vr < total) {
-          const uint16_t* vp;
-          if (vr < P.lenA) {
-            vp = vA + (size_t)vr * RI_DIM;
+      for (int k = 0; k < ND; ++k) {
+        desc[k] = -1;
+        wd[k] = 1.f;
+        const int row = b0 + 64 * k + lane;
+        if (row < r1 && 64 * k + lane < 16 * CH) {
+          if (row < P.lenA) {
+            desc[k] = row | ATT_FLAG_A;
           } else {
-            const int rb = vr - P.lenA;
-            vp = vB + (size_t)(rs ? rs[rb] : rb) * RI_DIM;
+            const int rb = row - P.lenA;
+            desc[k] = rs ? rs[rb] : rb;
+            if (wB) wd[k] = ri_bf16_to_f32(wB[rb]);
           }
-          v[i] = ri_ld16(vp + n * 8);
-        } else {
-          v[i] = ri_zero16();
         }
       }
-      f32x4_t acc = (f32x4_t){0.f, 0.f, 0.f, 0.f};
+      const int nch = min(CH, (r1 - b0 + 15) >> 4);
+      uint4 bk[CH][4], v[CH][4];
 #pragma unroll
-      for (int kk = 0; kk < 4; ++kk)
-        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ri_as_bf16x8(aq[kk]), ri_as_bf16x8(bk[kk]), acc, 0, 0, 0);
-      const float s[4] = {acc[0] * P.scale, acc[1] * P.scale, acc[2] * P.scale, acc[3] * P.scale};
-      chunk_update<GS_PAD>(st, s, valid, w, v, p_sh, al_sh, lane);
+      for (int ch = 0; ch < CH; ++ch) {
+        if (ch < nch) {
+          const int dk = __shfl(desc[ch / 4], (ch % 4) * 16 + n);
+          const uint16_t* kp = ((dk & ATT_FLAG_A) ? kA : kB) + (size_t)(dk & ~ATT_FLAG_A) * RI_DIM + h * 8;
+#pragma unroll
+          for (int kk = 0; kk < 4; ++kk) bk[ch][kk] = (dk >= 0) ? ri_ld16(kp + kk * 32) : ri_zero16();
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            const int dv = __shfl(desc[ch / 4], (ch % 4) * 16 + h + 4 * i);
+            const uint16_t* vp = ((dv & ATT_FLAG_A) ? vA : vB) + (size_t)(dv & ~ATT_FLAG_A) * RI_DIM + n * 8;
+            v[ch][i] = (dv >= 0) ? ri_ld16(vp) : ri_zero16();
+          }
+        }
+      }
+#pragma unroll
+      for (int ch = 0; ch < CH; ++ch) {
+        if (ch < nch) {
+          f32x4_t acc = (f32x4_t){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+          for (int kk = 0; kk < 4; ++kk)
+            acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+                ri_as_bf16x8(*reinterpret_cast<const uint4*>(qrow + kk * 32)), ri_as_bf16x8(bk[ch][kk]), acc, 0, 0, 0);
+          const float s[4] = {acc[0] * P.scale, acc[1] * P.scale, acc[2] * P.scale, acc[3] * P.scale};
+          const bool valid = __shfl(desc[ch / 4], (ch % 4) * 16 + n) >= 0;
+          const float w = __shfl(wd[ch / 4], (ch % 4) * 16 + n);
+          chunk_update<GS_PAD>(st, s, valid, w, v[ch], p_sh, al_sh, lane);
+        }
+      }
     }
   } else {
     // ---------------- estimation rows ----------------
     const int es = P.es;
-    const int chunks = (es + 15) >> 4;
-    const int nwaves = P.S_es * 4;
-    const int cpw = (chunks + nwaves - 1) / nwaves;
-    const int wid = (split - P.S_kv) * 4 + wave;
-    const int cb = wid * cpw;
-    const int ce = min(chunks, cb + cpw);
+    int r0, r1;
+    wave_rows(es, P.S_es * 4, (split - P.S_kv) * 4 + wave, &r0, &r1);
     const int32_t* ids = P.est_ids + (size_t)g * es;
     const uint16_t* vs = P.value_sum + (size_t)g * P.nc * RI_DIM;
     const uint16_t* cs = P.csize + (size_t)g * P.nc;
+    const float* lg = P.logits + (size_t)g * gs * P.nc;
 
-    for (int c = cb; c < ce; ++c) {
-      const int row = c * 16 + n;
-      const bool valid = row < es;
-      float s[4] = {-INFINITY, -INFINITY, -INFINITY, -INFINITY};
-      float w = 0.f;
-      if (valid) {
-        const int cid = ids[row];
-        w = ri_bf16_to_f32(cs[cid]);
+    for (int b0 = r0; b0 < r1; b0 += 16 * CH) {
+      int cid[ND];
+      float wd[ND];
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          const int head = (4 * h + i) % GS_PAD;
-          if (head < gs) s[i] = P.logits[((size_t)g * gs + head) * P.nc + cid];
+      for (int k = 0; k < ND; ++k) {
+        cid[k] = -1;
+        wd[k] = 0.f;
+        const int row = b0 + 64 * k + lane;
+        if (row < r1 && 64 * k + lane < 16 * CH) {
+          cid[k] = ids[row];
+          wd[k] = ri_bf16_to_f32(cs[cid[k]]);
         }
       }
-      uint4 v[4];
+      const int nch = min(CH, (r1 - b0 + 15) >> 4);
+      float sc[CH][4];
+      uint4 v[CH][4];
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const int vr = c * 16 + h + 4 * i;
-        v[i] = (vr < es) ? ri_ld16(vs + (size_t)ids[vr] * RI_DIM + n * 8) : ri_zero16();
+      for (int ch = 0; ch < CH; ++ch) {
+        if (ch < nch) {
+          const int ck = __shfl(cid[ch / 4], (ch % 4) * 16 + n);
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            const int head = (4 * h + i) % GS_PAD;
+            sc[ch][i] = (ck >= 0 && head < gs) ? lg[(size_t)head * P.nc + ck] : -INFINITY;
+          }
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            const int cv = __shfl(cid[ch / 4], (ch % 4) * 16 + h + 4 * i);
+            v[ch][i] = (cv >= 0) ? ri_ld16(vs + (size_t)cv * RI_DIM + n * 8) : ri_zero16();
+          }
+        }
       }
-      chunk_update<GS_PAD>(st, s, valid, w, v, p_sh, al_sh, lane);
+#pragma unroll
+      for (int ch = 0; ch < CH; ++ch) {
+        if (ch < nch) {
+          const bool valid = __shfl(cid[ch / 4], (ch % 4) * 16 + n) >= 0;
+          const float w = __shfl(wd[ch / 4], (ch % 4) * 16 + n);
+          chunk_update<GS_PAD>(st, sc[ch], valid, w, v[ch], p_sh, al_sh, lane);
+        }
+      }
     }
   }
 
@@ -310,40 +395,62 @@ __global__ __launch_bounds__(256) void attend_kernel(AttendParams P) {
       P.part_ml[o * 2 + 1] = l;
     }
   }
+
+  // ---------------- last workgroup of the group merges all splits ----------------
+  if (!P.fuse) return;
+  __syncthreads();  // this workgroup's partial is complete
+  if (threadIdx.x == 0) {
+    __threadfence();  // publish it device-wide before announcing it
+    sh_last = (atomicAdd(&P.counters[g], 1) == S - 1);
+  }
+  __syncthreads();
+  if (!sh_last) return;
+  __threadfence();  // see the other workgroups' partials
+  combine_group<GS_PAD>(P, g, S, lenB);
+  if (threadIdx.x == 0) P.counters[g] = 0;  // ready for the next launch
 }
 
-// combine: grid (gs, BG), 128 threads (one per dim)
-__global__ __launch_bounds__(128) void combine_kernel(const float* __restrict__ part_ml,
-                                                      const float* __restrict__ part_acc, int S, int gs_pad,
-                                                      const uint16_t* __restrict__ prev_out,
-                                                      const float* __restrict__ prev_lse,
-                                                      uint16_t* __restrict__ out, float* __restrict__ lse_out,
-                                                      int gs, const int32_t* __restrict__ lenB_ptr,
-                                                      int lenB_ptr_stride, int lenA,
-                                                      int32_t* __restrict__ valid_lengths) {
-  const int j = blockIdx.x, g = blockIdx.y, d = threadIdx.x;
-  float M = -INFINITY;
-  if (prev_lse) M = prev_lse[(size_t)g * gs + j];
-  for (int s = 0; s < S; ++s) M = fmaxf(M, part_ml[(((size_t)g * S + s) * gs_pad + j) * 2]);
-  float L = 0.f, A = 0.f;
-  if (prev_lse) {
-    const float pl = prev_lse[(size_t)g * gs + j];
-    const float f = (pl == -INFINITY) ? 0.f : __expf(pl - M);
-    L = f;
-    A = f * ri_bf16_to_f32(prev_out[((size_t)g * gs + j) * RI_DIM + d]);
+// separate merge pass: grid (gs, BG), one wave per (group, head); lanes first cover the
+// splits (statistics), then the dims (two each)
+template <int GS_PAD>
+__global__ __launch_bounds__(64) void combine_kernel(AttendParams P) {
+  const int j = blockIdx.x, g = blockIdx.y, lane = threadIdx.x;
+  const int S = P.S_kv + P.S_es, gs = P.gs;
+  const float* ml = P.part_ml + ((size_t)g * S * GS_PAD + j) * 2;
+  const float* pa = P.part_acc + ((size_t)g * S * GS_PAD + j) * RI_DIM + 2 * lane;
+  float2 ms = make_float2(-INFINITY, 0.f);
+  if (lane < S) ms = *reinterpret_cast<const float2*>(ml + (size_t)lane * GS_PAD * 2);
+  const float pl = P.prev_lse ? P.prev_lse[(size_t)g * gs + j] : -INFINITY;
+  float M = fmaxf(ms.x, pl);
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) M = fmaxf(M, __shfl_xor(M, o));
+  const float f = (ms.x == -INFINITY) ? 0.f : __expf(ms.x - M);
+  float L = ms.y * f;
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) L += __shfl_xor(L, o);
+  float A0 = 0.f, A1 = 0.f;
+  if (P.prev_lse) {
+    const float fp = (pl == -INFINITY) ? 0.f : __expf(pl - M);
+    const uint32_t po = *reinterpret_cast<const uint32_t*>(P.prev_out + ((size_t)g * gs + j) * RI_DIM + 2 * lane);
+    L += fp;
+    A0 = fp * __uint_as_float(po << 16);
+    A1 = fp * __uint_as_float(po & 0xffff0000u);
   }
+#pragma unroll 8
   for (int s = 0; s < S; ++s) {
-    const size_t o = ((size_t)g * S + s) * gs_pad + j;
-    const float m = part_ml[o * 2];
-    const float f = (m == -INFINITY) ? 0.f : __expf(m - M);
-    L += part_ml[o * 2 + 1] * f;
-    A += part_acc[o * RI_DIM + d] * f;
+    const float fs = __shfl(f, s);
+    const float2 a2 = *reinterpret_cast<const float2*>(pa + (size_t)s * GS_PAD * RI_DIM);
+    A0 += a2.x * fs;
+    A1 += a2.y * fs;
   }
-  out[((size_t)g * gs + j) * RI_DIM + d] = ri_f32_to_bf16(A / L);
-  if (d == 0) {
-    if (lse_out) lse_out[(size_t)g * gs + j] = M + __logf(L);
-    if (valid_lengths && j == 0)
-      valid_lengths[g] = lenA + (lenB_ptr ? lenB_ptr[(size_t)g * lenB_ptr_stride] : 0);
+  const uint32_t o = (uint32_t)ri_f32_to_bf16(A0 / L) | ((uint32_t)ri_f32_to_bf16(A1 / L) << 16);
+  *reinterpret_cast<uint32_t*>(P.out + ((size_t)g * gs + j) * RI_DIM + 2 * lane) = o;
+  if (lane == 0) {
+    if (P.lse_out) P.lse_out[(size_t)g * gs + j] = M + __logf(L);
+    if (P.valid_lengths && j == 0) {
+      const int lenB = P.lenB_ptr ? P.lenB_ptr[(size_t)g * P.lenB_ptr_stride] : P.lenB_const;
+      P.valid_lengths[g] = P.lenA + lenB;
+    }
   }
 }
 
@@ -351,33 +458,60 @@ __global__ __launch_bounds__(128) void combine_kernel(const float* __restrict__ 
 // host side
 // ------------------------------------------------------------------------------------
 #define RI_MAX_SPLITS 64
+#define RI_MAX_GROUPS 4096  // size of the counter area at the head of the workspace
 
 static inline int gs_pad_of(int gs) { return gs <= 4 ? 4 : (gs <= 8 ? 8 : 16); }
 
 static size_t attn_workspace_bytes(int BG, int gs) {
-  if (BG <= 0 || gs <= 0 || gs > 16) return 0;
+  if (BG <= 0 || BG > RI_MAX_GROUPS || gs <= 0 || gs > 16) return 0;
   const size_t per = (size_t)BG * RI_MAX_SPLITS * gs_pad_of(gs);
-  return per * (2 + RI_DIM) * sizeof(float);
+  return RI_MAX_GROUPS * sizeof(int) + per * (2 + RI_DIM) * sizeof(float);
 }
 
 extern "C" size_t ri_flash_decoding_workspace_bytes(int BG, int gs) { return attn_workspace_bytes(BG, gs); }
 extern "C" size_t ri_wave_attention_workspace_bytes(int BG, int gs) { return attn_workspace_bytes(BG, gs); }
 
+static void carve_workspace(AttendParams& P, void* workspace, int BG, int gp) {
+  P.counters = (int*)workspace;
+  P.part_ml = (float*)((char*)workspace + RI_MAX_GROUPS * sizeof(int));
+  P.part_acc = P.part_ml + (size_t)BG * RI_MAX_SPLITS * gp * 2;
+}
+
+static int fuse_default() {
+  static int v = -1;
+  if (v < 0) {
+    const char* e = getenv("RI_ATTN_FUSE");
+    v = e ? atoi(e) : 0;
+  }
+  return v;
+}
+
 static int launch_attend(AttendParams& P, int BG, int gs, hipStream_t s) {
   const int S = P.S_kv + P.S_es;
   const dim3 grid(S, BG);
+  P.fuse = fuse_default();
   switch (gs_pad_of(gs)) {
-    case 4: attend_kernel<4><<<grid, 256, 0, s>>>(P); break;
-    case 8: attend_kernel<8><<<grid, 256, 0, s>>>(P); break;
-    default: attend_kernel<16><<<grid, 256, 0, s>>>(P); break;
+    case 4: attend_kernel<4, 5><<<grid, 256, 0, s>>>(P); break;
+    case 8: attend_kernel<8, 4><<<grid, 256, 0, s>>>(P); break;
+    default: attend_kernel<16, 2><<<grid, 256, 0, s>>>(P); break;
   }
   RI_HIP_CHECK_LAUNCH();
+  if (!P.fuse) {
+    switch (gs_pad_of(gs)) {
+      case 4: combine_kernel<4><<<dim3(gs, BG), 64, 0, s>>>(P); break;
+      case 8: combine_kernel<8><<<dim3(gs, BG), 64, 0, s>>>(P); break;
+      default: combine_kernel<16><<<dim3(gs, BG), 64, 0, s>>>(P); break;
+    }
+    RI_HIP_CHECK_LAUNCH();
+  }
   return RI_OK;
 }
 
-// splits so that a wave sees about `rows_per_wave` rows, within [1, cap]
-static int pick_splits(int64_t rows, int BG, int cap) {
-  const int rows_per_wave = 64;
+static inline int chunks_ahead(int gs) { return gs <= 4 ? 5 : (gs <= 8 ? 4 : 2); }
+
+// splits so that a wave sees about one batch of rows, within [1, cap]
+static int pick_splits(int64_t rows, int BG, int cap, int gs) {
+  const int rows_per_wave = 16 * chunks_ahead(gs);
   int64_t s = (rows + 4 * rows_per_wave - 1) / (4 * rows_per_wave);
   // do not launch far more workgroups than the chip can hold at once
   const int64_t max_by_chip = (4096 + BG - 1) / BG;
@@ -393,7 +527,7 @@ extern "C" int ri_weighted_flash_decoding(const void* q, const void* k, const vo
                                           int S, int64_t kv_stride, float scale, void* workspace,
                                           size_t workspace_bytes, ri_stream_t stream) {
   if (!q || !k || !v || !out || !workspace) return RI_ERR_ARG;
-  if (BG <= 0 || gs <= 0 || gs > 16 || S < 0 || kv_stride < S) return RI_ERR_ARG;
+  if (BG <= 0 || BG > RI_MAX_GROUPS || gs <= 0 || gs > 16 || S < 0 || kv_stride < S) return RI_ERR_ARG;
   if ((prev_out == nullptr) != (prev_lse == nullptr)) return RI_ERR_ARG;
   if (workspace_bytes < attn_workspace_bytes(BG, gs)) return RI_ERR_WORKSPACE;
   const int gp = gs_pad_of(gs);
@@ -408,19 +542,16 @@ extern "C" int ri_weighted_flash_decoding(const void* q, const void* k, const vo
   P.lenB_const = S;
   P.weightB = (const uint16_t*)weight;
   P.weight_stride = S;
-  P.S_kv = pick_splits(S, BG, RI_MAX_SPLITS);
+  P.S_kv = pick_splits(S, BG, RI_MAX_SPLITS, gs);
   P.S_es = 0;
   P.gs = gs;
   P.scale = scale;
-  P.part_ml = (float*)workspace;
-  P.part_acc = P.part_ml + (size_t)BG * RI_MAX_SPLITS * gp * 2;
-  hipStream_t s = (hipStream_t)stream;
-  int rc = launch_attend(P, BG, gs, s);
-  if (rc) return rc;
-  combine_kernel<<<dim3(gs, BG), 128, 0, s>>>(P.part_ml, P.part_acc, P.S_kv, gp, (const uint16_t*)prev_out,
-                                              prev_lse, (uint16_t*)out, lse_out, gs, nullptr, 0, 0, nullptr);
-  RI_HIP_CHECK_LAUNCH();
-  return RI_OK;
+  P.prev_out = (const uint16_t*)prev_out;
+  P.prev_lse = prev_lse;
+  P.out = (uint16_t*)out;
+  P.lse_out = lse_out;
+  carve_workspace(P, workspace, BG, gp);
+  return launch_attend(P, BG, gs, (hipStream_t)stream);
 }
 
 extern "C" int ri_wave_attention(const void* q, const void* steady_k, const void* steady_v,
@@ -432,7 +563,8 @@ extern "C" int ri_wave_attention(const void* q, const void* steady_k, const void
                                  float scale, void* workspace, size_t workspace_bytes, ri_stream_t stream) {
   if (!q || !steady_k || !steady_v || !store_k || !store_v || !row_src || !meta || !out || !workspace)
     return RI_ERR_ARG;
-  if (BG <= 0 || gs <= 0 || gs > 16 || static_len < 0 || static_len > steady_stride || es < 0 || nc <= 0)
+  if (BG <= 0 || BG > RI_MAX_GROUPS || gs <= 0 || gs > 16 || static_len < 0 || static_len > steady_stride ||
+      es < 0 || nc <= 0)
     return RI_ERR_ARG;
   if (es > 0 && (!est_ids || !logits || !value_sum || !cluster_size_bf16)) return RI_ERR_ARG;
   if (workspace_bytes < attn_workspace_bytes(BG, gs)) return RI_ERR_WORKSPACE;
@@ -458,19 +590,13 @@ extern "C" int ri_wave_attention(const void* q, const void* steady_k, const void
   P.es = es;
   P.gs = gs;
   P.scale = scale;
+  P.out = (uint16_t*)out;
+  P.valid_lengths = valid_lengths;
   // the retrieved-token count is only known on the device: size the split for the row table
   // capacity scaled by the usual fill (a quarter), the estimation zone by its exact size
   const int cap_es = es > 0 ? RI_MAX_SPLITS / 2 : 0;
-  P.S_es = es > 0 ? pick_splits(es, BG, cap_es) : 0;
-  P.S_kv = pick_splits(static_len + row_src_stride / 4, BG, RI_MAX_SPLITS - P.S_es);
-  P.part_ml = (float*)workspace;
-  P.part_acc = P.part_ml + (size_t)BG * RI_MAX_SPLITS * gp * 2;
-  hipStream_t s = (hipStream_t)stream;
-  int rc = launch_attend(P, BG, gs, s);
-  if (rc) return rc;
-  combine_kernel<<<dim3(gs, BG), 128, 0, s>>>(P.part_ml, P.part_acc, P.S_kv + P.S_es, gp, nullptr, nullptr,
-                                              (uint16_t*)out, nullptr, gs, meta + 1, 4, static_len,
-                                              valid_lengths);
-  RI_HIP_CHECK_LAUNCH();
-  return RI_OK;
+  P.S_es = es > 0 ? pick_splits(es, BG, cap_es, gs) : 0;
+  P.S_kv = pick_splits(static_len + row_src_stride / 4, BG, RI_MAX_SPLITS - P.S_es, gs);
+  carve_workspace(P, workspace, BG, gp);
+  return launch_attend(P, BG, gs, (hipStream_t)stream);
 }

@@ -35,11 +35,12 @@ _workspaces = {}
 
 
 def _workspace(nbytes, device, tag):
-    """Per-(device, tag) scratch tensor, grown on demand and reused across calls."""
+    """Per-(device, tag) scratch tensor, grown on demand and reused across calls.  It starts
+    zeroed: the attention kernels keep arrival counters in it that they leave at zero."""
     key = (str(device), tag)
     w = _workspaces.get(key)
     if w is None or w.numel() < nbytes:
-        w = torch.empty(max(nbytes, 256), dtype=torch.uint8, device=device)
+        w = torch.zeros(max(nbytes, 256), dtype=torch.uint8, device=device)
         _workspaces[key] = w
     return w
 

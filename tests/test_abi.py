@@ -1,0 +1,47 @@
+"""The shared library loads without a GPU and exports every symbol the header declares."""
+import ctypes
+import os
+import re
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "retro_mi355.h")
+
+
+def _declared():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(ri_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    from retrievalattention_amd import _lib
+    assert os.path.exists(_lib.LIB_PATH), "build the library first: python -m retrievalattention_amd.build"
+    handle = ctypes.CDLL(_lib.LIB_PATH)
+    names = _declared()
+    assert len(names) >= 30
+    missing = [n for n in names if not hasattr(handle, n)]
+    assert not missing, f"declared in the header but not exported: {missing}"
+
+
+def test_python_binding_covers_the_header():
+    from retrievalattention_amd import _lib
+    assert sorted(_lib.SIGNATURES) == _declared()
+
+
+def test_status_strings_and_version():
+    from retrievalattention_amd import _lib
+    l = _lib.lib()
+    assert l.ri_abi_version() >= 1
+    assert l.ri_status_string(0) == b"ok"
+    assert b"workspace" in l.ri_status_string(-3)
+    assert l.ri_score_select_workspace_bytes(32, 4, 8192) == 2 * 32 * 32 * 4 * 4
+    assert l.ri_flash_decoding_workspace_bytes(0, 4) == 0
+
+
+def test_missing_library_is_a_loud_error(monkeypatch, tmp_path):
+    from retrievalattention_amd import _lib
+    monkeypatch.setattr(_lib, "_lib", None)
+    monkeypatch.setattr(_lib, "LIB_PATH", str(tmp_path / "nope.so"))
+    import pytest
+    with pytest.raises(RuntimeError, match="no CPU or PyTorch fallback"):
+        _lib.lib()
