@@ -68,57 +68,86 @@ struct AttendParams {
   int32_t* valid_lengths;    // [BG] or null: lenA + lenB(g)
 };
 
+// Softmax bookkeeping is spread over the four 16-lane groups of a wave: group h keeps
+// NH = GS_PAD/4 heads (the MFMA hands every group four heads; with GS_PAD = 4 all groups see the
+// same four, so each keeps one).  ri_head_reg(h) is the first accumulator register group h keeps,
+// ri_head_of(h, i) the head held in kept slot i.
+template <int GS_PAD>
+__device__ __forceinline__ int ri_head_reg(int h) {
+  return GS_PAD == 4 ? h : (GS_PAD == 8 ? (h >> 1) * 2 : 0);
+}
+template <int GS_PAD>
+__device__ __forceinline__ int ri_head_of(int h, int i) {
+  return (4 * h + ri_head_reg<GS_PAD>(h) + i) % GS_PAD;
+}
+
 template <int GS_PAD>
 struct WaveState {
-  float m[4];
-  float l[4];
+  float m[GS_PAD / 4];
+  float l[GS_PAD / 4];
   float acc[GS_PAD][8];
 };
 
-// softmax update for one chunk: scores s[4] (this lane: row n = lane%16, heads 4*(lane/16)+i mod
-// GS_PAD), validity and denominator weight; then the P·V accumulation of the four value rows
-// v[4] this lane owns.  p_sh: [16][GS_PAD] floats, al_sh: [GS_PAD] floats of this wave.
+// softmax update for one chunk: scores s_in[4] (this lane: row n = lane%16, MFMA registers of
+// lane group h = lane/16), validity and denominator weight; then the P·V accumulation of the
+// four value rows v[4] this lane owns.  p_sh: [16][GS_PAD] floats, al_sh: [GS_PAD] floats of this wave.
 template <int GS_PAD>
 __device__ __forceinline__ void chunk_update(WaveState<GS_PAD>& st, const float s_in[4], bool valid, float w,
                                              const uint4 v[4], float* p_sh, float* al_sh, int lane) {
+  constexpr int NH = GS_PAD / 4;
   const int n = lane & 15, h = lane >> 4;
-  float p[4], al[4];
+  const int r0 = ri_head_reg<GS_PAD>(h);
+  float al[NH];
+  bool rescale = false;
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    const float s = valid ? s_in[i] : -INFINITY;
+  for (int i = 0; i < NH; ++i) {
+    float sv;
+    if (GS_PAD == 16) {
+      sv = s_in[i];
+    } else {  // pick register r0 + i without dynamic indexing
+      const int r = r0 + i;
+      sv = r == 0 ? s_in[0] : (r == 1 ? s_in[1] : (r == 2 ? s_in[2] : s_in[3]));
+    }
+    const float s = valid ? sv : -INFINITY;
     float cm = s;
     cm = fmaxf(cm, __shfl_xor(cm, 1));
     cm = fmaxf(cm, __shfl_xor(cm, 2));
     cm = fmaxf(cm, __shfl_xor(cm, 4));
     cm = fmaxf(cm, __shfl_xor(cm, 8));
     const float mn = fmaxf(st.m[i], cm);
+    float p;
     if (mn == -INFINITY) {
       al[i] = 1.f;
-      p[i] = 0.f;
+      p = 0.f;
     } else {
       al[i] = __expf(st.m[i] - mn);  // exp(-inf) = 0 for the first chunk
-      p[i] = valid ? __expf(s - mn) : 0.f;
+      p = valid ? __expf(s - mn) : 0.f;
     }
-    st.l[i] = st.l[i] * al[i] + w * p[i];
+    rescale |= (al[i] != 1.f);
+    st.l[i] = st.l[i] * al[i] + w * p;
     st.m[i] = mn;
+    p_sh[n * GS_PAD + ri_head_of<GS_PAD>(h, i)] = p;
   }
-  if (h < GS_PAD / 4) {
-    *reinterpret_cast<float4*>(p_sh + n * GS_PAD + 4 * h) = make_float4(p[0], p[1], p[2], p[3]);
-    if (n == 0) *reinterpret_cast<float4*>(al_sh + 4 * h) = make_float4(al[0], al[1], al[2], al[3]);
+  // the running maximum rarely moves after the first chunks: rescale only when some head's did
+  const bool any_rescale = __any(rescale);
+  if (any_rescale && n == 0) {
+#pragma unroll
+    for (int i = 0; i < NH; ++i) al_sh[ri_head_of<GS_PAD>(h, i)] = al[i];
   }
   __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
   __builtin_amdgcn_wave_barrier();
   __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-  float alpha[GS_PAD];
+  if (any_rescale) {
 #pragma unroll
-  for (int j = 0; j < GS_PAD; j += 4) {
-    const float4 a4 = *reinterpret_cast<const float4*>(al_sh + j);
-    alpha[j] = a4.x; alpha[j + 1] = a4.y; alpha[j + 2] = a4.z; alpha[j + 3] = a4.w;
+    for (int j = 0; j < GS_PAD; j += 4) {
+      const float4 a4 = *reinterpret_cast<const float4*>(al_sh + j);
+      const float alpha[4] = {a4.x, a4.y, a4.z, a4.w};
+#pragma unroll
+      for (int jj = 0; jj < 4; ++jj)
+#pragma unroll
+        for (int e = 0; e < 8; ++e) st.acc[j + jj][e] *= alpha[jj];
+    }
   }
-#pragma unroll
-  for (int j = 0; j < GS_PAD; ++j)
-#pragma unroll
-    for (int e = 0; e < 8; ++e) st.acc[j][e] *= alpha[j];
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
     float vf[8];
@@ -204,7 +233,7 @@ __global__ __launch_bounds__(256, 2) void attend_kernel(AttendParams P) {
 
   WaveState<GS_PAD> st;
 #pragma unroll
-  for (int i = 0; i < 4; ++i) { st.m[i] = -INFINITY; st.l[i] = 0.f; }
+  for (int i = 0; i < GS_PAD / 4; ++i) { st.m[i] = -INFINITY; st.l[i] = 0.f; }
 #pragma unroll
   for (int j = 0; j < GS_PAD; ++j)
 #pragma unroll
@@ -342,19 +371,15 @@ __global__ __launch_bounds__(256, 2) void attend_kernel(AttendParams P) {
 
   // ---------------- wave partial -> LDS ----------------
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
+  for (int i = 0; i < GS_PAD / 4; ++i) {
     float l = st.l[i];
     l += __shfl_xor(l, 1);
     l += __shfl_xor(l, 2);
     l += __shfl_xor(l, 4);
     l += __shfl_xor(l, 8);
-    st.l[i] = l;
-  }
-  if (n == 0 && h < GS_PAD / 4) {
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      sh_m[wave][4 * h + i] = st.m[i];
-      sh_l[wave][4 * h + i] = st.l[i];
+    if (n == 0) {
+      sh_m[wave][ri_head_of<GS_PAD>(h, i)] = st.m[i];
+      sh_l[wave][ri_head_of<GS_PAD>(h, i)] = l;
     }
   }
 #pragma unroll

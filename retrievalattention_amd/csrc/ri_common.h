@@ -59,3 +59,26 @@ __host__ __device__ __forceinline__ uint32_t ri_bf16_sort_key(uint16_t b) {
   } while (0)
 
 void ri_set_last_hip_error(int e);
+
+// ---- shared between score.hip and select.hip ----
+#define RI_SCORE_TILE 256          // centroids per softmax partial
+#define RI_SEL_HI_BITS 11          // first radix pass of the selection: top 11 bits of the 16-bit key
+#define RI_SEL_HI_BINS (1 << RI_SEL_HI_BITS)
+int ri_launch_score(const void* q, const void* centroids, float* logits, float* tile_max, float* tile_sum,
+                    uint32_t* ghist, int BG, int gs, int nc, float scale, hipStream_t s);
+
+// Row statistics from the per-256-column partials [ntiles, gs]: one wave per row, lanes over
+// tiles, xor-butterfly reductions (fixed order, so the result is reproducible).
+__device__ __forceinline__ void ri_wave_reduce_partials(const float* pm, const float* ps, int ntiles, int gs,
+                                                        int j, int lane, float* m_out, float* invz_out) {
+  float m = -INFINITY;
+  for (int t = lane; t < ntiles; t += 64) m = fmaxf(m, pm[(size_t)t * gs + j]);
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) m = fmaxf(m, __shfl_xor(m, o));
+  float z = 0.f;
+  for (int t = lane; t < ntiles; t += 64) z += ps[(size_t)t * gs + j] * __expf(pm[(size_t)t * gs + j] - m);
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) z += __shfl_xor(z, o);
+  *m_out = m;
+  *invz_out = 1.0f / z;
+}
