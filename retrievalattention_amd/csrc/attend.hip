@@ -177,7 +177,12 @@ __device__ __forceinline__ void wave_rows(int total, int nwaves, int wid, int* r
 
 // Merges the S split partials of group g (and the optional previous result) and writes the
 // output; called by all 256 threads of one workgroup.
-template <int GS_PAD>
+template <bool COHERENT>
+__device__ __forceinline__ float ld_part(const float* p) {
+  return COHERENT ? __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : *p;
+}
+
+template <int GS_PAD, bool COHERENT>
 __device__ __forceinline__ void combine_group(const AttendParams& P, int g, int S, int lenB) {
   const int gs = P.gs;
   for (int idx = threadIdx.x; idx < gs * (RI_DIM / 2); idx += 256) {
@@ -186,7 +191,7 @@ __device__ __forceinline__ void combine_group(const AttendParams& P, int g, int 
     const float* pa = P.part_acc + ((size_t)g * S * GS_PAD + j) * RI_DIM + d2;
     float M = P.prev_lse ? P.prev_lse[(size_t)g * gs + j] : -INFINITY;
 #pragma unroll 8
-    for (int s = 0; s < S; ++s) M = fmaxf(M, ml[(size_t)s * GS_PAD * 2]);
+    for (int s = 0; s < S; ++s) M = fmaxf(M, ld_part<COHERENT>(ml + (size_t)s * GS_PAD * 2));
     float L = 0.f, A0 = 0.f, A1 = 0.f;
     if (P.prev_lse) {
       const float pl = P.prev_lse[(size_t)g * gs + j];
@@ -198,12 +203,13 @@ __device__ __forceinline__ void combine_group(const AttendParams& P, int g, int 
     }
 #pragma unroll 8
     for (int s = 0; s < S; ++s) {
-      const float m = ml[(size_t)s * GS_PAD * 2];
+      const float m = ld_part<COHERENT>(ml + (size_t)s * GS_PAD * 2);
       const float f = (m == -INFINITY) ? 0.f : __expf(m - M);
-      const float2 a2 = *reinterpret_cast<const float2*>(pa + (size_t)s * GS_PAD * RI_DIM);
-      L += ml[(size_t)s * GS_PAD * 2 + 1] * f;
-      A0 += a2.x * f;
-      A1 += a2.y * f;
+      const float a0 = ld_part<COHERENT>(pa + (size_t)s * GS_PAD * RI_DIM);
+      const float a1 = ld_part<COHERENT>(pa + (size_t)s * GS_PAD * RI_DIM + 1);
+      L += ld_part<COHERENT>(ml + (size_t)s * GS_PAD * 2 + 1) * f;
+      A0 += a0 * f;
+      A1 += a1 * f;
     }
     const uint32_t o = (uint32_t)ri_f32_to_bf16(A0 / L) | ((uint32_t)ri_f32_to_bf16(A1 / L) << 16);
     *reinterpret_cast<uint32_t*>(P.out + ((size_t)g * gs + j) * RI_DIM + d2) = o;
@@ -414,24 +420,33 @@ __global__ __launch_bounds__(256, 2) void attend_kernel(AttendParams P) {
       l += sh_l[w][j] * f;
     }
     const size_t o = ((size_t)g * S + split) * GS_PAD + j;
-    P.part_acc[o * RI_DIM + d] = a;
-    if (d == 0) {
-      P.part_ml[o * 2] = M;
-      P.part_ml[o * 2 + 1] = l;
+    if (P.fuse) {  // device-coherent stores: another workgroup of this launch reads them
+      __hip_atomic_store(&P.part_acc[o * RI_DIM + d], a, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      if (d == 0) {
+        __hip_atomic_store(&P.part_ml[o * 2], M, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __hip_atomic_store(&P.part_ml[o * 2 + 1], l, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      }
+    } else {
+      P.part_acc[o * RI_DIM + d] = a;
+      if (d == 0) {
+        P.part_ml[o * 2] = M;
+        P.part_ml[o * 2 + 1] = l;
+      }
     }
   }
 
   // ---------------- last workgroup of the group merges all splits ----------------
   if (!P.fuse) return;
-  __syncthreads();  // this workgroup's partial is complete
-  if (threadIdx.x == 0) {
-    __threadfence();  // publish it device-wide before announcing it
-    sh_last = (atomicAdd(&P.counters[g], 1) == S - 1);
-  }
+  // The partial went out with device-coherent stores; once they have completed (the barrier
+  // waits for this workgroup's outstanding stores) the arrival is announced.  The last
+  // workgroup to arrive reads every partial with device-coherent loads.
+  __builtin_amdgcn_s_waitcnt(0);
+  __syncthreads();
+  if (threadIdx.x == 0)
+    sh_last = (__hip_atomic_fetch_add(&P.counters[g], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == S - 1);
   __syncthreads();
   if (!sh_last) return;
-  __threadfence();  // see the other workgroups' partials
-  combine_group<GS_PAD>(P, g, S, lenB);
+  combine_group<GS_PAD, true>(P, g, S, lenB);
   if (threadIdx.x == 0) P.counters[g] = 0;  // ready for the next launch
 }
 
@@ -506,7 +521,7 @@ static int fuse_default() {
   static int v = -1;
   if (v < 0) {
     const char* e = getenv("RI_ATTN_FUSE");
-    v = e ? atoi(e) : 0;
+    v = e ? atoi(e) : 1;
   }
   return v;
 }

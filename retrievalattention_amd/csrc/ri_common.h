@@ -62,10 +62,8 @@ void ri_set_last_hip_error(int e);
 
 // ---- shared between score.hip and select.hip ----
 #define RI_SCORE_TILE 256          // centroids per softmax partial
-#define RI_SEL_HI_BITS 11          // first radix pass of the selection: top 11 bits of the 16-bit key
-#define RI_SEL_HI_BINS (1 << RI_SEL_HI_BITS)
 int ri_launch_score(const void* q, const void* centroids, float* logits, float* tile_max, float* tile_sum,
-                    uint32_t* ghist, int BG, int gs, int nc, float scale, hipStream_t s);
+                    int BG, int gs, int nc, float scale, hipStream_t s);
 
 // Row statistics from the per-256-column partials [ntiles, gs]: one wave per row, lanes over
 // tiles, xor-butterfly reductions (fixed order, so the result is reproducible).

@@ -18,7 +18,7 @@
 __global__ __launch_bounds__(256) void score_kernel(
     const uint16_t* __restrict__ q, const uint16_t* __restrict__ cent, float* __restrict__ logits,
     uint16_t* __restrict__ logits_bf16, float* __restrict__ tile_max, float* __restrict__ tile_sum,
-    uint32_t* __restrict__ ghist, int gs, int nc, int ntiles, float scale) {
+    int gs, int nc, int ntiles, float scale) {
   const int tile = blockIdx.x;
   const int g = blockIdx.y;
   const int lane = threadIdx.x & 63;
@@ -26,9 +26,6 @@ __global__ __launch_bounds__(256) void score_kernel(
   const int r = lane & 15;
   const int h = lane >> 4;
   const int c0 = tile * SCORE_TILE + wave * 64;
-  // the selection pass accumulates a per-group score histogram: start it from zero
-  if (ghist && tile == 0)
-    for (int i = threadIdx.x; i < RI_SEL_HI_BINS; i += 256) ghist[(size_t)blockIdx.y * RI_SEL_HI_BINS + i] = 0u;
 
   const uint16_t* cg = cent + (size_t)g * nc * RI_DIM;
   uint4 a[4][4];
@@ -166,7 +163,7 @@ extern "C" int ri_batch_gemm_softmax(const void* A, const void* B, void* D, floa
   // fp32 logits are not part of this interface: the partial statistics come from the fp32
   // accumulators inside the kernel, the softmax from the bf16 D, as in the reference.
   score_kernel<<<dim3(ntiles, batch_count), 256, 0, s>>>((const uint16_t*)A, (const uint16_t*)B, nullptr,
-                                                         (uint16_t*)D, Norm, Sum, nullptr, m, n, ntiles, alpha);
+                                                         (uint16_t*)D, Norm, Sum, m, n, ntiles, alpha);
   RI_HIP_CHECK_LAUNCH();
   softmax_reduce_kernel<<<batch_count, 64 * m, 0, s>>>(Norm, Sum, ntiles, m);
   RI_HIP_CHECK_LAUNCH();
@@ -181,10 +178,10 @@ extern "C" int ri_batch_gemm_softmax(const void* A, const void* B, void* D, floa
 
 // scoring pass used by the fused selection (select.hip)
 int ri_launch_score(const void* q, const void* centroids, float* logits, float* tile_max, float* tile_sum,
-                    uint32_t* ghist, int BG, int gs, int nc, float scale, hipStream_t s) {
+                    int BG, int gs, int nc, float scale, hipStream_t s) {
   const int ntiles = (nc + SCORE_TILE - 1) / SCORE_TILE;
   score_kernel<<<dim3(ntiles, BG), 256, 0, s>>>((const uint16_t*)q, (const uint16_t*)centroids, logits, nullptr,
-                                                tile_max, tile_sum, ghist, gs, nc, ntiles, scale);
+                                                tile_max, tile_sum, gs, nc, ntiles, scale);
   RI_HIP_CHECK_LAUNCH();
   return RI_OK;
 }

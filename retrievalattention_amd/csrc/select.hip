@@ -6,18 +6,16 @@
 //
 // Two launches:
 //   dist_kernel    many workgroups per group: score = bf16(sum_j bf16(exp(bf16(x_j)-m_j)/Z_j)),
-//                  mapped to a 16-bit key whose unsigned order is the score order; keys go to
-//                  global memory and into a per-group histogram of their top 11 bits.
-//   select_kernel  one workgroup per group: exact rank thresholds by radix select on the key
-//                  (11-bit histogram, then the low 5 bits inside the two boundary bins), zone
+//                  mapped to a 16-bit key whose unsigned order is the score order.
+//   select_kernel  one workgroup per group: exact rank thresholds from a histogram with one bin
+//                  per distinct key (scores lie in [0, 16], so ~16.8k bins cover every key), zone
 //                  membership with ties resolved by ascending id, rank order of the retrieval
-//                  zone, and the token layout (page cut-off, row table).
+//                  zone straight from the histogram prefix, and the token layout (page
+//                  cut-off, row table).
 #include "ri_common.h"
 
 #define SEL_THREADS 1024
 #define SEL_WAVES (SEL_THREADS / 64)
-#define SEL_LO_BITS (16 - RI_SEL_HI_BITS)
-#define SEL_LO_BINS (1 << SEL_LO_BITS)
 #define DIST_IDS 1024  // ids per dist workgroup (4 per thread)
 
 // Histogram add that survives a degenerate distribution: when the whole wave hits one bin
@@ -43,10 +41,8 @@ __global__ __launch_bounds__(256) void dist_kernel(const float* __restrict__ log
                                                    const float* __restrict__ tile_max,
                                                    const float* __restrict__ tile_sum,
                                                    const uint8_t* __restrict__ mask, uint16_t* __restrict__ keys,
-                                                   uint16_t* __restrict__ dist_out, uint32_t* __restrict__ ghist,
-                                                   int gs, int nc, int ntiles) {
+                                                   uint16_t* __restrict__ dist_out, int gs, int nc, int ntiles) {
   __shared__ float sh_m[16], sh_iz[16];
-  __shared__ uint32_t hist[RI_SEL_HI_BINS];
   const int g = blockIdx.y;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int c = blockIdx.x * DIST_IDS + tid * 4;
@@ -65,7 +61,6 @@ __global__ __launch_bounds__(256) void dist_kernel(const float* __restrict__ log
                             lane, &m, &iz);
     if (lane == 0) { sh_m[j] = m; sh_iz[j] = iz; }
   }
-  for (int i = tid; i < RI_SEL_HI_BINS; i += 256) hist[i] = 0u;
   __syncthreads();
 
   float d[4] = {0.f, 0.f, 0.f, 0.f};
@@ -84,7 +79,6 @@ __global__ __launch_bounds__(256) void dist_kernel(const float* __restrict__ log
     bits[i] = ri_f32_to_bf16(d[i]);
     if ((mk >> (8 * i)) & 0xffu) bits[i] = 0xff7f;  // finfo(bfloat16).min
     key[i] = (uint16_t)ri_bf16_sort_key(bits[i]);
-    hist_add(hist, (uint32_t)key[i] >> SEL_LO_BITS, in);
   }
   if (in) {
     uint2 w;
@@ -97,162 +91,175 @@ __global__ __launch_bounds__(256) void dist_kernel(const float* __restrict__ log
       *reinterpret_cast<uint2*>(dist_out + (size_t)g * nc + c) = w;
     }
   }
-  __syncthreads();
-  for (int i = tid; i < RI_SEL_HI_BINS; i += 256) {
-    const uint32_t v = hist[i];
-    if (v) atomicAdd(&ghist[(size_t)g * RI_SEL_HI_BINS + i], v);
-  }
 }
 
 // ------------------------------------------------------------------------------------
 // select_kernel helpers
 // ------------------------------------------------------------------------------------
-// exclusive prefix sum over the threads of the block; *total receives the sum
-template <typename T>
-__device__ __forceinline__ T block_excl_scan(T v, T* sh, T* total) {
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  T inc = v;
-#pragma unroll
-  for (int d = 1; d < 64; d <<= 1) {
-    const T n = __shfl_up(inc, d);
-    if (lane >= d) inc += n;
-  }
-  __syncthreads();  // sh may still be read from a previous scan
-  if (lane == 63) sh[wave] = inc;
-  __syncthreads();
-  T woff = 0, tot = 0;
-#pragma unroll
-  for (int w = 0; w < SEL_WAVES; ++w) {
-    const T s = sh[w];
-    if (w < wave) woff += s;
-    tot += s;
-  }
-  *total = tot;
-  return woff + inc - v;
+// Inclusive prefix sum over the 64 lanes of a wave with DPP row shifts and row broadcasts
+// (no LDS traffic): shifts by 1, 2, 3 build sums of four neighbours, shifts by 4 and 8 finish the
+// 16-lane rows, the two broadcasts carry row totals into the rows behind.
+__device__ __forceinline__ uint32_t wave_incl_scan(uint32_t v) {
+  uint32_t r = v;
+  r += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x111, 0xf, 0xf, true);   // row_shr:1
+  r += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x112, 0xf, 0xf, true);   // row_shr:2
+  r += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x113, 0xf, 0xf, true);   // row_shr:3
+  r += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)r, 0x114, 0xf, 0xe, false);  // row_shr:4, banks 1-3
+  r += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)r, 0x118, 0xf, 0xc, false);  // row_shr:8, banks 2-3
+  r += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)r, 0x142, 0xa, 0xf, false);  // row_bcast:15 -> rows 1, 3
+  r += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)r, 0x143, 0xc, 0xf, false);  // row_bcast:31 -> rows 2, 3
+  return r;
 }
 
-// Over a 32-bin histogram: bin holding descending rank `rank` and the count above it (one thread).
-__device__ __forceinline__ void find_lo_bin(const uint32_t* hist, uint32_t rank, uint32_t* out) {
-  uint32_t above = 0;
-  for (int b = SEL_LO_BINS - 1; b >= 0; --b) {
-    const uint32_t v = hist[b];
-    if (rank < above + v) { out[0] = (uint32_t)b; out[1] = above; return; }
-    above += v;
+// Exclusive prefix sums of N values over the threads of the block with one barrier.
+// sh: N * SEL_WAVES words that no other scan of the same parity is still reading: callers
+// alternate between two buffers.  tot[] receives the block totals.
+template <int N>
+__device__ __forceinline__ void block_excl_scan(const uint32_t (&v)[N], uint32_t (&pre)[N], uint32_t (&tot)[N],
+                                                uint32_t* sh) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  uint32_t inc[N];
+#pragma unroll
+  for (int k = 0; k < N; ++k) {
+    inc[k] = wave_incl_scan(v[k]);
+    if (lane == 63) sh[k * SEL_WAVES + wave] = inc[k];
   }
+  __syncthreads();
+#pragma unroll
+  for (int k = 0; k < N; ++k) {
+    uint32_t woff = 0, t = 0;
+#pragma unroll
+    for (int w = 0; w < SEL_WAVES; ++w) {
+      const uint32_t x = sh[k * SEL_WAVES + w];
+      if (w < wave) woff += x;
+      t += x;
+    }
+    tot[k] = t;
+    pre[k] = woff + inc[k] - v[k];
+  }
+}
+
+// Scores are sums of at most 16 probabilities, so their keys span a small range: key 0x8000
+// (score +0) .. 0xC180 (score 16), plus the masked value far below.  One histogram bin per
+// distinct key makes the rank search exact in a single pass.
+#define SEL_KEY_LO 0x8000u
+#define SEL_BPT 17                          // bins per thread
+#define SEL_BINS (SEL_THREADS * SEL_BPT)    // 17408 >= 0x4181 + 1
+__device__ __forceinline__ uint32_t sel_bin(uint32_t key) {
+  const uint32_t b = key >= SEL_KEY_LO ? key - SEL_KEY_LO + 1u : 0u;
+  return b < SEL_BINS ? b : SEL_BINS - 1;
 }
 
 // ------------------------------------------------------------------------------------
-// select_kernel: one workgroup per group.  dynamic LDS: nc * 2 bytes of keys.
+// select_kernel: one 1024-thread workgroup per group.
+// dynamic LDS: keys (2 B) + cluster sizes (2 B, clamped) per cluster.
 // Thread t owns the contiguous id range [t*E, t*E+E): ties are ranked by ascending id with
 // plain prefix sums.
 // ------------------------------------------------------------------------------------
 __global__ __launch_bounds__(SEL_THREADS) void select_kernel(
-    const uint16_t* __restrict__ keys, const uint32_t* __restrict__ ghist,
-    const int32_t* __restrict__ cluster_size, const int32_t* __restrict__ cluster_start,
-    int64_t* __restrict__ cI, int32_t* __restrict__ ret_ids, int32_t* __restrict__ est_ids,
-    int32_t* __restrict__ ret_tok_off, int32_t* __restrict__ row_src, int row_src_stride,
-    int32_t* __restrict__ meta, int nc, int np, int es, int page, int max_pages) {
+    const uint16_t* __restrict__ keys, const int32_t* __restrict__ cluster_size,
+    const int32_t* __restrict__ cluster_start, int64_t* __restrict__ cI, int32_t* __restrict__ ret_ids,
+    int32_t* __restrict__ est_ids, int32_t* __restrict__ ret_tok_off, int32_t* __restrict__ row_src,
+    int row_src_stride, int32_t* __restrict__ meta, int nc, int np, int es, int page, int max_pages) {
   extern __shared__ uint16_t sh_key[];
-  __shared__ uint32_t hist_b[SEL_LO_BINS], hist_c[SEL_LO_BINS];
-  __shared__ uint64_t sh_scan[SEL_WAVES];
-  __shared__ uint32_t sh_sel[8];  // hi1, above, hi2, above, lo1, above, lo2, above
+  __shared__ uint32_t hist[SEL_BINS];
+  __shared__ uint32_t sh_scan[2][3 * SEL_WAVES];  // two buffers, used alternately
+  __shared__ uint32_t sh_sel[4];  // bin of T1, entries above it, bin of T2, entries above it
   __shared__ uint32_t sh_ret[1024];
   __shared__ uint32_t sh_sorted[1024];
-  __shared__ int32_t sh_off[1025];
-  __shared__ uint32_t sh_cnt, sh_pages, sh_tret;
-  __shared__ int sh_nk;
+  __shared__ uint32_t sh_pages, sh_tret;
 
   const int g = blockIdx.x;
   const int tid = threadIdx.x;
   const int k2 = np + es;
-  constexpr int HB = RI_SEL_HI_BINS / SEL_THREADS;  // histogram bins per thread
 
-  // ---- loads: the group's histogram and keys ----
-  uint32_t hb[HB];
-#pragma unroll
-  for (int i = 0; i < HB; ++i) hb[i] = ghist[(size_t)g * RI_SEL_HI_BINS + tid * HB + i];
+  // ---- keys into LDS, histogram of all keys ----
   const int E = (((nc + SEL_THREADS - 1) / SEL_THREADS) + 7) & ~7;  // multiple of 8 (nc % 8 == 0)
   const int cbeg = min(tid * E, nc);
   const int cend = min(cbeg + E, nc);
-  for (int c = cbeg; c < cend; c += 8)
-    *reinterpret_cast<uint4*>(&sh_key[c]) = *reinterpret_cast<const uint4*>(keys + (size_t)g * nc + c);
-  if (tid < SEL_LO_BINS) hist_b[tid] = hist_c[tid] = 0;
-  if (tid == 0) { sh_cnt = 0; sh_pages = 0; sh_tret = 0; sh_nk = 0; }
-
-  // ---- bins of the two rank thresholds: T1 = key of rank np-1, T2 = key of rank k2-1 ----
-  {
-    uint32_t mine = 0;
+  uint4 kreg[8];  // E <= 64
 #pragma unroll
-    for (int i = 0; i < HB; ++i) mine += hb[i];
-    uint64_t tot;
-    const uint32_t below = (uint32_t)block_excl_scan<uint64_t>(mine, sh_scan, &tot);
-    uint32_t above = (uint32_t)tot - below - mine;  // entries in bins above this thread's
+  for (int i = 0; i < 8; ++i)
+    if (cbeg + 8 * i < cend) kreg[i] = *reinterpret_cast<const uint4*>(keys + (size_t)g * nc + cbeg + 8 * i);
+#pragma unroll
+  for (int i = 0; i < SEL_BPT; ++i) hist[tid * SEL_BPT + i] = 0u;
+  if (tid == 0) { sh_pages = 0; sh_tret = 0; }
+  __syncthreads();
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    if (cbeg + 8 * i < cend) {
+      *reinterpret_cast<uint4*>(&sh_key[cbeg + 8 * i]) = kreg[i];
+      const uint32_t w[4] = {kreg[i].x, kreg[i].y, kreg[i].z, kreg[i].w};
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        hist_add(hist, sel_bin(w[q] & 0xffffu), true);
+        hist_add(hist, sel_bin(w[q] >> 16), true);
+      }
+    }
+  }
+  __syncthreads();
+
+  // ---- rank thresholds: T1 = key of descending rank np-1, T2 = key of rank k2-1 ----
+  // thread t owns bins [t*17, t*17+17); afterwards hist[b] holds the number of keys above bin b
+  {
+    uint32_t hb[SEL_BPT], mine = 0;
+#pragma unroll
+    for (int i = 0; i < SEL_BPT; ++i) { hb[i] = hist[tid * SEL_BPT + i]; mine += hb[i]; }
+    uint32_t vin[1] = {mine}, below[1], tot[1];
+    block_excl_scan<1>(vin, below, tot, sh_scan[0]);
+    uint32_t above = tot[0] - below[0] - mine;  // entries in bins above this thread's
     const uint32_t rankA = (uint32_t)(np - 1), rankB = (uint32_t)(k2 - 1);
 #pragma unroll
-    for (int i = HB - 1; i >= 0; --i) {
-      if (above <= rankA && rankA < above + hb[i]) { sh_sel[0] = tid * HB + i; sh_sel[1] = above; }
-      if (above <= rankB && rankB < above + hb[i]) { sh_sel[2] = tid * HB + i; sh_sel[3] = above; }
+    for (int i = SEL_BPT - 1; i >= 0; --i) {
+      if (above <= rankA && rankA < above + hb[i]) { sh_sel[0] = tid * SEL_BPT + i; sh_sel[1] = above; }
+      if (above <= rankB && rankB < above + hb[i]) { sh_sel[2] = tid * SEL_BPT + i; sh_sel[3] = above; }
+      hist[tid * SEL_BPT + i] = above;
       above += hb[i];
     }
   }
   __syncthreads();
-  const uint32_t hi1 = sh_sel[0], hi2 = sh_sel[2];
-  for (int c = cbeg; c < cbeg + E; ++c) {  // same trip count in every lane
-    const bool in = c < cend;
-    const uint32_t key = in ? sh_key[c] : 0u;
-    hist_add(hist_b, key & (SEL_LO_BINS - 1), in && (key >> SEL_LO_BITS) == hi1);
-    hist_add(hist_c, key & (SEL_LO_BINS - 1), in && (key >> SEL_LO_BITS) == hi2);
-  }
-  __syncthreads();
-  if (tid == 0) find_lo_bin(hist_b, (uint32_t)(np - 1) - sh_sel[1], sh_sel + 4);
-  if (tid == 64) find_lo_bin(hist_c, (uint32_t)(k2 - 1) - sh_sel[3], sh_sel + 6);
-  __syncthreads();
-  const uint32_t T1 = (hi1 << SEL_LO_BITS) | sh_sel[4];
-  const uint32_t T2 = (hi2 << SEL_LO_BITS) | sh_sel[6];
-  const uint32_t g1 = sh_sel[1] + sh_sel[5];  // keys strictly above T1
-  const uint32_t g2 = sh_sel[3] + sh_sel[7];  // keys strictly above T2
+  const uint32_t B1 = sh_sel[0], B2 = sh_sel[2];  // threshold bins (bins order like keys)
+  const uint32_t g1 = sh_sel[1], g2 = sh_sel[3];  // keys strictly above T1 / T2
 
   // ---- one scan ranks everything: ties at T1, ties at T2 and the keys strictly between ----
   // Tied keys are taken in ascending id order: tie rank r at T1 belongs to the retrieval zone
   // while g1 + r < np, then to the estimation zone while g1 + r < k2; at T2 while g2 + r < k2.
   uint32_t n1 = 0, n2 = 0, nmid = 0;
   for (int c = cbeg; c < cend; ++c) {
-    const uint32_t key = sh_key[c];
-    n1 += (key == T1);
-    n2 += (key == T2 && T2 != T1);
-    nmid += (key < T1 && key > T2);
+    const uint32_t b = sel_bin(sh_key[c]);
+    n1 += (b == B1);
+    n2 += (b == B2 && B2 != B1);
+    nmid += (b < B1 && b > B2);
   }
-  uint64_t tot64;
-  const uint64_t pre = block_excl_scan<uint64_t>((uint64_t)n1 | ((uint64_t)n2 << 20) | ((uint64_t)nmid << 40),
-                                                 sh_scan, &tot64);
-  uint32_t r1 = (uint32_t)(pre & 0xfffff), r2 = (uint32_t)((pre >> 20) & 0xfffff);
-  const uint32_t mid_before = (uint32_t)(pre >> 40);
-  // estimation members among the first r ties
-  const uint32_t lo1 = (uint32_t)np > g1 ? (uint32_t)np - g1 : 0u;          // first tie rank of T1 in the est zone
-  const uint32_t hi1r = (uint32_t)k2 > g1 ? (uint32_t)k2 - g1 : 0u;         // one past the last
+  uint32_t cnt3[3] = {n1, n2, nmid}, pre3[3], tot3[3];
+  block_excl_scan<3>(cnt3, pre3, tot3, sh_scan[1]);
+  uint32_t r1 = pre3[0], r2 = pre3[1];
+  const uint32_t mid_before = pre3[2];
+  const uint32_t lo1 = (uint32_t)np > g1 ? (uint32_t)np - g1 : 0u;   // first tie rank of T1 in the est zone
+  const uint32_t hi1r = (uint32_t)k2 > g1 ? (uint32_t)k2 - g1 : 0u;  // one past the last
   const uint32_t hi2r = (uint32_t)k2 > g2 ? (uint32_t)k2 - g2 : 0u;
-  auto est_of_t1 = [&](uint32_t r) { return min(max(r, lo1), hi1r) - lo1; };
-  auto est_of_t2 = [&](uint32_t r) { return min(r, hi2r); };
-  uint32_t est_off = mid_before + est_of_t1(r1) + est_of_t2(r2);
+  uint32_t est_off = mid_before + (min(max(r1, lo1), hi1r) - lo1) + min(r2, hi2r);
   for (int c = cbeg; c < cend; ++c) {
     const uint32_t key = sh_key[c];
+    const uint32_t b = sel_bin(key);
     bool in_ret, in_est;
-    if (key == T1) {
+    uint32_t slot;
+    if (b == B1) {
       in_ret = r1 < lo1;
       in_est = !in_ret && r1 < hi1r;
+      slot = g1 + r1;  // ties enter in id order
       ++r1;
-    } else if (key == T2) {
+    } else if (b == B2) {
       in_ret = false;
       in_est = r2 < hi2r;
+      slot = 0;
       ++r2;
     } else {
-      in_ret = key > T1;
-      in_est = !in_ret && key > T2;
+      in_ret = b > B1;
+      in_est = !in_ret && b > B2;
+      slot = in_ret ? atomicAdd(&hist[b], 1u) : 0u;  // hist[b] = keys above b: ranks of b start there
     }
-    if (in_ret) {
-      const uint32_t slot = atomicAdd(&sh_cnt, 1u);
-      sh_ret[slot] = (key << 16) | (0xffffu - (uint32_t)c);
-    }
+    if (in_ret) sh_ret[slot] = (key << 16) | (0xffffu - (uint32_t)c);
     if (in_est) {
       est_ids[(size_t)g * es + est_off] = c;
       if (cI) cI[(size_t)g * k2 + np + est_off] = c;
@@ -261,87 +268,58 @@ __global__ __launch_bounds__(SEL_THREADS) void select_kernel(
   }
   __syncthreads();
 
-  // ---- order the retrieval zone: rank = number of larger composite keys (all distinct) ----
+  // ---- rank order: sh_ret is ordered by score; order runs of equal scores by ascending id ----
   for (int r = tid; r < np; r += SEL_THREADS) {
     const uint32_t mine = sh_ret[r];
-    int rank = 0;
-    for (int i = 0; i < np; ++i) rank += (sh_ret[i] > mine);
-    sh_sorted[rank] = mine;
+    const uint32_t kk = mine >> 16;
+    int lo = r, rank_in_run = 0;
+    while (lo > 0 && (sh_ret[lo - 1] >> 16) == kk) { --lo; rank_in_run += (sh_ret[lo] > mine); }
+    int hi = r;
+    while (hi + 1 < np && (sh_ret[hi + 1] >> 16) == kk) { ++hi; rank_in_run += (sh_ret[hi] > mine); }
+    sh_sorted[lo + rank_in_run] = mine;
   }
   __syncthreads();
 
   // ---- token layout of the retrieved clusters with the page cut-off ----
-  // thread t owns ranks [t*R, t*R+R)
-  const int R = (np + SEL_THREADS - 1) / SEL_THREADS;  // <= 4 for np <= 1023
-  uint32_t szs[4], pgs[4];
-  int32_t sts[4];
-  uint32_t psum = 0, tsum = 0;
-#pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    const int r = tid * R + i;
-    szs[i] = pgs[i] = 0;
-    sts[i] = 0;
-    if (i < R && r < np) {
-      const int c = (int)(0xffffu - (sh_sorted[r] & 0xffffu));
-      ret_ids[(size_t)g * np + r] = c;
-      if (cI) cI[(size_t)g * k2 + r] = c;
-      if (cluster_size) {
-        szs[i] = (uint32_t)cluster_size[(size_t)g * nc + c];
-        pgs[i] = (szs[i] + page - 1) / page;
-        if (cluster_start) sts[i] = cluster_start[(size_t)g * nc + c];
-      }
+  // thread r owns rank r (np <= 1023 < threads)
+  uint32_t sz = 0, pg = 0;
+  int32_t st = 0;
+  const int r = tid;
+  if (r < np) {
+    const int c = (int)(0xffffu - (sh_sorted[r] & 0xffffu));
+    ret_ids[(size_t)g * np + r] = c;
+    if (cI) cI[(size_t)g * k2 + r] = c;
+    if (cluster_size) {
+      sz = (uint32_t)cluster_size[(size_t)g * nc + c];
+      pg = (sz + page - 1) / page;
+      if (cluster_start) st = cluster_start[(size_t)g * nc + c];
     }
-    psum += pgs[i];
-    tsum += szs[i];
   }
   if (!cluster_size) return;
-  const uint64_t lay = block_excl_scan<uint64_t>((uint64_t)psum | ((uint64_t)tsum << 32), sh_scan, &tot64);
-  uint32_t pg_run = (uint32_t)lay, tok_run = (uint32_t)(lay >> 32);
+  uint32_t lay[2] = {pg, sz}, layp[2], layt[2];
+  block_excl_scan<2>(lay, layp, layt, sh_scan[0]);
+  const uint32_t pg_run = layp[0], tok_run = layp[1];
   // kept clusters form a prefix because the page prefix is monotone; tokens before a kept
   // cluster all belong to kept clusters
-  int kept_here = 0;
-#pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    const int r = tid * R + i;
-    if (i < R && r < np) {
-      const bool keep = pg_run + pgs[i] <= (uint32_t)max_pages;
-      if (keep) {
-        ++kept_here;
-        sh_off[r] = (int32_t)tok_run;
-        sh_ret[r] = (uint32_t)sts[i];  // sh_ret is free again: start row per rank
-        atomicMax(&sh_pages, pg_run + pgs[i]);
-        atomicMax(&sh_tret, tok_run + szs[i]);
-      } else {
-        sh_off[r] = -1;
-      }
-      pg_run += pgs[i];
-      tok_run += szs[i];
-    }
+  const bool keep = r < np && pg_run + pg <= (uint32_t)max_pages;
+  if (keep) {
+    atomicMax(&sh_pages, pg_run + pg);
+    atomicMax(&sh_tret, tok_run + sz);
   }
-  if (kept_here) atomicAdd(&sh_nk, kept_here);
-  __syncthreads();
-  const int nkeep = sh_nk;
+  const int nkeep = __syncthreads_count(keep);
   const int32_t T_ret = (int32_t)sh_tret;
-  for (int r = tid; r <= np; r += SEL_THREADS) {
-    const int32_t off = (r < nkeep) ? sh_off[r] : T_ret;
-    ret_tok_off[(size_t)g * (np + 1) + r] = off;
-  }
+  if (r <= np) ret_tok_off[(size_t)g * (np + 1) + r] = (r < nkeep) ? (int32_t)tok_run : T_ret;
   if (tid == 0) {
     meta[g * 4 + 0] = nkeep;
     meta[g * 4 + 1] = T_ret;
     meta[g * 4 + 2] = (int32_t)sh_pages;
     meta[g * 4 + 3] = 0;
   }
-  if (!row_src || !cluster_start) return;
-  for (int rho = tid; rho < T_ret && rho < row_src_stride; rho += SEL_THREADS) {
-    // last kept cluster r with sh_off[r] <= rho  (offsets of kept clusters are non-decreasing)
-    int lo = 0, hi = nkeep - 1;
-    while (lo < hi) {
-      const int mid = (lo + hi + 1) >> 1;
-      if (sh_off[mid] <= rho) lo = mid; else hi = mid - 1;
-    }
-    row_src[(size_t)g * row_src_stride + rho] = (int32_t)sh_ret[lo] + (rho - sh_off[lo]);
-  }
+  // row table: each kept cluster writes the rows of its tokens
+  if (!row_src || !cluster_start || !keep) return;
+  int32_t* dst = row_src + (size_t)g * row_src_stride + tok_run;
+  const int room = row_src_stride - (int)tok_run;
+  for (int i = 0; i < (int)sz && i < room; ++i) dst[i] = st + i;
 }
 
 // ------------------------------------------------------------------------------------
@@ -352,8 +330,7 @@ static size_t align256(size_t x) { return (x + 255) & ~(size_t)255; }
 extern "C" size_t ri_score_select_workspace_bytes(int BG, int gs, int nc) {
   if (BG <= 0 || gs <= 0 || nc <= 0) return 0;
   const size_t ntiles = (size_t)(nc + RI_SCORE_TILE - 1) / RI_SCORE_TILE;
-  return 2 * align256((size_t)BG * ntiles * gs * sizeof(float)) + align256((size_t)BG * nc * sizeof(uint16_t)) +
-         align256((size_t)BG * RI_SEL_HI_BINS * sizeof(uint32_t));
+  return 2 * align256((size_t)BG * ntiles * gs * sizeof(float)) + align256((size_t)BG * nc * sizeof(uint16_t));
 }
 
 extern "C" int ri_score_select(const void* q, const void* centroids, const uint8_t* mask,
@@ -377,21 +354,19 @@ extern "C" int ri_score_select(const void* q, const void* centroids, const uint8
   float* tsum = (float*)w;
   w += align256((size_t)BG * ntiles * gs * sizeof(float));
   uint16_t* keys = (uint16_t*)w;
-  w += align256((size_t)BG * nc * sizeof(uint16_t));
-  uint32_t* ghist = (uint32_t*)w;
-  int rc = ri_launch_score(q, centroids, logits, tmax, tsum, ghist, BG, gs, nc, scale, s);
+  int rc = ri_launch_score(q, centroids, logits, tmax, tsum, BG, gs, nc, scale, s);
   if (rc) return rc;
   const dim3 dgrid((nc + DIST_IDS - 1) / DIST_IDS, BG);
   if (gs <= 4)
-    dist_kernel<4><<<dgrid, 256, 0, s>>>(logits, tmax, tsum, mask, keys, (uint16_t*)dist, ghist, gs, nc, ntiles);
+    dist_kernel<4><<<dgrid, 256, 0, s>>>(logits, tmax, tsum, mask, keys, (uint16_t*)dist, gs, nc, ntiles);
   else if (gs <= 8)
-    dist_kernel<8><<<dgrid, 256, 0, s>>>(logits, tmax, tsum, mask, keys, (uint16_t*)dist, ghist, gs, nc, ntiles);
+    dist_kernel<8><<<dgrid, 256, 0, s>>>(logits, tmax, tsum, mask, keys, (uint16_t*)dist, gs, nc, ntiles);
   else
-    dist_kernel<16><<<dgrid, 256, 0, s>>>(logits, tmax, tsum, mask, keys, (uint16_t*)dist, ghist, gs, nc, ntiles);
+    dist_kernel<16><<<dgrid, 256, 0, s>>>(logits, tmax, tsum, mask, keys, (uint16_t*)dist, gs, nc, ntiles);
   RI_HIP_CHECK_LAUNCH();
   select_kernel<<<BG, SEL_THREADS, (size_t)nc * sizeof(uint16_t) + 64, s>>>(
-      keys, ghist, cluster_size_i32, cluster_start, cI, ret_ids, est_ids, ret_tok_off, row_src, row_src_stride,
-      meta, nc, np, es, page, max_pages);
+      keys, cluster_size_i32, cluster_start, cI, ret_ids, est_ids, ret_tok_off, row_src, row_src_stride, meta, nc,
+      np, es, page, max_pages);
   RI_HIP_CHECK_LAUNCH();
   return RI_OK;
 }
