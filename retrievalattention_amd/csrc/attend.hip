@@ -81,34 +81,44 @@ __device__ __forceinline__ int ri_head_of(int h, int i) {
   return (4 * h + ri_head_reg<GS_PAD>(h) + i) % GS_PAD;
 }
 
+typedef short bf16x4s_t __attribute__((ext_vector_type(4)));
+
+#define ATT_VT_STRIDE 144  // LDS row stride of the 16 x 128 value tile in bf16 elements (288 bytes)
+
 template <int GS_PAD>
 struct WaveState {
   float m[GS_PAD / 4];
   float l[GS_PAD / 4];
-  float acc[GS_PAD][8];
+  // P·V accumulators in MFMA 16x16 layout: acc[dt][i] of lane l = head 4*(l/16)+i, dim 16*dt + l%16
+  f32x4_t acc[8];
 };
 
-// softmax update for one chunk: scores s_in[4] (this lane: row n = lane%16, MFMA registers of
-// lane group h = lane/16), validity and denominator weight; then the P·V accumulation of the
-// four value rows v[4] this lane owns.  p_sh: [16][GS_PAD] floats, al_sh: [GS_PAD] floats of this wave.
+__device__ __forceinline__ uint16_t ri_to_bf16_hw(float x) {
+  const __bf16 b = (__bf16)x;
+  return __builtin_bit_cast(uint16_t, b);
+}
+
+// One chunk of 16 rows.
+//   sv[NH]  scores of the heads this lane keeps for row n = lane%16 (lane group h = lane/16)
+//   v[4]    value rows h, h+4, h+8, h+12 of the chunk, dims 8n..8n+7 (as loaded from memory)
+// Softmax bookkeeping in fp32 per lane; P goes to LDS as bf16 [head][row], the value tile to LDS
+// row-major; P·V = 8 MFMA 16x16x16 whose B operands come from LDS transpose reads
+// (ds_read_b64_tr_b16: lane l of a 16-lane group receives element l%4 of the 8-byte pieces
+// addressed by lanes l/4, l/4+4, l/4+8, l/4+12 — four consecutive rows of one column).
 template <int GS_PAD>
-__device__ __forceinline__ void chunk_update(WaveState<GS_PAD>& st, const float s_in[4], bool valid, float w,
-                                             const uint4 v[4], float* p_sh, float* al_sh, int lane) {
+__device__ __forceinline__ void chunk_update(WaveState<GS_PAD>& st, const float* sv, bool valid, float w,
+                                             const uint4 v[4], uint16_t* vt, uint16_t* pb, float* al_sh,
+                                             int lane) {
   constexpr int NH = GS_PAD / 4;
   const int n = lane & 15, h = lane >> 4;
-  const int r0 = ri_head_reg<GS_PAD>(h);
+  // value tile -> LDS
+#pragma unroll
+  for (int i = 0; i < 4; ++i) *reinterpret_cast<uint4*>(vt + (h + 4 * i) * ATT_VT_STRIDE + 8 * n) = v[i];
   float al[NH];
   bool rescale = false;
 #pragma unroll
   for (int i = 0; i < NH; ++i) {
-    float sv;
-    if (GS_PAD == 16) {
-      sv = s_in[i];
-    } else {  // pick register r0 + i without dynamic indexing
-      const int r = r0 + i;
-      sv = r == 0 ? s_in[0] : (r == 1 ? s_in[1] : (r == 2 ? s_in[2] : s_in[3]));
-    }
-    const float s = valid ? sv : -INFINITY;
+    const float s = valid ? sv[i] : -INFINITY;
     float cm = s;
     cm = fmaxf(cm, __shfl_xor(cm, 1));
     cm = fmaxf(cm, __shfl_xor(cm, 2));
@@ -126,7 +136,7 @@ __device__ __forceinline__ void chunk_update(WaveState<GS_PAD>& st, const float 
     rescale |= (al[i] != 1.f);
     st.l[i] = st.l[i] * al[i] + w * p;
     st.m[i] = mn;
-    p_sh[n * GS_PAD + ri_head_of<GS_PAD>(h, i)] = p;
+    pb[ri_head_of<GS_PAD>(h, i) * 16 + n] = ri_to_bf16_hw(p);
   }
   // the running maximum rarely moves after the first chunks: rescale only when some head's did
   const bool any_rescale = __any(rescale);
@@ -138,33 +148,23 @@ __device__ __forceinline__ void chunk_update(WaveState<GS_PAD>& st, const float 
   __builtin_amdgcn_wave_barrier();
   __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
   if (any_rescale) {
+    const float4 a4 = *reinterpret_cast<const float4*>(al_sh + 4 * h);
 #pragma unroll
-    for (int j = 0; j < GS_PAD; j += 4) {
-      const float4 a4 = *reinterpret_cast<const float4*>(al_sh + j);
-      const float alpha[4] = {a4.x, a4.y, a4.z, a4.w};
-#pragma unroll
-      for (int jj = 0; jj < 4; ++jj)
-#pragma unroll
-        for (int e = 0; e < 8; ++e) st.acc[j + jj][e] *= alpha[jj];
+    for (int dt = 0; dt < 8; ++dt) {
+      st.acc[dt][0] *= a4.x; st.acc[dt][1] *= a4.y; st.acc[dt][2] *= a4.z; st.acc[dt][3] *= a4.w;
     }
   }
+  // A operand: P[head n][rows 4h..4h+3]
+  const bf16x4s_t pa = *reinterpret_cast<const bf16x4s_t*>(pb + n * 16 + 4 * h);
+  const uint16_t* vsrc = vt + (4 * h + (n >> 2)) * ATT_VT_STRIDE + 4 * (n & 3);
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    float vf[8];
-    ri_unpack8(v[i], vf);
-    const int row = h + 4 * i;
-#pragma unroll
-    for (int j = 0; j < GS_PAD; j += 4) {
-      const float4 p4 = *reinterpret_cast<const float4*>(p_sh + row * GS_PAD + j);
-      const float pj[4] = {p4.x, p4.y, p4.z, p4.w};
-#pragma unroll
-      for (int jj = 0; jj < 4; ++jj)
-#pragma unroll
-        for (int e = 0; e < 8; ++e) st.acc[j + jj][e] = fmaf(pj[jj], vf[e], st.acc[j + jj][e]);
-    }
+  for (int dt = 0; dt < 8; ++dt) {
+    const bf16x4s_t vb = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+        (bf16x4s_t __attribute__((address_space(3)))*)(vsrc + 16 * dt));
+    st.acc[dt] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(pa, vb, st.acc[dt], 0, 0, 0);
   }
   __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-  __builtin_amdgcn_wave_barrier();  // p_sh is rewritten by the next chunk
+  __builtin_amdgcn_wave_barrier();  // the tile and P are rewritten by the next chunk
 }
 
 // rows of a wave: the group's `total` rows are cut into `nwaves` runs of a multiple of 16 rows
@@ -176,57 +176,70 @@ __device__ __forceinline__ void wave_rows(int total, int nwaves, int wid, int* r
 }
 
 // Merges the S split partials of group g (and the optional previous result) and writes the
-// output; called by all 256 threads of one workgroup.
-template <bool COHERENT>
-__device__ __forceinline__ float ld_part(const float* p) {
-  return COHERENT ? __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : *p;
-}
-
-template <int GS_PAD, bool COHERENT>
+// output: wave w of the calling workgroup takes heads w, w+4, ...; lanes first cover the splits
+// (statistics), then two dims each.
+template <int GS_PAD>
 __device__ __forceinline__ void combine_group(const AttendParams& P, int g, int S, int lenB) {
   const int gs = P.gs;
-  for (int idx = threadIdx.x; idx < gs * (RI_DIM / 2); idx += 256) {
-    const int j = idx / (RI_DIM / 2), d2 = (idx % (RI_DIM / 2)) * 2;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  for (int j = wave; j < gs; j += 4) {
     const float* ml = P.part_ml + ((size_t)g * S * GS_PAD + j) * 2;
-    const float* pa = P.part_acc + ((size_t)g * S * GS_PAD + j) * RI_DIM + d2;
-    float M = P.prev_lse ? P.prev_lse[(size_t)g * gs + j] : -INFINITY;
-#pragma unroll 8
-    for (int s = 0; s < S; ++s) M = fmaxf(M, ld_part<COHERENT>(ml + (size_t)s * GS_PAD * 2));
-    float L = 0.f, A0 = 0.f, A1 = 0.f;
+    const float* pa = P.part_acc + ((size_t)g * S * GS_PAD + j) * RI_DIM + 2 * lane;
+    float2 ms = make_float2(-INFINITY, 0.f);
+    if (lane < S) ms = *reinterpret_cast<const float2*>(ml + (size_t)lane * GS_PAD * 2);
+    const float pl = P.prev_lse ? P.prev_lse[(size_t)g * gs + j] : -INFINITY;
+    float M = fmaxf(ms.x, pl);
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) M = fmaxf(M, __shfl_xor(M, o));
+    const float f = (ms.x == -INFINITY) ? 0.f : __expf(ms.x - M);
+    float L = ms.y * f;
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) L += __shfl_xor(L, o);
+    float A0 = 0.f, A1 = 0.f;
     if (P.prev_lse) {
-      const float pl = P.prev_lse[(size_t)g * gs + j];
-      const float f = (pl == -INFINITY) ? 0.f : __expf(pl - M);
-      const uint32_t po = *reinterpret_cast<const uint32_t*>(P.prev_out + ((size_t)g * gs + j) * RI_DIM + d2);
-      L = f;
-      A0 = f * __uint_as_float(po << 16);
-      A1 = f * __uint_as_float(po & 0xffff0000u);
+      const float fp = (pl == -INFINITY) ? 0.f : __expf(pl - M);
+      const uint32_t po = *reinterpret_cast<const uint32_t*>(P.prev_out + ((size_t)g * gs + j) * RI_DIM + 2 * lane);
+      L += fp;
+      A0 = fp * __uint_as_float(po << 16);
+      A1 = fp * __uint_as_float(po & 0xffff0000u);
     }
-#pragma unroll 8
-    for (int s = 0; s < S; ++s) {
-      const float m = ld_part<COHERENT>(ml + (size_t)s * GS_PAD * 2);
-      const float f = (m == -INFINITY) ? 0.f : __expf(m - M);
-      const float a0 = ld_part<COHERENT>(pa + (size_t)s * GS_PAD * RI_DIM);
-      const float a1 = ld_part<COHERENT>(pa + (size_t)s * GS_PAD * RI_DIM + 1);
-      L += ld_part<COHERENT>(ml + (size_t)s * GS_PAD * 2 + 1) * f;
-      A0 += a0 * f;
-      A1 += a1 * f;
+    // numerators: loads are issued eight at a time, ahead of the factors they are scaled by
+    for (int s0 = 0; s0 < S; s0 += 8) {
+      float2 a2[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u)
+        a2[u] = (s0 + u < S) ? *reinterpret_cast<const float2*>(pa + (size_t)(s0 + u) * GS_PAD * RI_DIM)
+                             : make_float2(0.f, 0.f);
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        const float fs = __shfl(f, (s0 + u) & 63);
+        A0 += a2[u].x * fs;
+        A1 += a2[u].y * fs;
+      }
     }
     const uint32_t o = (uint32_t)ri_f32_to_bf16(A0 / L) | ((uint32_t)ri_f32_to_bf16(A1 / L) << 16);
-    *reinterpret_cast<uint32_t*>(P.out + ((size_t)g * gs + j) * RI_DIM + d2) = o;
-    if (d2 == 0 && P.lse_out) P.lse_out[(size_t)g * gs + j] = M + __logf(L);
+    *reinterpret_cast<uint32_t*>(P.out + ((size_t)g * gs + j) * RI_DIM + 2 * lane) = o;
+    if (lane == 0 && P.lse_out) P.lse_out[(size_t)g * gs + j] = M + __logf(L);
   }
   if (threadIdx.x == 0 && P.valid_lengths) P.valid_lengths[g] = P.lenA + lenB;
 }
 
-// CH = chunks (of 16 rows) a wave loads ahead of computing
-template <int GS_PAD, int CH>
-__global__ __launch_bounds__(256, 2) void attend_kernel(AttendParams P) {
-  __shared__ float sh_p[4][16 * GS_PAD];
-  __shared__ float sh_al[4][GS_PAD];
+#define ATT_DESC_MAX 512  // rows of one wave whose descriptors are staged in LDS at a time
+
+// PF = chunks (of 16 rows) in flight per wave: the loads of chunk j+PF are issued before chunk j
+// is computed
+template <int GS_PAD, int PF>
+__global__ __launch_bounds__(256, GS_PAD == 16 ? 1 : 2) void attend_kernel(AttendParams P) {
+  constexpr int NH = GS_PAD / 4;
+  __shared__ __attribute__((aligned(16))) uint16_t sh_vt[4][16 * ATT_VT_STRIDE];
+  __shared__ __attribute__((aligned(16))) uint16_t sh_pb[4][16 * 16];
+  __shared__ float sh_al[4][16];
   __shared__ float sh_m[4][GS_PAD];
   __shared__ float sh_l[4][GS_PAD];
   __shared__ float sh_acc[4][GS_PAD][RI_DIM];
   __shared__ __attribute__((aligned(16))) uint16_t sh_q[GS_PAD][RI_DIM];
+  __shared__ int sh_desc[4][ATT_DESC_MAX];
+  __shared__ float sh_w[4][ATT_DESC_MAX];
   __shared__ int sh_last;
 
   const int g = blockIdx.y;
@@ -235,18 +248,21 @@ __global__ __launch_bounds__(256, 2) void attend_kernel(AttendParams P) {
   const int wave = threadIdx.x >> 6;
   const int n = lane & 15, h = lane >> 4;
   const int gs = P.gs;
-  constexpr int ND = (CH * 16 + 63) / 64;  // descriptor registers per batch
 
   WaveState<GS_PAD> st;
 #pragma unroll
-  for (int i = 0; i < GS_PAD / 4; ++i) { st.m[i] = -INFINITY; st.l[i] = 0.f; }
+  for (int i = 0; i < NH; ++i) { st.m[i] = -INFINITY; st.l[i] = 0.f; }
 #pragma unroll
-  for (int j = 0; j < GS_PAD; ++j)
-#pragma unroll
-    for (int e = 0; e < 8; ++e) st.acc[j][e] = 0.f;
+  for (int dt = 0; dt < 8; ++dt) st.acc[dt] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
 
-  float* p_sh = sh_p[wave];
+  uint16_t* vt = sh_vt[wave];
+  uint16_t* pb = sh_pb[wave];
   float* al_sh = sh_al[wave];
+  // P rows of heads that do not exist stay zero; alpha of such heads must not scale by garbage
+  for (int i = lane; i < 16 * 16 / 2; i += 64) reinterpret_cast<uint32_t*>(pb)[i] = 0u;
+  if (lane < 16) al_sh[lane] = 1.f;
+  int* dsc = sh_desc[wave];
+  float* wsh = sh_w[wave];
   const int lenB = P.lenB_ptr ? P.lenB_ptr[(size_t)g * P.lenB_ptr_stride] : P.lenB_const;
 
   if (split < P.S_kv) {
@@ -262,7 +278,6 @@ __global__ __launch_bounds__(256, 2) void attend_kernel(AttendParams P) {
       *reinterpret_cast<uint4*>(&sh_q[head][piece * 8]) =
           (head < gs) ? ri_ld16(P.q + ((size_t)g * gs + head) * RI_DIM + piece * 8) : ri_zero16();
     }
-    __syncthreads();
     const uint16_t* qrow = &sh_q[n % GS_PAD][h * 8];
     const uint16_t* kA = P.kA + (size_t)g * P.strideA * RI_DIM;
     const uint16_t* vA = P.vA + (size_t)g * P.strideA * RI_DIM;
@@ -270,58 +285,84 @@ __global__ __launch_bounds__(256, 2) void attend_kernel(AttendParams P) {
     const uint16_t* vB = P.vB + (size_t)g * P.strideB * RI_DIM;
     const int32_t* rs = P.row_src ? P.row_src + (size_t)g * P.rs_stride : nullptr;
     const uint16_t* wB = P.weightB ? P.weightB + (size_t)g * P.weight_stride : nullptr;
+    const int r_first = ri_head_reg<GS_PAD>(h);
+    bool q_ready = false;
 
-    for (int b0 = r0; b0 < r1; b0 += 16 * CH) {
-      // descriptors, one row per lane and register: where row b0 + 64*k + lane lives (-1 = past the end)
-      int desc[ND];
-      float wd[ND];
-#pragma unroll
-      for (int k = 0; k < ND; ++k) {
-        desc[k] = -1;
-        wd[k] = 1.f;
-        const int row = b0 + 64 * k + lane;
-        if (row < r1 && 64 * k + lane < 16 * CH) {
+    for (int s0 = r0; s0 < r1; s0 += ATT_DESC_MAX) {
+      const int s1 = min(r1, s0 + ATT_DESC_MAX);
+      // stage the descriptors of rows [s0, s1): where each row lives (-1 = padding row)
+      for (int i = lane; i < ATT_DESC_MAX; i += 64) {
+        const int row = s0 + i;
+        int d = -1;
+        float w = 1.f;
+        if (row < s1) {
           if (row < P.lenA) {
-            desc[k] = row | ATT_FLAG_A;
+            d = row | ATT_FLAG_A;
           } else {
             const int rb = row - P.lenA;
-            desc[k] = rs ? rs[rb] : rb;
-            if (wB) wd[k] = ri_bf16_to_f32(wB[rb]);
+            d = rs ? rs[rb] : rb;
+            if (wB) w = ri_bf16_to_f32(wB[rb]);
           }
         }
+        dsc[i] = d;
+        wsh[i] = w;
       }
-      const int nch = min(CH, (r1 - b0 + 15) >> 4);
-      uint4 bk[CH][4], v[CH][4];
+      if (!q_ready) { __syncthreads(); q_ready = true; }  // sh_q complete (also orders dsc writes)
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+      const int nch = (s1 - s0 + 15) >> 4;
+      uint4 bk[PF][4], v[PF][4];
+      auto issue = [&](int slot_unused, uint4* bks, uint4* vs_, int j) {
+        (void)slot_unused;
+        const int dk = dsc[j * 16 + n];
+        const uint16_t* kp = ((dk & ATT_FLAG_A) ? kA : kB) + (size_t)(dk & ~ATT_FLAG_A) * RI_DIM + h * 8;
 #pragma unroll
-      for (int ch = 0; ch < CH; ++ch) {
-        if (ch < nch) {
-          const int dk = __shfl(desc[ch / 4], (ch % 4) * 16 + n);
-          const uint16_t* kp = ((dk & ATT_FLAG_A) ? kA : kB) + (size_t)(dk & ~ATT_FLAG_A) * RI_DIM + h * 8;
+        for (int kk = 0; kk < 4; ++kk) bks[kk] = (dk >= 0) ? ri_ld16(kp + kk * 32) : ri_zero16();
 #pragma unroll
-          for (int kk = 0; kk < 4; ++kk) bk[ch][kk] = (dk >= 0) ? ri_ld16(kp + kk * 32) : ri_zero16();
-#pragma unroll
-          for (int i = 0; i < 4; ++i) {
-            const int dv = __shfl(desc[ch / 4], (ch % 4) * 16 + h + 4 * i);
-            const uint16_t* vp = ((dv & ATT_FLAG_A) ? vA : vB) + (size_t)(dv & ~ATT_FLAG_A) * RI_DIM + n * 8;
-            v[ch][i] = (dv >= 0) ? ri_ld16(vp) : ri_zero16();
-          }
+        for (int i = 0; i < 4; ++i) {
+          const int dv = dsc[j * 16 + h + 4 * i];
+          const uint16_t* vp = ((dv & ATT_FLAG_A) ? vA : vB) + (size_t)(dv & ~ATT_FLAG_A) * RI_DIM + n * 8;
+          vs_[i] = (dv >= 0) ? ri_ld16(vp) : ri_zero16();
         }
-      }
+      };
+      auto compute = [&](const uint4* bks, const uint4* vs_, int j) {
+        f32x4_t acc = (f32x4_t){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-      for (int ch = 0; ch < CH; ++ch) {
-        if (ch < nch) {
-          f32x4_t acc = (f32x4_t){0.f, 0.f, 0.f, 0.f};
+        for (int kk = 0; kk < 4; ++kk)
+          acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+              ri_as_bf16x8(*reinterpret_cast<const uint4*>(qrow + kk * 32)), ri_as_bf16x8(bks[kk]), acc, 0, 0, 0);
+        float sv[NH];
 #pragma unroll
-          for (int kk = 0; kk < 4; ++kk)
-            acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
-                ri_as_bf16x8(*reinterpret_cast<const uint4*>(qrow + kk * 32)), ri_as_bf16x8(bk[ch][kk]), acc, 0, 0, 0);
-          const float s[4] = {acc[0] * P.scale, acc[1] * P.scale, acc[2] * P.scale, acc[3] * P.scale};
-          const bool valid = __shfl(desc[ch / 4], (ch % 4) * 16 + n) >= 0;
-          const float w = __shfl(wd[ch / 4], (ch % 4) * 16 + n);
-          chunk_update<GS_PAD>(st, s, valid, w, v[ch], p_sh, al_sh, lane);
+        for (int i = 0; i < NH; ++i) {
+          float x;
+          if (GS_PAD == 16) {
+            x = acc[i];
+          } else {  // register r_first + i without dynamic indexing
+            const int r = r_first + i;
+            x = r == 0 ? acc[0] : (r == 1 ? acc[1] : (r == 2 ? acc[2] : acc[3]));
+          }
+          sv[i] = x * P.scale;
+        }
+        const bool valid = dsc[j * 16 + n] >= 0;
+        const float w = wsh[j * 16 + n];
+        chunk_update<GS_PAD>(st, sv, valid, w, vs_, vt, pb, al_sh, lane);
+      };
+#pragma unroll
+      for (int s = 0; s < PF; ++s)
+        if (s < nch) issue(s, bk[s], v[s], s);
+      for (int j0 = 0; j0 < nch; j0 += PF) {
+#pragma unroll
+        for (int s = 0; s < PF; ++s) {
+          const int j = j0 + s;
+          if (j < nch) {
+            compute(bk[s], v[s], j);
+            if (j + PF < nch) issue(s, bk[s], v[s], j + PF);
+          }
         }
       }
     }
+    if (!q_ready) __syncthreads();  // keep the barrier count uniform for waves without rows
   } else {
     // ---------------- estimation rows ----------------
     const int es = P.es;
@@ -332,44 +373,51 @@ __global__ __launch_bounds__(256, 2) void attend_kernel(AttendParams P) {
     const uint16_t* cs = P.csize + (size_t)g * P.nc;
     const float* lg = P.logits + (size_t)g * gs * P.nc;
 
-    for (int b0 = r0; b0 < r1; b0 += 16 * CH) {
-      int cid[ND];
-      float wd[ND];
-#pragma unroll
-      for (int k = 0; k < ND; ++k) {
-        cid[k] = -1;
-        wd[k] = 0.f;
-        const int row = b0 + 64 * k + lane;
-        if (row < r1 && 64 * k + lane < 16 * CH) {
-          cid[k] = ids[row];
-          wd[k] = ri_bf16_to_f32(cs[cid[k]]);
+    for (int s0 = r0; s0 < r1; s0 += ATT_DESC_MAX) {
+      const int s1 = min(r1, s0 + ATT_DESC_MAX);
+      for (int i = lane; i < ATT_DESC_MAX; i += 64) {
+        const int row = s0 + i;
+        int d = -1;
+        float w = 0.f;
+        if (row < s1) {
+          d = ids[row];
+          w = ri_bf16_to_f32(cs[d]);
         }
+        dsc[i] = d;
+        wsh[i] = w;
       }
-      const int nch = min(CH, (r1 - b0 + 15) >> 4);
-      float sc[CH][4];
-      uint4 v[CH][4];
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+      const int nch = (s1 - s0 + 15) >> 4;
+      float sc[PF][NH];
+      uint4 v[PF][4];
+      auto issue = [&](float* scs, uint4* vs_, int j) {
+        const int ck = dsc[j * 16 + n];
 #pragma unroll
-      for (int ch = 0; ch < CH; ++ch) {
-        if (ch < nch) {
-          const int ck = __shfl(cid[ch / 4], (ch % 4) * 16 + n);
-#pragma unroll
-          for (int i = 0; i < 4; ++i) {
-            const int head = (4 * h + i) % GS_PAD;
-            sc[ch][i] = (ck >= 0 && head < gs) ? lg[(size_t)head * P.nc + ck] : -INFINITY;
-          }
-#pragma unroll
-          for (int i = 0; i < 4; ++i) {
-            const int cv = __shfl(cid[ch / 4], (ch % 4) * 16 + h + 4 * i);
-            v[ch][i] = (cv >= 0) ? ri_ld16(vs + (size_t)cv * RI_DIM + n * 8) : ri_zero16();
-          }
+        for (int i = 0; i < NH; ++i) {
+          const int head = ri_head_of<GS_PAD>(h, i);
+          scs[i] = (ck >= 0 && head < gs) ? lg[(size_t)head * P.nc + ck] : -INFINITY;
         }
-      }
 #pragma unroll
-      for (int ch = 0; ch < CH; ++ch) {
-        if (ch < nch) {
-          const bool valid = __shfl(cid[ch / 4], (ch % 4) * 16 + n) >= 0;
-          const float w = __shfl(wd[ch / 4], (ch % 4) * 16 + n);
-          chunk_update<GS_PAD>(st, sc[ch], valid, w, v[ch], p_sh, al_sh, lane);
+        for (int i = 0; i < 4; ++i) {
+          const int cv = dsc[j * 16 + h + 4 * i];
+          vs_[i] = (cv >= 0) ? ri_ld16(vs + (size_t)cv * RI_DIM + n * 8) : ri_zero16();
+        }
+      };
+#pragma unroll
+      for (int s = 0; s < PF; ++s)
+        if (s < nch) issue(sc[s], v[s], s);
+      for (int j0 = 0; j0 < nch; j0 += PF) {
+#pragma unroll
+        for (int s = 0; s < PF; ++s) {
+          const int j = j0 + s;
+          if (j < nch) {
+            const bool valid = dsc[j * 16 + n] >= 0;
+            const float w = wsh[j * 16 + n];
+            chunk_update<GS_PAD>(st, sc[s], valid, w, v[s], vt, pb, al_sh, lane);
+            if (j + PF < nch) issue(sc[s], v[s], j + PF);
+          }
         }
       }
     }
@@ -377,7 +425,7 @@ __global__ __launch_bounds__(256, 2) void attend_kernel(AttendParams P) {
 
   // ---------------- wave partial -> LDS ----------------
 #pragma unroll
-  for (int i = 0; i < GS_PAD / 4; ++i) {
+  for (int i = 0; i < NH; ++i) {
     float l = st.l[i];
     l += __shfl_xor(l, 1);
     l += __shfl_xor(l, 2);
@@ -388,21 +436,13 @@ __global__ __launch_bounds__(256, 2) void attend_kernel(AttendParams P) {
       sh_l[wave][ri_head_of<GS_PAD>(h, i)] = l;
     }
   }
+  // accumulators are already summed over rows: lane (n, h) register i holds head 4h+i, dim 16*dt+n
 #pragma unroll
-  for (int j = 0; j < GS_PAD; ++j)
+  for (int i = 0; i < 4; ++i) {
+    const int head = 4 * h + i;
+    if (head < GS_PAD) {
 #pragma unroll
-    for (int e = 0; e < 8; ++e) {
-      float a = st.acc[j][e];
-      a += __shfl_xor(a, 16);
-      a += __shfl_xor(a, 32);
-      st.acc[j][e] = a;
-    }
-  if (h == 0) {
-#pragma unroll
-    for (int j = 0; j < GS_PAD; ++j) {
-      float4* dst = reinterpret_cast<float4*>(&sh_acc[wave][j][n * 8]);
-      dst[0] = make_float4(st.acc[j][0], st.acc[j][1], st.acc[j][2], st.acc[j][3]);
-      dst[1] = make_float4(st.acc[j][4], st.acc[j][5], st.acc[j][6], st.acc[j][7]);
+      for (int dt = 0; dt < 8; ++dt) sh_acc[wave][head][16 * dt + n] = st.acc[dt][i];
     }
   }
   __syncthreads();
@@ -437,61 +477,26 @@ __global__ __launch_bounds__(256, 2) void attend_kernel(AttendParams P) {
 
   // ---------------- last workgroup of the group merges all splits ----------------
   if (!P.fuse) return;
-  // The partial went out with device-coherent stores; once they have completed (the barrier
-  // waits for this workgroup's outstanding stores) the arrival is announced.  The last
-  // workgroup to arrive reads every partial with device-coherent loads.
+  // The partial went out with device-coherent stores; once they have completed the arrival is
+  // announced.  The last workgroup to arrive drops its stale cache lines (acquire) and reads
+  // every partial.
   __builtin_amdgcn_s_waitcnt(0);
   __syncthreads();
   if (threadIdx.x == 0)
     sh_last = (__hip_atomic_fetch_add(&P.counters[g], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == S - 1);
   __syncthreads();
   if (!sh_last) return;
-  combine_group<GS_PAD, true>(P, g, S, lenB);
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+  combine_group<GS_PAD>(P, g, S, lenB);
   if (threadIdx.x == 0) P.counters[g] = 0;  // ready for the next launch
 }
 
-// separate merge pass: grid (gs, BG), one wave per (group, head); lanes first cover the
-// splits (statistics), then the dims (two each)
+// separate merge pass: grid (BG), 256 threads
 template <int GS_PAD>
-__global__ __launch_bounds__(64) void combine_kernel(AttendParams P) {
-  const int j = blockIdx.x, g = blockIdx.y, lane = threadIdx.x;
-  const int S = P.S_kv + P.S_es, gs = P.gs;
-  const float* ml = P.part_ml + ((size_t)g * S * GS_PAD + j) * 2;
-  const float* pa = P.part_acc + ((size_t)g * S * GS_PAD + j) * RI_DIM + 2 * lane;
-  float2 ms = make_float2(-INFINITY, 0.f);
-  if (lane < S) ms = *reinterpret_cast<const float2*>(ml + (size_t)lane * GS_PAD * 2);
-  const float pl = P.prev_lse ? P.prev_lse[(size_t)g * gs + j] : -INFINITY;
-  float M = fmaxf(ms.x, pl);
-#pragma unroll
-  for (int o = 32; o > 0; o >>= 1) M = fmaxf(M, __shfl_xor(M, o));
-  const float f = (ms.x == -INFINITY) ? 0.f : __expf(ms.x - M);
-  float L = ms.y * f;
-#pragma unroll
-  for (int o = 32; o > 0; o >>= 1) L += __shfl_xor(L, o);
-  float A0 = 0.f, A1 = 0.f;
-  if (P.prev_lse) {
-    const float fp = (pl == -INFINITY) ? 0.f : __expf(pl - M);
-    const uint32_t po = *reinterpret_cast<const uint32_t*>(P.prev_out + ((size_t)g * gs + j) * RI_DIM + 2 * lane);
-    L += fp;
-    A0 = fp * __uint_as_float(po << 16);
-    A1 = fp * __uint_as_float(po & 0xffff0000u);
-  }
-#pragma unroll 8
-  for (int s = 0; s < S; ++s) {
-    const float fs = __shfl(f, s);
-    const float2 a2 = *reinterpret_cast<const float2*>(pa + (size_t)s * GS_PAD * RI_DIM);
-    A0 += a2.x * fs;
-    A1 += a2.y * fs;
-  }
-  const uint32_t o = (uint32_t)ri_f32_to_bf16(A0 / L) | ((uint32_t)ri_f32_to_bf16(A1 / L) << 16);
-  *reinterpret_cast<uint32_t*>(P.out + ((size_t)g * gs + j) * RI_DIM + 2 * lane) = o;
-  if (lane == 0) {
-    if (P.lse_out) P.lse_out[(size_t)g * gs + j] = M + __logf(L);
-    if (P.valid_lengths && j == 0) {
-      const int lenB = P.lenB_ptr ? P.lenB_ptr[(size_t)g * P.lenB_ptr_stride] : P.lenB_const;
-      P.valid_lengths[g] = P.lenA + lenB;
-    }
-  }
+__global__ __launch_bounds__(256) void combine_kernel(AttendParams P) {
+  const int g = blockIdx.x;
+  const int lenB = P.lenB_ptr ? P.lenB_ptr[(size_t)g * P.lenB_ptr_stride] : P.lenB_const;
+  combine_group<GS_PAD>(P, g, P.S_kv + P.S_es, lenB);
 }
 
 // ------------------------------------------------------------------------------------
@@ -531,34 +536,45 @@ static int launch_attend(AttendParams& P, int BG, int gs, hipStream_t s) {
   const dim3 grid(S, BG);
   P.fuse = fuse_default();
   switch (gs_pad_of(gs)) {
-    case 4: attend_kernel<4, 5><<<grid, 256, 0, s>>>(P); break;
-    case 8: attend_kernel<8, 4><<<grid, 256, 0, s>>>(P); break;
+    case 4: attend_kernel<4, 3><<<grid, 256, 0, s>>>(P); break;
+    case 8: attend_kernel<8, 2><<<grid, 256, 0, s>>>(P); break;
     default: attend_kernel<16, 2><<<grid, 256, 0, s>>>(P); break;
   }
   RI_HIP_CHECK_LAUNCH();
   if (!P.fuse) {
     switch (gs_pad_of(gs)) {
-      case 4: combine_kernel<4><<<dim3(gs, BG), 64, 0, s>>>(P); break;
-      case 8: combine_kernel<8><<<dim3(gs, BG), 64, 0, s>>>(P); break;
-      default: combine_kernel<16><<<dim3(gs, BG), 64, 0, s>>>(P); break;
+      case 4: combine_kernel<4><<<BG, 256, 0, s>>>(P); break;
+      case 8: combine_kernel<8><<<BG, 256, 0, s>>>(P); break;
+      default: combine_kernel<16><<<BG, 256, 0, s>>>(P); break;
     }
     RI_HIP_CHECK_LAUNCH();
   }
   return RI_OK;
 }
 
-static inline int chunks_ahead(int gs) { return gs <= 4 ? 5 : (gs <= 8 ? 4 : 2); }
-
-// splits so that a wave sees about one batch of rows, within [1, cap]
-static int pick_splits(int64_t rows, int BG, int cap, int gs) {
-  const int rows_per_wave = 16 * chunks_ahead(gs);
-  int64_t s = (rows + 4 * rows_per_wave - 1) / (4 * rows_per_wave);
-  // do not launch far more workgroups than the chip can hold at once
-  const int64_t max_by_chip = (4096 + BG - 1) / BG;
-  if (s > max_by_chip) s = max_by_chip;
-  if (s > cap) s = cap;
-  if (s < 1) s = 1;
-  return (int)s;
+// Split plan: about two workgroups per compute unit in total (an even load over the 256 CUs,
+// all resident at once), at least 128 rows per workgroup, the budget shared between the
+// key/value rows and the estimation rows in proportion to their counts.
+static void plan_splits(int64_t kv_rows, int64_t es_rows, int BG, int* S_kv, int* S_es) {
+  const int target_wgs = 512;
+  int per_group = target_wgs / BG;
+  if (per_group < 1) per_group = 1;
+  if (per_group > RI_MAX_SPLITS) per_group = RI_MAX_SPLITS;
+  const int64_t rows = kv_rows + es_rows;
+  int64_t by_rows = (rows + 127) / 128;
+  if (by_rows < 1) by_rows = 1;
+  if (per_group > by_rows) per_group = (int)by_rows;
+  if (es_rows <= 0) {
+    *S_kv = per_group;
+    *S_es = 0;
+    return;
+  }
+  if (per_group < 2) per_group = 2;
+  int kv = (int)((kv_rows * per_group + rows / 2) / rows);
+  if (kv < 1) kv = 1;
+  if (kv > per_group - 1) kv = per_group - 1;
+  *S_kv = kv;
+  *S_es = per_group - kv;
 }
 
 extern "C" int ri_weighted_flash_decoding(const void* q, const void* k, const void* v, const void* weight,
@@ -582,8 +598,7 @@ extern "C" int ri_weighted_flash_decoding(const void* q, const void* k, const vo
   P.lenB_const = S;
   P.weightB = (const uint16_t*)weight;
   P.weight_stride = S;
-  P.S_kv = pick_splits(S, BG, RI_MAX_SPLITS, gs);
-  P.S_es = 0;
+  plan_splits(S, 0, BG, &P.S_kv, &P.S_es);
   P.gs = gs;
   P.scale = scale;
   P.prev_out = (const uint16_t*)prev_out;
@@ -634,9 +649,7 @@ extern "C" int ri_wave_attention(const void* q, const void* steady_k, const void
   P.valid_lengths = valid_lengths;
   // the retrieved-token count is only known on the device: size the split for the row table
   // capacity scaled by the usual fill (a quarter), the estimation zone by its exact size
-  const int cap_es = es > 0 ? RI_MAX_SPLITS / 2 : 0;
-  P.S_es = es > 0 ? pick_splits(es, BG, cap_es, gs) : 0;
-  P.S_kv = pick_splits(static_len + row_src_stride / 4, BG, RI_MAX_SPLITS - P.S_es, gs);
+  plan_splits(static_len + row_src_stride / 4, es, BG, &P.S_kv, &P.S_es);
   carve_workspace(P, workspace, BG, gp);
   return launch_attend(P, BG, gs, (hipStream_t)stream);
 }
