@@ -54,7 +54,8 @@ __global__ __launch_bounds__(256) void score_kernel(
                                                        acc[t], 0, 0, 0);
   }
 
-  // scale, store, and the partial row max over this lane's valid centroids
+  // scale, and the partial row max over this lane's valid centroids.  The logits are stored at
+  // the very end: a barrier waits for outstanding stores too, and two barriers follow.
   float lmax = -INFINITY;
 #pragma unroll
   for (int t = 0; t < 4; ++t) {
@@ -63,17 +64,6 @@ __global__ __launch_bounds__(256) void score_kernel(
     for (int i = 0; i < 4; ++i) {
       acc[t][i] *= scale;
       if (cbase + i < nc) lmax = fmaxf(lmax, acc[t][i]);
-    }
-    if (r < gs && cbase < nc) {  // nc % 4 == 0, so the four columns are valid together
-      const size_t o = ((size_t)g * gs + r) * nc + cbase;
-      if (logits)
-        *reinterpret_cast<float4*>(logits + o) = make_float4(acc[t][0], acc[t][1], acc[t][2], acc[t][3]);
-      if (logits_bf16) {
-        uint2 pk;
-        pk.x = (uint32_t)ri_f32_to_bf16(acc[t][0]) | ((uint32_t)ri_f32_to_bf16(acc[t][1]) << 16);
-        pk.y = (uint32_t)ri_f32_to_bf16(acc[t][2]) | ((uint32_t)ri_f32_to_bf16(acc[t][3]) << 16);
-        *reinterpret_cast<uint2*>(logits_bf16 + o) = pk;
-      }
     }
   }
 
@@ -103,6 +93,21 @@ __global__ __launch_bounds__(256) void score_kernel(
     const size_t o = ((size_t)g * ntiles + tile) * gs + j;
     tile_max[o] = m;
     tile_sum[o] = s;
+  }
+#pragma unroll
+  for (int t = 0; t < 4; ++t) {
+    const int cbase = c0 + t * 16 + 4 * h;
+    if (r < gs && cbase < nc) {  // nc % 4 == 0, so the four columns are valid together
+      const size_t o = ((size_t)g * gs + r) * nc + cbase;
+      if (logits)
+        *reinterpret_cast<float4*>(logits + o) = make_float4(acc[t][0], acc[t][1], acc[t][2], acc[t][3]);
+      if (logits_bf16) {
+        uint2 pk;
+        pk.x = (uint32_t)ri_f32_to_bf16(acc[t][0]) | ((uint32_t)ri_f32_to_bf16(acc[t][1]) << 16);
+        pk.y = (uint32_t)ri_f32_to_bf16(acc[t][2]) | ((uint32_t)ri_f32_to_bf16(acc[t][3]) << 16);
+        *reinterpret_cast<uint2*>(logits_bf16 + o) = pk;
+      }
+    }
   }
 }
 

@@ -24,7 +24,7 @@ __device__ __forceinline__ void hist_add(uint32_t* hist, uint32_t bin, bool acti
   const uint64_t act = __ballot(active);
   if (act == 0) return;
   const int lead = __ffsll((long long)act) - 1;
-  const uint32_t first = __shfl(bin, lead);
+  const uint32_t first = (uint32_t)__builtin_amdgcn_readlane((int)bin, lead);
   const uint64_t same = __ballot(active && bin == first);
   if (same == act) {
     if ((int)(threadIdx.x & 63) == lead) atomicAdd(&hist[first], (uint32_t)__popcll(act));
@@ -152,16 +152,17 @@ __device__ __forceinline__ uint32_t sel_bin(uint32_t key) {
 
 // ------------------------------------------------------------------------------------
 // select_kernel: one 1024-thread workgroup per group.
-// dynamic LDS: keys (2 B) + cluster sizes (2 B, clamped) per cluster.
-// Thread t owns the contiguous id range [t*E, t*E+E): ties are ranked by ascending id with
-// plain prefix sums.
+// dynamic LDS: the group's cluster sizes (4 B each) when they fit.
+// Thread t owns the contiguous id range [t*E, t*E+E) and keeps those keys in registers: ties
+// are ranked by ascending id with plain prefix sums.
 // ------------------------------------------------------------------------------------
 __global__ __launch_bounds__(SEL_THREADS) void select_kernel(
     const uint16_t* __restrict__ keys, const int32_t* __restrict__ cluster_size,
     const int32_t* __restrict__ cluster_start, int64_t* __restrict__ cI, int32_t* __restrict__ ret_ids,
     int32_t* __restrict__ est_ids, int32_t* __restrict__ ret_tok_off, int32_t* __restrict__ row_src,
-    int row_src_stride, int32_t* __restrict__ meta, int nc, int np, int es, int page, int max_pages) {
-  extern __shared__ uint16_t sh_key[];
+    int row_src_stride, int32_t* __restrict__ meta, int nc, int np, int es, int page, int max_pages,
+    int sizes_in_lds) {
+  extern __shared__ int32_t sh_size[];  // nc cluster sizes when sizes_in_lds
   __shared__ uint32_t hist[SEL_BINS];
   __shared__ uint32_t sh_scan[2][3 * SEL_WAVES];  // two buffers, used alternately
   __shared__ uint32_t sh_sel[4];  // bin of T1, entries above it, bin of T2, entries above it
@@ -173,30 +174,38 @@ __global__ __launch_bounds__(SEL_THREADS) void select_kernel(
   const int tid = threadIdx.x;
   const int k2 = np + es;
 
-  // ---- keys into LDS, histogram of all keys ----
-  const int E = (((nc + SEL_THREADS - 1) / SEL_THREADS) + 7) & ~7;  // multiple of 8 (nc % 8 == 0)
+  // ---- loads: this thread's keys (registers), all cluster sizes (LDS) ----
+  // thread t owns the contiguous id range [t*E, t*E+E), E a multiple of 8 (nc % 8 == 0), E <= 64
+  const int E = (((nc + SEL_THREADS - 1) / SEL_THREADS) + 7) & ~7;
   const int cbeg = min(tid * E, nc);
   const int cend = min(cbeg + E, nc);
-  uint4 kreg[8];  // E <= 64
+  uint4 kreg[8];
 #pragma unroll
   for (int i = 0; i < 8; ++i)
-    if (cbeg + 8 * i < cend) kreg[i] = *reinterpret_cast<const uint4*>(keys + (size_t)g * nc + cbeg + 8 * i);
+    kreg[i] = (cbeg + 8 * i < cend) ? *reinterpret_cast<const uint4*>(keys + (size_t)g * nc + cbeg + 8 * i)
+                                     : ri_zero16();
+  if (sizes_in_lds && cluster_size)
+    for (int c = tid * 4; c < nc; c += SEL_THREADS * 4)
+      *reinterpret_cast<int4*>(&sh_size[c]) = *reinterpret_cast<const int4*>(cluster_size + (size_t)g * nc + c);
 #pragma unroll
   for (int i = 0; i < SEL_BPT; ++i) hist[tid * SEL_BPT + i] = 0u;
   if (tid == 0) { sh_pages = 0; sh_tret = 0; }
   __syncthreads();
+  // calls f(id, key) for every owned key in ascending id order
+  auto for_each_key = [&](auto&& f) {
 #pragma unroll
-  for (int i = 0; i < 8; ++i) {
-    if (cbeg + 8 * i < cend) {
-      *reinterpret_cast<uint4*>(&sh_key[cbeg + 8 * i]) = kreg[i];
-      const uint32_t w[4] = {kreg[i].x, kreg[i].y, kreg[i].z, kreg[i].w};
+    for (int i = 0; i < 8; ++i) {
+      if (cbeg + 8 * i < cend) {
+        const uint32_t w[4] = {kreg[i].x, kreg[i].y, kreg[i].z, kreg[i].w};
 #pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        hist_add(hist, sel_bin(w[q] & 0xffffu), true);
-        hist_add(hist, sel_bin(w[q] >> 16), true);
+        for (int q = 0; q < 4; ++q) {
+          f(cbeg + 8 * i + 2 * q, w[q] & 0xffffu);
+          f(cbeg + 8 * i + 2 * q + 1, w[q] >> 16);
+        }
       }
     }
-  }
+  };
+  for_each_key([&](int, uint32_t key) { hist_add(hist, sel_bin(key), true); });
   __syncthreads();
 
   // ---- rank thresholds: T1 = key of descending rank np-1, T2 = key of rank k2-1 ----
@@ -225,12 +234,12 @@ __global__ __launch_bounds__(SEL_THREADS) void select_kernel(
   // Tied keys are taken in ascending id order: tie rank r at T1 belongs to the retrieval zone
   // while g1 + r < np, then to the estimation zone while g1 + r < k2; at T2 while g2 + r < k2.
   uint32_t n1 = 0, n2 = 0, nmid = 0;
-  for (int c = cbeg; c < cend; ++c) {
-    const uint32_t b = sel_bin(sh_key[c]);
+  for_each_key([&](int, uint32_t key) {
+    const uint32_t b = sel_bin(key);
     n1 += (b == B1);
     n2 += (b == B2 && B2 != B1);
     nmid += (b < B1 && b > B2);
-  }
+  });
   uint32_t cnt3[3] = {n1, n2, nmid}, pre3[3], tot3[3];
   block_excl_scan<3>(cnt3, pre3, tot3, sh_scan[1]);
   uint32_t r1 = pre3[0], r2 = pre3[1];
@@ -238,9 +247,12 @@ __global__ __launch_bounds__(SEL_THREADS) void select_kernel(
   const uint32_t lo1 = (uint32_t)np > g1 ? (uint32_t)np - g1 : 0u;   // first tie rank of T1 in the est zone
   const uint32_t hi1r = (uint32_t)k2 > g1 ? (uint32_t)k2 - g1 : 0u;  // one past the last
   const uint32_t hi2r = (uint32_t)k2 > g2 ? (uint32_t)k2 - g2 : 0u;
-  uint32_t est_off = mid_before + (min(max(r1, lo1), hi1r) - lo1) + min(r2, hi2r);
-  for (int c = cbeg; c < cend; ++c) {
-    const uint32_t key = sh_key[c];
+  // Global stores are kept for the end of the kernel: a barrier waits for every outstanding
+  // memory operation of the wave, stores included, so a store issued here would put its round
+  // trip on the critical path of each later phase.
+  const uint32_t est_first = mid_before + (min(max(r1, lo1), hi1r) - lo1) + min(r2, hi2r);
+  uint64_t est_bits = 0;  // bit i: owned key i is in the estimation zone (E <= 64)
+  for_each_key([&](int c, uint32_t key) {
     const uint32_t b = sel_bin(key);
     bool in_ret, in_est;
     uint32_t slot;
@@ -260,12 +272,8 @@ __global__ __launch_bounds__(SEL_THREADS) void select_kernel(
       slot = in_ret ? atomicAdd(&hist[b], 1u) : 0u;  // hist[b] = keys above b: ranks of b start there
     }
     if (in_ret) sh_ret[slot] = (key << 16) | (0xffffu - (uint32_t)c);
-    if (in_est) {
-      est_ids[(size_t)g * es + est_off] = c;
-      if (cI) cI[(size_t)g * k2 + np + est_off] = c;
-      ++est_off;
-    }
-  }
+    if (in_est) est_bits |= 1ull << (c - cbeg);
+  });
   __syncthreads();
 
   // ---- rank order: sh_ret is ordered by score; order runs of equal scores by ascending id ----
@@ -285,29 +293,51 @@ __global__ __launch_bounds__(SEL_THREADS) void select_kernel(
   uint32_t sz = 0, pg = 0;
   int32_t st = 0;
   const int r = tid;
+  int my_c = -1;
   if (r < np) {
-    const int c = (int)(0xffffu - (sh_sorted[r] & 0xffffu));
-    ret_ids[(size_t)g * np + r] = c;
-    if (cI) cI[(size_t)g * k2 + r] = c;
+    my_c = (int)(0xffffu - (sh_sorted[r] & 0xffffu));
     if (cluster_size) {
-      sz = (uint32_t)cluster_size[(size_t)g * nc + c];
+      if (cluster_start) st = cluster_start[(size_t)g * nc + my_c];
+      sz = (uint32_t)(sizes_in_lds ? sh_size[my_c] : cluster_size[(size_t)g * nc + my_c]);
       pg = (sz + page - 1) / page;
-      if (cluster_start) st = cluster_start[(size_t)g * nc + c];
+    }
+  }
+  bool keep = false;
+  uint32_t tok_run = 0;
+  int nkeep = 0;
+  int32_t T_ret = 0;
+  if (cluster_size) {
+    uint32_t lay[2] = {pg, sz}, layp[2], layt[2];
+    block_excl_scan<2>(lay, layp, layt, sh_scan[0]);
+    const uint32_t pg_run = layp[0];
+    tok_run = layp[1];
+    // kept clusters form a prefix because the page prefix is monotone; tokens before a kept
+    // cluster all belong to kept clusters
+    keep = r < np && pg_run + pg <= (uint32_t)max_pages;
+    if (keep) {
+      atomicMax(&sh_pages, pg_run + pg);
+      atomicMax(&sh_tret, tok_run + sz);
+    }
+    nkeep = __syncthreads_count(keep);
+    T_ret = (int32_t)sh_tret;
+  }
+
+  // ---- all global stores ----
+  if (r < np) {
+    ret_ids[(size_t)g * np + r] = my_c;
+    if (cI) cI[(size_t)g * k2 + r] = my_c;
+  }
+  {
+    uint32_t est_off = est_first;
+    for (int i = 0; i < E; ++i) {
+      if ((est_bits >> i) & 1ull) {
+        est_ids[(size_t)g * es + est_off] = cbeg + i;
+        if (cI) cI[(size_t)g * k2 + np + est_off] = cbeg + i;
+        ++est_off;
+      }
     }
   }
   if (!cluster_size) return;
-  uint32_t lay[2] = {pg, sz}, layp[2], layt[2];
-  block_excl_scan<2>(lay, layp, layt, sh_scan[0]);
-  const uint32_t pg_run = layp[0], tok_run = layp[1];
-  // kept clusters form a prefix because the page prefix is monotone; tokens before a kept
-  // cluster all belong to kept clusters
-  const bool keep = r < np && pg_run + pg <= (uint32_t)max_pages;
-  if (keep) {
-    atomicMax(&sh_pages, pg_run + pg);
-    atomicMax(&sh_tret, tok_run + sz);
-  }
-  const int nkeep = __syncthreads_count(keep);
-  const int32_t T_ret = (int32_t)sh_tret;
   if (r <= np) ret_tok_off[(size_t)g * (np + 1) + r] = (r < nkeep) ? (int32_t)tok_run : T_ret;
   if (tid == 0) {
     meta[g * 4 + 0] = nkeep;
@@ -364,9 +394,11 @@ extern "C" int ri_score_select(const void* q, const void* centroids, const uint8
   else
     dist_kernel<16><<<dgrid, 256, 0, s>>>(logits, tmax, tsum, mask, keys, (uint16_t*)dist, gs, nc, ntiles);
   RI_HIP_CHECK_LAUNCH();
-  select_kernel<<<BG, SEL_THREADS, (size_t)nc * sizeof(uint16_t) + 64, s>>>(
+  // all cluster sizes fit in LDS next to the histogram up to 16384 clusters
+  const int sizes_in_lds = (cluster_size_i32 && nc <= 16384) ? 1 : 0;
+  select_kernel<<<BG, SEL_THREADS, sizes_in_lds ? (size_t)nc * sizeof(int32_t) : 0, s>>>(
       keys, cluster_size_i32, cluster_start, cI, ret_ids, est_ids, ret_tok_off, row_src, row_src_stride, meta, nc,
-      np, es, page, max_pages);
+      np, es, page, max_pages, sizes_in_lds);
   RI_HIP_CHECK_LAUNCH();
   return RI_OK;
 }
