@@ -22,6 +22,11 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK = 8.0e12  # bytes/s, MI355X
 
+# HBM bytes per attend_kernel launch from rocprofv3 counter runs of this script (FETCH_SIZE and
+# WRITE_SIZE, each scaled by what the counter reads for the known-size copy of --copy-probe);
+# the summaries are kept under profiles/.
+MEASURED_TRAFFIC = {"c2": int((31752.4 * 2.000 + 1201.1 * 1.000) * 1024)}
+
 CONFIGS = {
     # name: batch, kv heads, group size, clustered tokens, mixture centres, centroids, segments, outliers, layers
     "c1": dict(B=1, Hkv=8, gs=4, N=8192, K=512, nc=512, S=1, outliers=False, L=1,
@@ -146,6 +151,8 @@ def main():
     ap.add_argument("--layers", type=int, default=0, help="distinct layers (default: the config's)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-graph", action="store_true", help="time eager launches instead of HIP graph replays")
+    ap.add_argument("--copy-probe", action="store_true",
+                    help="also run 8 device copies of 256 MiB (a known-size kernel to scale rocprofv3 byte counters by)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: the wave-index path has no cross-GPU exchange (run with --gpus 1)")
@@ -157,6 +164,13 @@ def main():
     L = args.layers or cfg["L"]
     B, Hkv, gs = cfg["B"], cfg["Hkv"], cfg["gs"]
     BG = B * Hkv
+    if args.copy_probe:
+        a = torch.empty(256 << 20, dtype=torch.uint8, device=dev).fill_(1)
+        b = torch.empty_like(a)
+        for _ in range(8):
+            b.copy_(a)
+        torch.cuda.synchronize()
+        del a, b
     cache, queries, nprobe, es = build_cache(cfg, L, dev)
     static_len = cache.static_pattern_total  # 4 + 64 + the token being decoded (already counted)
 
@@ -207,18 +221,37 @@ def main():
     torch.cuda.synchronize()
     t_step = (time.perf_counter() - t0) / args.steps
 
-    # per-kernel timings with events on the launch stream, each stage alone
-    from retrievalattention_amd import kernels
-    l0 = 0
-    t_select = time_region(lambda: cache._select(queries[l0], l0, 0, True), 200)
+    # per-kernel pass: the same layer cycle launched eagerly, one event pair around each entry point's
+    # launches on the launch stream (cold caches as in the timed region: every step is another layer)
+    from retrievalattention_amd import kernels, _lib
+    stream = torch.cuda.current_stream().cuda_stream
+    n_k = min(args.steps, 256)
+    ev = [[torch.cuda.Event(enable_timing=True) for _ in range(4)] for _ in range(n_k)]
     out_tmp = torch.empty((BG, gs, 128), dtype=torch.bfloat16, device=dev)
-    t_attn = time_region(lambda: kernels.wave_attention(
-        queries[l0].view(BG, gs, 128), cache.steady_zone_keys[l0], cache.steady_zone_values[l0], static_len,
-        cache.list_keys[l0], cache.list_values[l0], cache.row_src, cache.meta, cache.est_ids[0], cache.logits,
-        cache.value_sum[l0], cache.cluster_size[l0], out_tmp, cache.valid_lengths[0], es, cache.RSQRT_DIM), 200)
-    cache._select(queries[l0], l0, 0, True)
+
+    def attend(l, slot):
+        kernels.wave_attention(
+            queries[l].view(BG, gs, 128), cache.steady_zone_keys[l], cache.steady_zone_values[l], static_len,
+            cache.list_keys[l], cache.list_values[l], cache.row_src, cache.meta, cache.est_ids[slot], cache.logits,
+            cache.value_sum[l], cache.cluster_size[l], out_tmp, cache.valid_lengths[slot], es, cache.RSQRT_DIM)
+
+    for i in range(n_k + 8):
+        l, slot = i % L, i % 2
+        e = ev[max(i - 8, 0)]
+        e[0].record()
+        cache._select(queries[l], l, slot, True)      # score_kernel + dist_kernel + select_kernel
+        e[1].record()
+        attend(l, slot)                                # attend_kernel (merge fused in)
+        e[2].record()
+        _lib.check(_lib.lib().ri_null_launch(stream), "ri_null_launch")
+        e[3].record()
+        if i % 32 == 31:
+            torch.cuda.synchronize()                   # keep the launch queue short: events stay adjacent
     torch.cuda.synchronize()
-    parts, t_ret = algorithmic_bytes(cache, cfg, nprobe, es, l0, static_len)
+    t_select = sum(e[0].elapsed_time(e[1]) for e in ev) * 1e-3 / n_k
+    t_attn = sum(e[1].elapsed_time(e[2]) for e in ev) * 1e-3 / n_k
+    t_null = sum(e[2].elapsed_time(e[3]) for e in ev) * 1e-3 / n_k
+    parts, t_ret = algorithmic_bytes(cache, cfg, nprobe, es, (n_k + 7) % L, static_len)
     total_bytes = sum(parts.values())
     score_bytes = parts["centroids"]
     attn_bytes = parts["estimation"] + parts["kv"] + parts["out"]
@@ -244,9 +277,14 @@ def main():
                                "GBps": attn_bytes / t_attn / 1e9},
         },
     }
-    dom = max(result["stages"].items(), key=lambda kv: kv[1]["us"])
-    result["roofline"] = {"bound": "hbm", "kernel": dom[0], "achieved": dom[1]["GBps"], "peak": HBM_PEAK / 1e9,
-                          "unit": "GB/s", "frac": dom[1]["GBps"] * 1e9 / HBM_PEAK, "traffic": None}
+    # dominant kernel: attend_kernel, the one launch of ri_wave_attention (longest kernel, and the one that
+    # moves the K/V bytes).  Its event time includes the dispatch of the launch; null_launch_us is what
+    # the same event pair reads around an empty kernel.
+    result["roofline"] = {"bound": "hbm", "kernel": "attend_kernel (ri_wave_attention)",
+                          "achieved": attn_bytes / t_attn / 1e9, "peak": HBM_PEAK / 1e9, "unit": "GB/s",
+                          "frac": attn_bytes / t_attn / HBM_PEAK, "traffic": MEASURED_TRAFFIC.get(args.config),
+                          "launch_us": t_attn * 1e6, "null_launch_us": t_null * 1e6,
+                          "algorithmic_bytes": attn_bytes, "launches_timed": n_k}
     if not args.no_cpu_baseline:
         t_cpu, n, ref = cpu_baseline(cache, cfg, queries, nprobe, es, static_len)
         d = (outs[0].view(BG, gs, 128).cpu().float() - ref.float()).abs()

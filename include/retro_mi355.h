@@ -44,6 +44,9 @@ const char* ri_status_string(int status);
 int ri_last_hip_error(void);
 /* ABI version: bumped when a signature changes. */
 int ri_abi_version(void);
+/* Launches an empty kernel on `stream`: lets a caller measure the per-dispatch overhead that
+ * event timings of back-to-back launches include.  No counterpart in the reference. */
+int ri_null_launch(ri_stream_t stream);
 
 /* ------------------------------------------------------------------------------------
  * (2) Centroid scoring

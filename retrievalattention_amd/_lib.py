@@ -15,6 +15,7 @@ SIGNATURES = {
     "ri_status_string": (C.c_char_p, [I]),
     "ri_last_hip_error": (I, []),
     "ri_abi_version": (I, []),
+    "ri_null_launch": (I, [P]),
     "ri_batch_gemm_softmax": (I, [P, P, P, P, P, P, I, I, I, I, F, F, P]),
     "ri_score_select_workspace_bytes": (SZ, [I, I, I]),
     "ri_score_select": (I, [P, P, P, P, P, P, P, P, P, P, P, P, I, P, I, I, I, I, I, I, I, F, P, SZ, P]),

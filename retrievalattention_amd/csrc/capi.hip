@@ -9,6 +9,16 @@ extern "C" int ri_last_hip_error(void) { return g_last_hip_error; }
 
 extern "C" int ri_abi_version(void) { return 1; }
 
+// An empty launch: what a dependent kernel dispatch costs on this stream, for callers that want to
+// separate dispatch overhead from kernel time in event measurements.
+__global__ void null_kernel() {}
+
+extern "C" int ri_null_launch(ri_stream_t stream) {
+  null_kernel<<<1, 64, 0, (hipStream_t)stream>>>();
+  RI_HIP_CHECK_LAUNCH();
+  return RI_OK;
+}
+
 extern "C" const char* ri_status_string(int status) {
   switch (status) {
     case RI_OK: return "ok";

@@ -34,7 +34,8 @@ def test_status_strings_and_version():
     assert l.ri_abi_version() >= 1
     assert l.ri_status_string(0) == b"ok"
     assert b"workspace" in l.ri_status_string(-3)
-    assert l.ri_score_select_workspace_bytes(32, 4, 8192) == 2 * 32 * 32 * 4 * 4
+    # two fp32 tile partials per (group, 256-centroid tile, head) and one 16-bit sort key per centroid
+    assert l.ri_score_select_workspace_bytes(32, 4, 8192) == 2 * 32 * 32 * 4 * 4 + 32 * 8192 * 2
     assert l.ri_flash_decoding_workspace_bytes(0, 4) == 0
 
 
