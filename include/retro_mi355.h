@@ -202,17 +202,23 @@ int ri_kmeans_build_lists(const int32_t* assign, int32_t* counts, int32_t* offse
 
 /* Centroid update: replaces the atomic accumulation of _triton_assign_kernel
  * (kmeans.py:48-49) plus _triton_update_kernel (kmeans.py:52-80).  For every cluster with
- * counts > 0: mean = (Σ member rows, fp32, ascending token order) / count; if normalize,
- * mean /= ||mean||₂; centroids[p,c,:] = bf16(mean).  Empty clusters keep their centroid. */
+ * counts > 0: mean = (Σ member rows) / count; if normalize, mean /= ||mean||₂;
+ * centroids[p,c,:] = bf16(mean).  Empty clusters keep their centroid.
+ * Σ is a fixed-order fp32 sum (the reference's atomics leave the order open): the list, in
+ * ascending token order, is cut into blocks of 256 rows; each block is summed one row at a time
+ * from +0, and the block sums are added in block order starting from the first block's.
+ * workspace: ri_kmeans_reduce_workspace_bytes(P, N, nc), no initialisation needed. */
+size_t ri_kmeans_reduce_workspace_bytes(int P, int N, int nc);
 int ri_kmeans_update(const void* data, const int32_t* counts, const int32_t* offsets,
                      const int32_t* members, void* centroids, int P, int N, int nc, int seg,
-                     int64_t head_rows, int normalize, ri_stream_t stream);
+                     int64_t head_rows, int normalize, void* workspace, size_t workspace_bytes,
+                     ri_stream_t stream);
 
 /* Per-cluster value sums: replaces triton_index_add (cache_hub/kmeans.py:176-221).
- * value_sum[p,c,:] = bf16(Σ member value rows, fp32, ascending token order). */
+ * value_sum[p,c,:] = bf16(Σ member value rows), Σ in the same fixed order as above. */
 int ri_kmeans_value_sum(const void* values, const int32_t* counts, const int32_t* offsets,
                         const int32_t* members, void* value_sum, int P, int N, int nc,
-                        ri_stream_t stream);
+                        void* workspace, size_t workspace_bytes, ri_stream_t stream);
 
 /* Device-side replacement of WaveBufferCPU::organize_kv (wave_buffer_cpu.cpp:545-567):
  * out[p, i, :] = in[p, members[p, i], :] — K/V rows permuted into cluster-contiguous order. */

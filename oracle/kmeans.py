@@ -1,8 +1,10 @@
 """Segmented spherical k-means of cache_hub/kmeans.py, restated on the CPU.
 
 The reference accumulates cluster sums with fp32 atomics, so its own result depends on the
-order the hardware retires them.  This restatement fixes that order to ascending token index
-(fp32, one add per token), which is what the HIP kernels implement.
+order the hardware retires them.  This restatement fixes the order the way the HIP kernels do:
+a cluster's tokens in ascending index are cut into blocks of SUM_BLOCK; each block is summed
+one fp32 add per token starting from +0, and the block sums are added in block order starting
+from the first block's.  Up to SUM_BLOCK tokens that is the plain ascending-index sum.
 """
 import numpy as np
 import torch
@@ -36,11 +38,30 @@ def assign(data: torch.Tensor, cent: torch.Tensor):
     return a.astype(np.int64), best, second
 
 
+SUM_BLOCK = 256
+
+
 def cluster_sums(rows: torch.Tensor, a: np.ndarray, nc: int):
-    """sum[c] = fp32 sum of rows with a[n] == c in ascending n; cnt[c] (kmeans.py:48-49)."""
-    s = np.zeros((nc, rows.shape[1]), dtype=np.float32)
-    np.add.at(s, a, _f32(rows))  # unbuffered, in index order: one fp32 add per token
+    """sum[c] = blocked fp32 sum (see the module header) of rows with a[n] == c; cnt[c]
+    (kmeans.py:48-49)."""
+    a = np.asarray(a, dtype=np.int64)
     cnt = np.bincount(a, minlength=nc).astype(np.int32)
+    order = np.argsort(a, kind="stable")                       # tokens grouped by cluster, ascending inside
+    start = np.concatenate([[0], np.cumsum(cnt)])[:-1]
+    pos = np.empty(a.shape[0], dtype=np.int64)
+    pos[order] = np.arange(a.shape[0]) - np.repeat(start, cnt)  # rank of a token inside its cluster
+    blk = pos // SUM_BLOCK
+    maxblk = int(blk.max()) + 1 if a.shape[0] else 1
+    item_key, item_of = np.unique(a * maxblk + blk, return_inverse=True)
+    part = np.zeros((item_key.shape[0], rows.shape[1]), dtype=np.float32)
+    np.add.at(part, item_of, _f32(rows))  # unbuffered, in index order: one fp32 add per token
+    item_c, item_b = item_key // maxblk, item_key % maxblk
+    s = np.zeros((nc, rows.shape[1]), dtype=np.float32)
+    first = item_b == 0
+    s[item_c[first]] = part[first]
+    for b in range(1, maxblk):
+        sel = item_b == b
+        s[item_c[sel]] = (s[item_c[sel]] + part[sel]).astype(np.float32)
     return s, cnt
 
 

@@ -29,8 +29,9 @@ SIGNATURES = {
     "ri_kmeans_assign": (I, [P, P, P, I, I, I, I, I64, P]),
     "ri_kmeans_workspace_bytes": (SZ, [I, I, I]),
     "ri_kmeans_build_lists": (I, [P, P, P, P, I, I, I, P, SZ, P]),
-    "ri_kmeans_update": (I, [P, P, P, P, P, I, I, I, I, I64, I, P]),
-    "ri_kmeans_value_sum": (I, [P, P, P, P, P, I, I, I, P]),
+    "ri_kmeans_reduce_workspace_bytes": (SZ, [I, I, I]),
+    "ri_kmeans_update": (I, [P, P, P, P, P, I, I, I, I, I64, I, P, SZ, P]),
+    "ri_kmeans_value_sum": (I, [P, P, P, P, P, I, I, I, P, SZ, P]),
     "ri_permute_rows": (I, [P, P, P, I, I, I64, I64, P]),
     "ri_threadpool_create": (P, [I]),
     "ri_threadpool_destroy": (None, [P]),

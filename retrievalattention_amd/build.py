@@ -20,6 +20,9 @@ ARCH = "gfx950"
 # because some of its instruction forms have been unreliable on this hardware pool.
 HIP_FLAGS = ["-O3", "-std=c++17", "-fPIC", f"--offload-arch={ARCH}", "-ffp-contract=off",
              "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-Wno-unused-command-line-argument"]
+# per-file additions: the k-means assignment reads every MFMA accumulator in its argmax
+# epilogue, so its accumulators live in ordinary VGPRs (no accumulator-register copies)
+EXTRA_HIP_FLAGS = {"kmeans.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"]}
 CPP_FLAGS = ["-O3", "-std=c++17", "-fPIC", "-pthread"]
 
 
@@ -37,7 +40,7 @@ def build(verbose=False):
     jobs = []
     for s in HIP_SOURCES:
         o = os.path.join(objdir, s + ".o")
-        jobs.append(([hipcc] + HIP_FLAGS + ["-c", os.path.join(CSRC, s), "-o", o], o))
+        jobs.append(([hipcc] + HIP_FLAGS + EXTRA_HIP_FLAGS.get(s, []) + ["-c", os.path.join(CSRC, s), "-o", o], o))
     for s in CPP_SOURCES:
         o = os.path.join(objdir, s + ".o")
         jobs.append(([hipcc] + CPP_FLAGS + ["-c", os.path.join(CSRC, s), "-o", o], o))

@@ -6,7 +6,9 @@
 
 typedef float f32x16_t __attribute__((ext_vector_type(16)));
 
-#define KM_CT 32          // centroids per LDS tile
+#define KM_CT 64          // centroid rows per LDS tile (two 32-row MFMA halves)
+#define KM_TT 4           // 32-token MFMA columns per wave: 128 tokens held in registers
+#define KM_WG_TOKENS (4 * 32 * KM_TT)
 #define KM_ROW_U16 136    // padded LDS row (272 bytes) to spread ds_read_b128 over the banks
 
 // first data row of problem p: problems are `seg` consecutive N-row slices of each head
@@ -15,68 +17,108 @@ __device__ __forceinline__ size_t km_row0(int p, int seg, int64_t head_rows, int
 }
 
 // ------------------------------------------------------------------------------------
-// assign: grid (ceil(N/256), P), 256 threads; wave = 64 tokens (two 32-token MFMA columns),
-// centroid tiles of 32 rows staged in LDS and shared by the four waves.
+// assign: grid (ceil(N/512), P), 256 threads; wave = 128 tokens (four 32-token MFMA columns,
+// four independent accumulator chains) held in registers for the whole kernel.  Centroid tiles of 64 rows go through two LDS
+// buffers shared by the four waves: the next tile's global loads are issued before the MFMAs
+// of the current one and stored to the other buffer after them, one barrier per tile.
 // MFMA 32x32x16: A = centroid rows, B = token columns; accumulator i of lane l is
-// row (i/4)*8 + (l/32)*4 + i%4, column l%32.
+// row (i/4)*8 + (l/32)*4 + i%4, column l%32.  nc is a multiple of 32; the last tile may hold
+// one half only.
 // ------------------------------------------------------------------------------------
 __global__ __launch_bounds__(256) void km_assign_kernel(const uint16_t* __restrict__ data,
                                                         const uint16_t* __restrict__ cent,
                                                         int32_t* __restrict__ assign, int N, int nc, int seg,
                                                         int64_t head_rows) {
-  __shared__ __attribute__((aligned(16))) uint16_t sh_c[KM_CT][KM_ROW_U16];
+  __shared__ __attribute__((aligned(16))) uint16_t sh_c[2][KM_CT][KM_ROW_U16];
   const int p = blockIdx.y;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int r = lane & 31, hh = lane >> 5;
-  const int t0 = blockIdx.x * 256 + wave * 64;
+  const int t0 = blockIdx.x * KM_WG_TOKENS + wave * (32 * KM_TT);
   const uint16_t* dp = data + km_row0(p, seg, head_rows, N) * RI_DIM;
   const uint16_t* cp = cent + (size_t)p * nc * RI_DIM;
+  // this thread's four 16-byte pieces of a tile: rows prow + 16 u, piece ppiece
+  const int prow = threadIdx.x >> 4, ppiece = threadIdx.x & 15;
 
-  uint4 b[2][8];
+  uint4 pf[4];
 #pragma unroll
-  for (int tt = 0; tt < 2; ++tt) {
+  for (int u = 0; u < 4; ++u) {
+    const int row = prow + 16 * u;
+    pf[u] = (row < nc) ? ri_ld16(cp + (size_t)row * RI_DIM + ppiece * 8) : ri_zero16();
+  }
+  uint4 b[KM_TT][8];
+#pragma unroll
+  for (int tt = 0; tt < KM_TT; ++tt) {
     const int tok = t0 + tt * 32 + r;
     const uint16_t* q = dp + (size_t)tok * RI_DIM + hh * 8;
 #pragma unroll
     for (int kk = 0; kk < 8; ++kk) b[tt][kk] = (tok < N) ? ri_ld16(q + kk * 16) : ri_zero16();
   }
-  float best[2] = {-INFINITY, -INFINITY};
-  int bidx[2] = {0, 0};
+#pragma unroll
+  for (int u = 0; u < 4; ++u) *reinterpret_cast<uint4*>(&sh_c[0][prow + 16 * u][ppiece * 8]) = pf[u];
+  __syncthreads();
 
-  for (int ct = 0; ct < nc; ct += KM_CT) {
-    __syncthreads();
+  float best[KM_TT];
+  int bidx[KM_TT];
 #pragma unroll
-    for (int u = 0; u < 2; ++u) {
-      const int idx = threadIdx.x + 256 * u;
-      const int row = idx >> 4, piece = idx & 15;
-      *reinterpret_cast<uint4*>(&sh_c[row][piece * 8]) = ri_ld16(cp + (size_t)(ct + row) * RI_DIM + piece * 8);
-    }
-    __syncthreads();
-    f32x16_t acc[2];
+  for (int tt = 0; tt < KM_TT; ++tt) {
+    best[tt] = -INFINITY;
+    bidx[tt] = 0;
+  }
+  int buf = 0;
+  for (int ct = 0; ct < nc; ct += KM_CT, buf ^= 1) {
+    const int nxt = ct + KM_CT;
+    if (nxt < nc) {
 #pragma unroll
-    for (int tt = 0; tt < 2; ++tt)
-#pragma unroll
-      for (int i = 0; i < 16; ++i) acc[tt][i] = 0.f;
-#pragma unroll
-    for (int kk = 0; kk < 8; ++kk) {
-      const uint4 a = *reinterpret_cast<const uint4*>(&sh_c[r][kk * 16 + hh * 8]);
-#pragma unroll
-      for (int tt = 0; tt < 2; ++tt)
-        acc[tt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ri_as_bf16x8(a), ri_as_bf16x8(b[tt][kk]), acc[tt], 0, 0, 0);
+      for (int u = 0; u < 4; ++u) {
+        const int row = nxt + prow + 16 * u;
+        pf[u] = (row < nc) ? ri_ld16(cp + (size_t)row * RI_DIM + ppiece * 8) : ri_zero16();
+      }
     }
 #pragma unroll
-    for (int tt = 0; tt < 2; ++tt)
+    for (int half = 0; half < 2; ++half) {
+      if (ct + half * 32 < nc) {  // uniform: only the last tile can lack its second half
+        f32x16_t acc[KM_TT];
 #pragma unroll
-      for (int i = 0; i < 16; ++i) {
-        const float v = acc[tt][i];
-        if (v > best[tt]) {
-          best[tt] = v;
-          bidx[tt] = ct + (i >> 2) * 8 + hh * 4 + (i & 3);
+        for (int tt = 0; tt < KM_TT; ++tt)
+#pragma unroll
+          for (int i = 0; i < 16; ++i) acc[tt][i] = 0.f;
+#pragma unroll
+        for (int kk = 0; kk < 8; ++kk) {
+          const uint4 a = *reinterpret_cast<const uint4*>(&sh_c[buf][half * 32 + r][kk * 16 + hh * 8]);
+#pragma unroll
+          for (int tt = 0; tt < KM_TT; ++tt)
+            acc[tt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ri_as_bf16x8(a), ri_as_bf16x8(b[tt][kk]), acc[tt], 0, 0,
+                                                              0);
+        }
+        // argmax epilogue: the lane's 16 scores are in ascending row order, so the first score
+        // equal to their maximum is the lowest row; the index search only runs when some lane
+        // of the wave improves on its best (rare once a few tiles have gone by)
+#pragma unroll
+        for (int tt = 0; tt < KM_TT; ++tt) {
+          float m = acc[tt][0];
+#pragma unroll
+          for (int i = 1; i < 16; ++i) m = fmaxf(m, acc[tt][i]);
+          const bool upd = m > best[tt];
+          if (__builtin_amdgcn_ballot_w64(upd) != 0ull) {
+            int sel = 15;
+#pragma unroll
+            for (int i = 14; i >= 0; --i) sel = (acc[tt][i] == m) ? i : sel;
+            if (upd) {
+              best[tt] = m;
+              bidx[tt] = ct + half * 32 + (sel >> 2) * 8 + hh * 4 + (sel & 3);
+            }
+          }
         }
       }
+    }
+    if (nxt < nc) {
+#pragma unroll
+      for (int u = 0; u < 4; ++u) *reinterpret_cast<uint4*>(&sh_c[buf ^ 1][prow + 16 * u][ppiece * 8]) = pf[u];
+    }
+    __syncthreads();
   }
 #pragma unroll
-  for (int tt = 0; tt < 2; ++tt) {
+  for (int tt = 0; tt < KM_TT; ++tt) {
     const float ob = __shfl_xor(best[tt], 32);
     const int oi = __shfl_xor(bidx[tt], 32);
     if (ob > best[tt] || (ob == best[tt] && oi < bidx[tt])) {
@@ -230,35 +272,39 @@ __global__ __launch_bounds__(1024) void km_sort_big_kernel(const int32_t* __rest
 }
 
 // ------------------------------------------------------------------------------------
-// list-ordered reductions: one wave per cluster, lane l owns dims 2l and 2l+1
+// list-ordered reductions.  A list is summed in blocks of KM_BLK rows: inside a block one fp32
+// add per row in list order starting from +0, then the block sums are added in block order
+// starting from block 0's.  One wave per block, lane l owns dims 2l and 2l+1.  Lists of at
+// most KM_BLK rows (nearly all of them) finish in the first kernel; longer lists are split into
+// block items that run in parallel and are folded by a third kernel, so that a few huge
+// clusters (the first Lloyd iterations produce them) do not serialise the pass.
 // ------------------------------------------------------------------------------------
-template <bool MEAN>
-__global__ __launch_bounds__(256) void km_reduce_kernel(const uint16_t* __restrict__ rows,
-                                                        const int32_t* __restrict__ counts,
-                                                        const int32_t* __restrict__ offsets,
-                                                        const int32_t* __restrict__ members,
-                                                        uint16_t* __restrict__ out, int N, int nc, int seg,
-                                                        int64_t head_rows, int normalize) {
-  const int p = blockIdx.y;
-  const int c = blockIdx.x * 4 + (threadIdx.x >> 6);
-  const int lane = threadIdx.x & 63;
-  if (c >= nc) return;
-  const int s = counts[(size_t)p * nc + c];
-  uint32_t* op = reinterpret_cast<uint32_t*>(out + ((size_t)p * nc + c) * RI_DIM) + lane;
-  if (s == 0) {
-    if (!MEAN) *op = 0u;  // empty cluster: zero value sum; the centroid is left untouched
-    return;
+#define KM_BLK 256
+
+__device__ __forceinline__ void km_sum_rows(const uint32_t* __restrict__ rp, const int32_t* __restrict__ mem, int k0,
+                                            int k1, float& s0, float& s1) {
+  int k = k0;
+  for (; k + 8 <= k1; k += 8) {
+    uint32_t v[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) v[j] = rp[(size_t)mem[k + j] * (RI_DIM / 2)];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      s0 += __uint_as_float(v[j] << 16);
+      s1 += __uint_as_float(v[j] & 0xffff0000u);
+    }
   }
-  const int32_t* mem = members + (size_t)p * N + offsets[(size_t)p * (nc + 1) + c];
-  const uint32_t* rp = reinterpret_cast<const uint32_t*>(rows + km_row0(p, seg, head_rows, N) * RI_DIM) + lane;
-  float s0 = 0.f, s1 = 0.f;
-  for (int k = 0; k < s; ++k) {
+  for (; k < k1; ++k) {
     const uint32_t v = rp[(size_t)mem[k] * (RI_DIM / 2)];
     s0 += __uint_as_float(v << 16);
     s1 += __uint_as_float(v & 0xffff0000u);
   }
+}
+
+template <bool MEAN>
+__device__ __forceinline__ void km_finish(float s0, float s1, int count, int normalize, uint32_t* op) {
   if (MEAN) {
-    const float cnt = (float)s;
+    const float cnt = (float)count;
     s0 = s0 / cnt;
     s1 = s1 / cnt;
     if (normalize) {
@@ -271,6 +317,112 @@ __global__ __launch_bounds__(256) void km_reduce_kernel(const uint16_t* __restri
     }
   }
   *op = (uint32_t)ri_f32_to_bf16(s0) | ((uint32_t)ri_f32_to_bf16(s1) << 16);
+}
+
+// item slots of one problem: every list longer than KM_BLK takes ceil(s / KM_BLK) <= 2 s / KM_BLK
+static inline int km_item_cap(int N) { return 2 * (N / KM_BLK) + 2; }
+
+template <bool MEAN>
+__global__ __launch_bounds__(256) void km_reduce_kernel(const uint16_t* __restrict__ rows,
+                                                        const int32_t* __restrict__ counts,
+                                                        const int32_t* __restrict__ offsets,
+                                                        const int32_t* __restrict__ members,
+                                                        uint16_t* __restrict__ out, int32_t* __restrict__ item_count,
+                                                        int32_t* __restrict__ item_base,
+                                                        int32_t* __restrict__ items, int cap, int N, int nc, int seg,
+                                                        int64_t head_rows, int normalize) {
+  const int p = blockIdx.y;
+  const int c = blockIdx.x * 4 + (threadIdx.x >> 6);
+  const int lane = threadIdx.x & 63;
+  if (c >= nc) return;
+  const int s = counts[(size_t)p * nc + c];
+  uint32_t* op = reinterpret_cast<uint32_t*>(out + ((size_t)p * nc + c) * RI_DIM) + lane;
+  if (s == 0) {
+    if (!MEAN) *op = 0u;  // empty cluster: zero value sum; the centroid is left untouched
+    return;
+  }
+  if (s > KM_BLK) {  // queue the blocks of a long list
+    const int nb = (s + KM_BLK - 1) / KM_BLK;
+    int base = 0;
+    if (lane == 0) {
+      base = atomicAdd(&item_count[p], nb);
+      item_base[(size_t)p * nc + c] = base;
+    }
+    base = __shfl(base, 0);
+    for (int j = lane; j < nb; j += 64) items[(size_t)p * cap + base + j] = c;
+    return;
+  }
+  const int32_t* mem = members + (size_t)p * N + offsets[(size_t)p * (nc + 1) + c];
+  const uint32_t* rp = reinterpret_cast<const uint32_t*>(rows + km_row0(p, seg, head_rows, N) * RI_DIM) + lane;
+  float s0 = 0.f, s1 = 0.f;
+  km_sum_rows(rp, mem, 0, s, s0, s1);
+  km_finish<MEAN>(s0, s1, s, normalize, op);
+}
+
+// one wave per queued block: its fp32 sum goes to partial[item]
+__global__ __launch_bounds__(256) void km_reduce_blocks_kernel(const uint16_t* __restrict__ rows,
+                                                               const int32_t* __restrict__ counts,
+                                                               const int32_t* __restrict__ offsets,
+                                                               const int32_t* __restrict__ members,
+                                                               const int32_t* __restrict__ item_count,
+                                                               const int32_t* __restrict__ item_base,
+                                                               const int32_t* __restrict__ items,
+                                                               float2* __restrict__ partial, int cap, int N, int nc,
+                                                               int seg, int64_t head_rows) {
+  const int p = blockIdx.y;
+  const int lane = threadIdx.x & 63;
+  const int n_items = item_count[p];
+  for (int it = blockIdx.x * 4 + (threadIdx.x >> 6); it < n_items; it += gridDim.x * 4) {
+    const int c = items[(size_t)p * cap + it];
+    const int j = it - item_base[(size_t)p * nc + c];
+    const int s = counts[(size_t)p * nc + c];
+    const int k0 = j * KM_BLK, k1 = min(s, k0 + KM_BLK);
+    const int32_t* mem = members + (size_t)p * N + offsets[(size_t)p * (nc + 1) + c];
+    const uint32_t* rp = reinterpret_cast<const uint32_t*>(rows + km_row0(p, seg, head_rows, N) * RI_DIM) + lane;
+    float s0 = 0.f, s1 = 0.f;
+    km_sum_rows(rp, mem, k0, k1, s0, s1);
+    partial[((size_t)p * cap + it) * 64 + lane] = make_float2(s0, s1);
+  }
+}
+
+// the wave of a long list's first item folds the block sums in block order and finishes
+template <bool MEAN>
+__global__ __launch_bounds__(256) void km_reduce_fold_kernel(const int32_t* __restrict__ counts,
+                                                             const int32_t* __restrict__ item_count,
+                                                             const int32_t* __restrict__ item_base,
+                                                             const int32_t* __restrict__ items,
+                                                             const float2* __restrict__ partial,
+                                                             uint16_t* __restrict__ out, int cap, int nc,
+                                                             int normalize) {
+  const int p = blockIdx.y;
+  const int lane = threadIdx.x & 63;
+  const int n_items = item_count[p];
+  for (int it = blockIdx.x * 4 + (threadIdx.x >> 6); it < n_items; it += gridDim.x * 4) {
+    const int c = items[(size_t)p * cap + it];
+    if (it != item_base[(size_t)p * nc + c]) continue;
+    const int s = counts[(size_t)p * nc + c];
+    const int nb = (s + KM_BLK - 1) / KM_BLK;
+    const float2* pp = partial + ((size_t)p * cap + it) * 64 + lane;
+    float2 t = pp[0];
+    int j = 1;
+    for (; j + 4 <= nb; j += 4) {
+      float2 v[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) v[u] = pp[(size_t)(j + u) * 64];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        t.x += v[u].x;
+        t.y += v[u].y;
+      }
+    }
+    for (; j < nb; ++j) {
+      const float2 v = pp[(size_t)j * 64];
+      t.x += v.x;
+      t.y += v.y;
+    }
+    uint32_t* op = reinterpret_cast<uint32_t*>(out + ((size_t)p * nc + c) * RI_DIM) + lane;
+    km_finish<MEAN>(t.x, t.y, s, normalize, op);
+  }
 }
 
 // out[p, i, :] = in[p, members[p, i], :]; 16 lanes per row
@@ -299,8 +451,8 @@ extern "C" int ri_kmeans_assign(const void* data, const void* centroids, int32_t
   if (!data || !centroids || !assign) return RI_ERR_ARG;
   int rc = km_check(P, N, nc);
   if (rc) return rc;
-  if (nc % KM_CT != 0 || seg <= 0 || P % seg != 0) return RI_ERR_ARG;
-  km_assign_kernel<<<dim3((N + 255) / 256, P), 256, 0, (hipStream_t)stream>>>(
+  if (nc % 32 != 0 || seg <= 0 || P % seg != 0) return RI_ERR_ARG;
+  km_assign_kernel<<<dim3((N + KM_WG_TOKENS - 1) / KM_WG_TOKENS, P), 256, 0, (hipStream_t)stream>>>(
       (const uint16_t*)data, (const uint16_t*)centroids, assign, N, nc, seg, head_rows);
   RI_HIP_CHECK_LAUNCH();
   return RI_OK;
@@ -341,29 +493,61 @@ extern "C" int ri_kmeans_build_lists(const int32_t* assign, int32_t* counts, int
   return RI_OK;
 }
 
-extern "C" int ri_kmeans_update(const void* data, const int32_t* counts, const int32_t* offsets,
-                                const int32_t* members, void* centroids, int P, int N, int nc, int seg,
-                                int64_t head_rows, int normalize, ri_stream_t stream) {
-  if (!data || !counts || !offsets || !members || !centroids) return RI_ERR_ARG;
-  int rc = km_check(P, N, nc);
-  if (rc) return rc;
-  if (seg <= 0 || P % seg != 0) return RI_ERR_ARG;
-  km_reduce_kernel<true><<<dim3((nc + 3) / 4, P), 256, 0, (hipStream_t)stream>>>(
-      (const uint16_t*)data, counts, offsets, members, (uint16_t*)centroids, N, nc, seg, head_rows, normalize);
+extern "C" size_t ri_kmeans_reduce_workspace_bytes(int P, int N, int nc) {
+  if (P <= 0 || N <= 0 || nc <= 0) return 0;
+  const size_t cap = (size_t)km_item_cap(N);
+  // item_count [P] + item_base [P, nc] + items [P, cap] + partial [P, cap, 128] fp32
+  return ((size_t)P + (size_t)P * nc + (size_t)P * cap) * sizeof(int32_t) + (size_t)P * cap * RI_DIM * sizeof(float) +
+         256;
+}
+
+template <bool MEAN>
+static int km_reduce(const void* rows, const int32_t* counts, const int32_t* offsets, const int32_t* members,
+                     void* out, int P, int N, int nc, int seg, int64_t head_rows, int normalize, void* workspace,
+                     size_t workspace_bytes, hipStream_t s) {
+  if (workspace_bytes < ri_kmeans_reduce_workspace_bytes(P, N, nc)) return RI_ERR_WORKSPACE;
+  const int cap = km_item_cap(N);
+  int32_t* item_count = (int32_t*)workspace;
+  int32_t* item_base = item_count + P;
+  int32_t* items = item_base + (size_t)P * nc;
+  uintptr_t pa = (uintptr_t)(items + (size_t)P * cap);
+  float2* partial = (float2*)((pa + 255) & ~(uintptr_t)255);
+  km_zero_kernel<<<1, 256, 0, s>>>(item_count, (size_t)P);
+  RI_HIP_CHECK_LAUNCH();
+  km_reduce_kernel<MEAN><<<dim3((nc + 3) / 4, P), 256, 0, s>>>((const uint16_t*)rows, counts, offsets, members,
+                                                               (uint16_t*)out, item_count, item_base, items, cap, N,
+                                                               nc, seg, head_rows, normalize);
+  RI_HIP_CHECK_LAUNCH();
+  const int gx = min((cap + 3) / 4, 1024);
+  km_reduce_blocks_kernel<<<dim3(gx, P), 256, 0, s>>>((const uint16_t*)rows, counts, offsets, members, item_count,
+                                                      item_base, items, partial, cap, N, nc, seg, head_rows);
+  RI_HIP_CHECK_LAUNCH();
+  km_reduce_fold_kernel<MEAN><<<dim3(gx, P), 256, 0, s>>>(counts, item_count, item_base, items, partial,
+                                                          (uint16_t*)out, cap, nc, normalize);
   RI_HIP_CHECK_LAUNCH();
   return RI_OK;
 }
 
-extern "C" int ri_kmeans_value_sum(const void* values, const int32_t* counts, const int32_t* offsets,
-                                   const int32_t* members, void* value_sum, int P, int N, int nc,
-                                   ri_stream_t stream) {
-  if (!values || !counts || !offsets || !members || !value_sum) return RI_ERR_ARG;
+extern "C" int ri_kmeans_update(const void* data, const int32_t* counts, const int32_t* offsets,
+                                const int32_t* members, void* centroids, int P, int N, int nc, int seg,
+                                int64_t head_rows, int normalize, void* workspace, size_t workspace_bytes,
+                                ri_stream_t stream) {
+  if (!data || !counts || !offsets || !members || !centroids || !workspace) return RI_ERR_ARG;
   int rc = km_check(P, N, nc);
   if (rc) return rc;
-  km_reduce_kernel<false><<<dim3((nc + 3) / 4, P), 256, 0, (hipStream_t)stream>>>(
-      (const uint16_t*)values, counts, offsets, members, (uint16_t*)value_sum, N, nc, 1, (int64_t)N, 0);
-  RI_HIP_CHECK_LAUNCH();
-  return RI_OK;
+  if (seg <= 0 || P % seg != 0) return RI_ERR_ARG;
+  return km_reduce<true>(data, counts, offsets, members, centroids, P, N, nc, seg, head_rows, normalize, workspace,
+                         workspace_bytes, (hipStream_t)stream);
+}
+
+extern "C" int ri_kmeans_value_sum(const void* values, const int32_t* counts, const int32_t* offsets,
+                                   const int32_t* members, void* value_sum, int P, int N, int nc, void* workspace,
+                                   size_t workspace_bytes, ri_stream_t stream) {
+  if (!values || !counts || !offsets || !members || !value_sum || !workspace) return RI_ERR_ARG;
+  int rc = km_check(P, N, nc);
+  if (rc) return rc;
+  return km_reduce<false>(values, counts, offsets, members, value_sum, P, N, nc, 1, (int64_t)N, 0, workspace,
+                          workspace_bytes, (hipStream_t)stream);
 }
 
 extern "C" int ri_permute_rows(const void* in, const int32_t* members, void* out, int P, int N,

@@ -69,12 +69,16 @@ int ri_launch_score(const void* q, const void* centroids, float* logits, float* 
 // tiles, xor-butterfly reductions (fixed order, so the result is reproducible).
 __device__ __forceinline__ void ri_wave_reduce_partials(const float* pm, const float* ps, int ntiles, int gs,
                                                         int j, int lane, float* m_out, float* invz_out) {
-  float m = -INFINITY;
-  for (int t = lane; t < ntiles; t += 64) m = fmaxf(m, pm[(size_t)t * gs + j]);
+  // the first 64 tiles' partials are loaded together, ahead of the reductions
+  const bool has0 = lane < ntiles;
+  const float pm0 = has0 ? pm[(size_t)lane * gs + j] : -INFINITY;
+  const float ps0 = has0 ? ps[(size_t)lane * gs + j] : 0.f;
+  float m = pm0;
+  for (int t = lane + 64; t < ntiles; t += 64) m = fmaxf(m, pm[(size_t)t * gs + j]);
 #pragma unroll
   for (int o = 32; o > 0; o >>= 1) m = fmaxf(m, __shfl_xor(m, o));
-  float z = 0.f;
-  for (int t = lane; t < ntiles; t += 64) z += ps[(size_t)t * gs + j] * __expf(pm[(size_t)t * gs + j] - m);
+  float z = has0 ? ps0 * __expf(pm0 - m) : 0.f;
+  for (int t = lane + 64; t < ntiles; t += 64) z += ps[(size_t)t * gs + j] * __expf(pm[(size_t)t * gs + j] - m);
 #pragma unroll
   for (int o = 32; o > 0; o >>= 1) z += __shfl_xor(z, o);
   *m_out = m;

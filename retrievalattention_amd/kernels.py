@@ -272,13 +272,15 @@ def kmeans_build_lists(assign, counts, offsets, members, P, N, nc):
 
 
 def kmeans_update(data, counts, offsets, members, centroids, P, N, nc, seg, head_rows, normalize):
+    ws = _workspace(lib().ri_kmeans_reduce_workspace_bytes(P, N, nc), data.device, "kmeans_reduce")
     check(lib().ri_kmeans_update(_p(data), _p(counts), _p(offsets), _p(members), _p(centroids), P, N, nc, seg,
-                                 head_rows, int(bool(normalize)), _stream()), "kmeans_update")
+                                 head_rows, int(bool(normalize)), _p(ws), ws.numel(), _stream()), "kmeans_update")
 
 
 def kmeans_value_sum(values, counts, offsets, members, value_sum, P, N, nc):
+    ws = _workspace(lib().ri_kmeans_reduce_workspace_bytes(P, N, nc), values.device, "kmeans_reduce")
     check(lib().ri_kmeans_value_sum(_p(values), _p(counts), _p(offsets), _p(members), _p(value_sum), P, N, nc,
-                                    _stream()), "kmeans_value_sum")
+                                    _p(ws), ws.numel(), _stream()), "kmeans_value_sum")
 
 
 def permute_rows(src, members, dst, P, N, in_stride_rows, out_stride_rows):

@@ -117,6 +117,41 @@ def test_medium_clusters_sorted(dev):
         assert np.array_equal(members[p].cpu().numpy(), order.astype(np.int32))
 
 
+def test_long_lists_blocked_sums(dev):
+    """Lists of 1 to several thousand random rows: update and value sums equal the oracle's
+    blocked fixed-order sums bit for bit (lists over 256 rows take the block-item path, several
+    of them per problem, next to short lists and empty clusters)."""
+    from retrievalattention_amd import kernels
+    P, N, nc = 3, 20011, 96
+    g = torch.Generator().manual_seed(16)
+    keys = torch.randn(P, N, 128, generator=g).to(torch.bfloat16)
+    vals = torch.randn(P, N, 128, generator=g).to(torch.bfloat16)
+    assign = torch.randint(0, 5, (P, N), generator=g, dtype=torch.int32)       # five lists of ~4000
+    small = torch.randint(8, 90, (P, N), generator=g, dtype=torch.int32)       # the rest: ~100 each, 90..95 empty
+    pick = torch.rand(P, N, generator=g) < 0.4
+    assign[pick] = small[pick]
+    assign[1, :700] = 7                                                        # 700+: three blocks, last one ragged
+    assign[2, 5] = 95                                                          # a single-row list
+    cent = torch.randn(P, nc, 128, generator=g).to(torch.bfloat16)
+    ad, kd, vd = assign.to(dev), keys.to(dev), vals.to(dev)
+    counts = torch.empty(P, nc, dtype=torch.int32, device=dev)
+    offsets = torch.empty(P, nc + 1, dtype=torch.int32, device=dev)
+    members = torch.empty(P, N, dtype=torch.int32, device=dev)
+    kernels.kmeans_build_lists(ad, counts, offsets, members, P, N, nc)
+    for normalize in (True, False):
+        cd = cent.to(dev).clone()
+        kernels.kmeans_update(kd, counts, offsets, members, cd, P, N, nc, 1, N, normalize)
+        vs = torch.full((P, nc, 128), 7.0, dtype=torch.bfloat16, device=dev)
+        kernels.kmeans_value_sum(vd, counts, offsets, members, vs, P, N, nc)
+        torch.cuda.synchronize()
+        for p in range(P):
+            a = assign[p].numpy().astype(np.int64)
+            s, cnt = okm.cluster_sums(keys[p], a, nc)
+            assert np.array_equal(counts[p].cpu().numpy(), cnt)
+            assert torch.equal(cd[p].cpu(), okm.update(cent[p], s, cnt, normalize))
+            assert torch.equal(vs[p].cpu(), okm.value_sum(vals[p], a, nc))
+
+
 @pytest.mark.parametrize("G,N,nc,S,seed", [(2, 4096, 256, 4, 0), (1, 8192, 512, 1, 1), (2, 3001, 192, 3, 2)])
 def test_segment_k_means_teacher_forced(dev, G, N, nc, S, seed):
     """Whole driver against the oracle, iteration by iteration: every step is checked on the

@@ -183,6 +183,31 @@ def test_update_mean_normalise_and_empty_clusters():
     assert np.allclose(no[:12].float().numpy(), mean / np.linalg.norm(mean, axis=1, keepdims=True), atol=1e-2)
 
 
+def test_cluster_sums_blocked_order_by_brute_force():
+    """The fixed summation order, restated as plain loops: blocks of 256 tokens in ascending
+    index, one fp32 add per token from +0 inside a block, block sums added in block order."""
+    g = torch.Generator().manual_seed(17)
+    data = _r((1500, 128), g)
+    a = np.random.default_rng(1).integers(0, 3, 1500)
+    a[700:] = np.minimum(a[700:], 1)                        # cluster 1 grows past three blocks
+    a[:40] = 5                                              # a short list; clusters 3, 4 stay empty
+    s, cnt = okm.cluster_sums(data, a, 6)
+    x = data.float().numpy()
+    for c in range(6):
+        ids = [n for n in range(1500) if a[n] == c]
+        assert cnt[c] == len(ids)
+        total = None
+        for b in range(0, len(ids), okm.SUM_BLOCK):
+            part = np.zeros(128, dtype=np.float32)
+            for n in ids[b:b + okm.SUM_BLOCK]:
+                part = (part + x[n]).astype(np.float32)
+            total = part if total is None else (total + part).astype(np.float32)
+        if total is None:
+            total = np.zeros(128, dtype=np.float32)
+        assert np.array_equal(s[c], total)
+    assert max(cnt) > 2 * okm.SUM_BLOCK                     # the blocked path was exercised
+
+
 def test_segment_k_means_invariants_and_remainder_tokens():
     """Each token in exactly one list; sizes add up; centroid * size = sum of keys (fp32 -> bf16);
     value_sum = sum of values; tokens past Nseg*S are only seen by the final pass."""
