@@ -44,7 +44,7 @@ def log(*a):
     print(*a, file=sys.stderr, flush=True)
 
 
-def build_cache(cfg, L, dev):
+def build_cache(cfg, L, dev, residency="device"):
     from retrievalattention_amd import synth
     from retrievalattention_amd.cache_hub import retroinfer_cache
     B, Hkv, gs, N = cfg["B"], cfg["Hkv"], cfg["gs"], cfg["N"]
@@ -57,7 +57,7 @@ def build_cache(cfg, L, dev):
         num_heads=Hkv * gs, head_dim=128, dtype=torch.bfloat16, layer_mapping={str(l): "cuda:0" for l in range(L)},
         max_new_length=new, static_pattern_start=synth.STEADY_START, static_pattern_end=synth.STEADY_END, core=8,
         n_centroids=cfg["nc"], n_segment=cfg["S"], nprobe=nprobe, max_compute_cluster_num=nprobe + es,
-        cache_unit_size=8, cache_cluster_num=3 * nprobe, num_gpus=1, model_size=0, kv_residency="device")
+        cache_unit_size=8, cache_cluster_num=3 * nprobe, num_gpus=1, model_size=0, kv_residency=residency)
     queries = []
     t0 = time.time()
     for l in range(L):
@@ -117,6 +117,35 @@ def time_region(fn, iters):
     return s.elapsed_time(e) * 1e-3 / iters
 
 
+MFMA_BF16_PEAK = 2.5e15  # FLOP/s, MI355X dense bf16
+
+
+def bench_kmeans(cfg, dev, iters=10, reps=3):
+    """Prefill clustering of one sequence (all kv heads) with the library's own driver:
+    9 segmented spherical Lloyd iterations + 1 global one + value sums + inverted lists."""
+    from retrievalattention_amd import synth, kernels
+    from retrievalattention_amd.cache_hub.kmeans import segment_k_means_csr
+    Hkv, N, nc, S = cfg["Hkv"], cfg["N"], cfg["nc"], cfg["S"]
+    ks, vs = [], []
+    for h in range(Hkv):
+        k, v, _ = synth.make_group(0, 0, h, N, cfg["K"], cfg["gs"], outliers=cfg["outliers"], n_extra=0, device=dev)
+        ks.append(k.to(torch.bfloat16)); vs.append(v.to(torch.bfloat16))
+    K, V = torch.stack(ks).contiguous(), torch.stack(vs).contiguous()
+    K = (K - K.mean(dim=1, keepdim=True)).contiguous()          # keys are centred before clustering
+    r = segment_k_means_csr(K, V, nc, iters, S)                  # warm-up
+    t = time_region(lambda: segment_k_means_csr(K, V, nc, iters, S), reps)
+    # the global assignment alone: the one launch that holds most of the FLOPs
+    assign = torch.empty((Hkv, N), dtype=torch.int32, device=dev)
+    t_as = time_region(lambda: kernels.kmeans_assign(K, r.centroids, assign, Hkv, N, nc, 1, N), reps)
+    flops = 2.0 * 128 * Hkv * N * ((iters - 1) * nc / S + nc)
+    flops_as = 2.0 * 128 * Hkv * N * nc
+    return {"ms_per_sequence": t * 1e3, "tokens": N, "kv_heads": Hkv, "centroids": nc, "segments": S,
+            "iterations": iters, "algorithmic_flops": flops, "bound": "mfma", "achieved": flops / t / 1e12,
+            "peak": MFMA_BF16_PEAK / 1e12, "unit": "TFLOP/s", "frac": flops / t / MFMA_BF16_PEAK,
+            "global_assign": {"us": t_as * 1e6, "achieved": flops_as / t_as / 1e12,
+                              "frac": flops_as / t_as / MFMA_BF16_PEAK}}
+
+
 def cpu_baseline(cache, cfg, queries, nprobe, es, static_len, max_seconds=30.0):
     """The CPU restatement (oracle/) of the same decode step, layer 0, on the host cores."""
     from oracle import pipeline
@@ -142,6 +171,46 @@ def cpu_baseline(cache, cfg, queries, nprobe, es, static_len, max_seconds=30.0):
     return times[len(times) // 2], len(times), ref
 
 
+def bench_host(args, cfg, cache, queries, L, nprobe, es, static_len):
+    """Host-resident clustered K/V: the reference's operator sequence (score+select, id copy to the
+    host, block-cache look-up on the worker pool, gather of misses over the host link and hits
+    from the device cache, attention, cache admission).  The first pass over the layers runs
+    with an empty block cache (every retrieved block is a miss); repeating the same queries then
+    hits for every block that was admitted."""
+    B = cfg["B"]
+
+    def step(l):
+        return cache._compute_staged(queries[l], l, None, static_len, l % 2, (l + 1) % 2, True, False)
+
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for l in range(L):
+        step(l)
+    torch.cuda.synchronize()
+    t_cold = (time.perf_counter() - t0) / L
+    for i in range(args.warmup):
+        step(i % L)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(args.steps):
+        step(i % L)
+    torch.cuda.synchronize()
+    t_warm = (time.perf_counter() - t0) / args.steps
+    miss = sum(int(cache.miss_num_units[l].sum()) for l in range(L))
+    hit = sum(int(cache.hit_num_units[l].sum()) for l in range(L))
+    print(json.dumps({
+        "metric": "decode tokens/s at 128K ctx (attention only, B / (L * t_layer_step)); us/layer-step and % HBM roofline alongside",
+        "value": B / (cfg["L"] * t_warm), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": t_warm * 1e3, "us_per_layer_step": t_warm * 1e6, "cold_us_per_layer_step": t_cold * 1e6,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": f"{args.config}: {cfg['desc']}; clustered K/V in pinned host memory, block cache of "
+                               f"{cache.cache_size if hasattr(cache, 'cache_size') else '?'} blocks per group, "
+                               f"nprobe {nprobe}, estimation zone {es}, {L} layers, eager launches, warm = same "
+                               f"queries repeated", "batch": B, "context_tokens": cfg["N"],
+                   "layers_for_tokens_per_s": cfg["L"], "warm_hit_blocks": hit, "warm_miss_blocks": miss},
+        "roofline": None, "cpu_baseline": None}))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -151,6 +220,10 @@ def main():
     ap.add_argument("--layers", type=int, default=0, help="distinct layers (default: the config's)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-graph", action="store_true", help="time eager launches instead of HIP graph replays")
+    ap.add_argument("--residency", default="device", choices=["device", "host"],
+                    help="host: clustered K/V in pinned host memory behind the block cache (staged operator path, "
+                         "eager launches; reports the cold first pass and the warm steady state)")
+    ap.add_argument("--no-kmeans", action="store_true", help="skip the prefill clustering measurement")
     ap.add_argument("--copy-probe", action="store_true",
                     help="also run 8 device copies of 256 MiB (a known-size kernel to scale rocprofv3 byte counters by)")
     args = ap.parse_args()
@@ -171,8 +244,10 @@ def main():
             b.copy_(a)
         torch.cuda.synchronize()
         del a, b
-    cache, queries, nprobe, es = build_cache(cfg, L, dev)
+    cache, queries, nprobe, es = build_cache(cfg, L, dev, args.residency)
     static_len = cache.static_pattern_total  # 4 + 64 + the token being decoded (already counted)
+    if args.residency == "host":
+        return bench_host(args, cfg, cache, queries, L, nprobe, es, static_len)
 
     # every layer-step is "not the last layer" for timing purposes: same static_len everywhere
     def step(l):
@@ -285,6 +360,8 @@ def main():
                           "frac": attn_bytes / t_attn / HBM_PEAK, "traffic": MEASURED_TRAFFIC.get(args.config),
                           "launch_us": t_attn * 1e6, "null_launch_us": t_null * 1e6,
                           "algorithmic_bytes": attn_bytes, "launches_timed": n_k}
+    if not args.no_kmeans:
+        result["prefill_kmeans"] = bench_kmeans(cfg, dev)
     if not args.no_cpu_baseline:
         t_cpu, n, ref = cpu_baseline(cache, cfg, queries, nprobe, es, static_len)
         d = (outs[0].view(BG, gs, 128).cpu().float() - ref.float()).abs()

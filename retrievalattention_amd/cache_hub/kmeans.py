@@ -2,8 +2,9 @@
 (cache_hub/kmeans.py:224-259 of the reference), driven by the gfx950 kernels.
 
 Differences that a caller can observe, both within what the reference leaves open:
-  * cluster sums are accumulated in ascending token order (fp32) instead of by atomics, so
-    the result is reproducible run to run;
+  * cluster sums are accumulated in a fixed order (fp32: ascending token order in blocks of 256
+    tokens, block sums added in block order) instead of by atomics, so the result is
+    reproducible run to run;
   * tokens inside a cluster list are ascending (the reference's order is whatever its atomics
     produced).
 """
