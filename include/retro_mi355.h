@@ -140,6 +140,21 @@ int ri_wave_attention(const void* q, const void* steady_k, const void* steady_v,
                       int BG, int gs, int nc, int es, float scale, void* workspace,
                       size_t workspace_bytes, ri_stream_t stream);
 
+/* Attention over an execution buffer with the estimation zone fused in: replaces
+ * gather_copy_vectors → weighted_flash_decoding (estimation) and the final
+ * weighted_flash_decoding with previous_out/previous_lse
+ * (cache_hub/retroinfer_cache.py:598-617 and :666-674) when the retrieved K/V were staged by
+ * gather_copy_and_concat (host-resident cluster store).
+ *   buf_k/v [BG, buf_stride, 128]: rows [0, cache_seqlens[g]) attended, cache_seqlens [BG] int32
+ *   as written by ri_gather_copy_and_concat; max_len: upper bound of the lengths (<= buf_stride);
+ *   est_ids, logits: as written by ri_score_select for the same query; value_sum, cluster_size_bf16
+ *   as for ri_wave_attention.  Workspace: ri_wave_attention_workspace_bytes, same rules. */
+int ri_buffer_attention(const void* q, const void* buf_k, const void* buf_v, int64_t buf_stride,
+                        const int32_t* cache_seqlens, int max_len, const int32_t* est_ids,
+                        const float* logits, const void* value_sum, const void* cluster_size_bf16,
+                        void* out, int BG, int gs, int nc, int es, float scale, void* workspace,
+                        size_t workspace_bytes, ri_stream_t stream);
+
 /* ------------------------------------------------------------------------------------
  * (3) Wave-buffer copies
  * ---------------------------------------------------------------------------------- */

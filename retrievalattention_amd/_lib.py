@@ -23,6 +23,7 @@ SIGNATURES = {
     "ri_weighted_flash_decoding": (I, [P, P, P, P, P, P, P, P, P, I, I, I, I64, F, P, SZ, P]),
     "ri_wave_attention_workspace_bytes": (SZ, [I, I]),
     "ri_wave_attention": (I, [P, P, P, I64, I, P, P, I64, P, I, P, P, P, P, P, P, P, I, I, I, I, F, P, SZ, P]),
+    "ri_buffer_attention": (I, [P, P, P, I64, P, I, P, P, P, P, P, I, I, I, I, F, P, SZ, P]),
     "ri_gather_copy_vectors": (I, [P, P, P, P, P, P, P, I, I, I, I, I, I, P]),
     "ri_gather_copy_and_concat": (I, [P] * 17 + [I] * 7 + [P]),
     "ri_gather_copy_and_scatter": (I, [P] * 8 + [I] * 5 + [P]),

@@ -388,7 +388,11 @@ class retroinfer_cache(KV_Cache):
             self._search(queries, layer_idx, buf)
         if search_next:
             self._search(queries_next, layer_idx + 1, nbuf)
-        if self.es_cluster_num > 0:
+        # without next-layer estimation the logits of this layer's own query are at hand, so the
+        # estimation zone is merged inside the final attention launch; otherwise it is computed the
+        # reference's way, from gathered centroids and the true query
+        fuse_est = self.es_cluster_num > 0 and not self.use_cluster_estimation
+        if self.es_cluster_num > 0 and not fuse_est:
             kernels.gather_copy_vectors(
                 self.centroids[layer_idx], self.es_centroids, self.value_sum[layer_idx], self.es_value_sum,
                 self.cluster_size[layer_idx], self.es_cluster_size, self.cI[buf], BG, self.n_centroids,
@@ -411,9 +415,16 @@ class retroinfer_cache(KV_Cache):
         if not search_here:
             # this layer's buffer was assembled on the copy stream during the previous layer
             torch.cuda.current_stream().wait_stream(self.copystream)
-        attn = kernels.weighted_flash_decoding(
-            q4, self.execution_buffer_keys[buf], self.execution_buffer_values[buf], previous_out=es_out,
-            previous_lse=es_lse, cache_seqlens=self.valid_lengths[buf])
+        if fuse_est:
+            attn = torch.empty((BG, gs, D), dtype=self.dtype, device=queries.device)
+            kernels.buffer_attention(
+                queries.view(BG, gs, D), self.execution_buffer_keys[buf], self.execution_buffer_values[buf],
+                self.valid_lengths[buf], self.est_ids[buf], self.logits, self.value_sum[layer_idx],
+                self.cluster_size[layer_idx], attn, self.es_cluster_num, self.RSQRT_DIM)
+        else:
+            attn = kernels.weighted_flash_decoding(
+                q4, self.execution_buffer_keys[buf], self.execution_buffer_values[buf], previous_out=es_out,
+                previous_lse=es_lse, cache_seqlens=self.valid_lengths[buf])
         self.wave_buffer[layer_idx].sync()
         kernels.gather_copy_and_scatter(
             self.execution_buffer_keys[buf], self.cache_keys[layer_idx], self.execution_buffer_values[buf],

@@ -653,3 +653,40 @@ extern "C" int ri_wave_attention(const void* q, const void* steady_k, const void
   carve_workspace(P, workspace, BG, gp);
   return launch_attend(P, BG, gs, (hipStream_t)stream);
 }
+
+extern "C" int ri_buffer_attention(const void* q, const void* buf_k, const void* buf_v, int64_t buf_stride,
+                                   const int32_t* cache_seqlens, int max_len, const int32_t* est_ids,
+                                   const float* logits, const void* value_sum, const void* cluster_size_bf16,
+                                   void* out, int BG, int gs, int nc, int es, float scale, void* workspace,
+                                   size_t workspace_bytes, ri_stream_t stream) {
+  if (!q || !buf_k || !buf_v || !cache_seqlens || !out || !workspace) return RI_ERR_ARG;
+  if (BG <= 0 || BG > RI_MAX_GROUPS || gs <= 0 || gs > 16 || max_len <= 0 || max_len > buf_stride || es < 0 ||
+      nc <= 0)
+    return RI_ERR_ARG;
+  if (es > 0 && (!est_ids || !logits || !value_sum || !cluster_size_bf16)) return RI_ERR_ARG;
+  if (workspace_bytes < attn_workspace_bytes(BG, gs)) return RI_ERR_WORKSPACE;
+  const int gp = gs_pad_of(gs);
+  AttendParams P = {};
+  P.q = (const uint16_t*)q;
+  P.kA = P.kB = (const uint16_t*)buf_k;
+  P.vA = P.vB = (const uint16_t*)buf_v;
+  P.strideA = P.strideB = buf_stride;
+  P.lenA = 0;
+  P.lenB_ptr = cache_seqlens;
+  P.lenB_ptr_stride = 1;
+  P.lenB_const = max_len;
+  P.est_ids = est_ids;
+  P.logits = logits;
+  P.value_sum = (const uint16_t*)value_sum;
+  P.csize = (const uint16_t*)cluster_size_bf16;
+  P.nc = nc;
+  P.es = es;
+  P.gs = gs;
+  P.scale = scale;
+  P.out = (uint16_t*)out;
+  // the valid lengths are only known on the device: size the split for a quarter of the buffer
+  plan_splits(max_len / 4 + 64, es, BG, &P.S_kv, &P.S_es);
+  carve_workspace(P, workspace, BG, gp);
+  return launch_attend(P, BG, gs, (hipStream_t)stream);
+}
+

@@ -259,6 +259,19 @@ def wave_attention(q, steady_k, steady_v, static_len, store_k, store_v, row_src,
           "wave_attention")
 
 
+def buffer_attention(q, buf_k, buf_v, cache_seqlens, est_ids, logits, value_sum, cluster_size_bf16, out, es, scale,
+                     slot=0):
+    """Attention over the rows [0, cache_seqlens[g]) of an execution buffer [BG, stride, 128] with the
+    estimation zone (ids and logits from score_select) merged in the same launch."""
+    BG, gs, D = q.shape
+    nc = value_sum.shape[1]
+    stride = buf_k.shape[-3] if buf_k.dim() == 4 else buf_k.shape[-2]
+    ws = _workspace(lib().ri_wave_attention_workspace_bytes(BG, gs), q.device, f"attn{slot}")
+    check(lib().ri_buffer_attention(_p(q), _p(buf_k), _p(buf_v), stride, _p(cache_seqlens), stride, _p(est_ids),
+                                    _p(logits), _p(value_sum), _p(cluster_size_bf16), _p(out), BG, gs, nc, es,
+                                    float(scale), _p(ws), ws.numel(), _stream()), "buffer_attention")
+
+
 def kmeans_assign(data, centroids, assign, P, N, nc, seg, head_rows):
     check(lib().ri_kmeans_assign(_p(data), _p(centroids), _p(assign), P, N, nc, seg, head_rows, _stream()),
           "kmeans_assign")
