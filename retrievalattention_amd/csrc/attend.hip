@@ -185,9 +185,18 @@ __device__ __forceinline__ void combine_group(const AttendParams& P, int g, int 
   for (int j = wave; j < gs; j += 4) {
     const float* ml = P.part_ml + ((size_t)g * S * GS_PAD + j) * 2;
     const float* pa = P.part_acc + ((size_t)g * S * GS_PAD + j) * RI_DIM + 2 * lane;
+    // every load of the merge is issued up front: the statistics (one split per lane) and the
+    // first CB_PRE splits' numerators; their latencies overlap instead of adding up
+    constexpr int CB_PRE = 24;
     float2 ms = make_float2(-INFINITY, 0.f);
     if (lane < S) ms = *reinterpret_cast<const float2*>(ml + (size_t)lane * GS_PAD * 2);
+    float2 a2[CB_PRE];
+#pragma unroll
+    for (int u = 0; u < CB_PRE; ++u)
+      a2[u] = (u < S) ? *reinterpret_cast<const float2*>(pa + (size_t)u * GS_PAD * RI_DIM) : make_float2(0.f, 0.f);
     const float pl = P.prev_lse ? P.prev_lse[(size_t)g * gs + j] : -INFINITY;
+    uint32_t po = 0u;
+    if (P.prev_lse) po = *reinterpret_cast<const uint32_t*>(P.prev_out + ((size_t)g * gs + j) * RI_DIM + 2 * lane);
     float M = fmaxf(ms.x, pl);
 #pragma unroll
     for (int o = 32; o > 0; o >>= 1) M = fmaxf(M, __shfl_xor(M, o));
@@ -198,23 +207,27 @@ __device__ __forceinline__ void combine_group(const AttendParams& P, int g, int 
     float A0 = 0.f, A1 = 0.f;
     if (P.prev_lse) {
       const float fp = (pl == -INFINITY) ? 0.f : __expf(pl - M);
-      const uint32_t po = *reinterpret_cast<const uint32_t*>(P.prev_out + ((size_t)g * gs + j) * RI_DIM + 2 * lane);
       L += fp;
       A0 = fp * __uint_as_float(po << 16);
       A1 = fp * __uint_as_float(po & 0xffff0000u);
     }
-    // numerators: loads are issued eight at a time, ahead of the factors they are scaled by
-    for (int s0 = 0; s0 < S; s0 += 8) {
-      float2 a2[8];
+#pragma unroll
+    for (int u = 0; u < CB_PRE; ++u) {
+      const float fs = __shfl(f, u);
+      A0 += a2[u].x * fs;
+      A1 += a2[u].y * fs;
+    }
+    for (int s0 = CB_PRE; s0 < S; s0 += 8) {
+      float2 b2[8];
 #pragma unroll
       for (int u = 0; u < 8; ++u)
-        a2[u] = (s0 + u < S) ? *reinterpret_cast<const float2*>(pa + (size_t)(s0 + u) * GS_PAD * RI_DIM)
+        b2[u] = (s0 + u < S) ? *reinterpret_cast<const float2*>(pa + (size_t)(s0 + u) * GS_PAD * RI_DIM)
                              : make_float2(0.f, 0.f);
 #pragma unroll
       for (int u = 0; u < 8; ++u) {
         const float fs = __shfl(f, (s0 + u) & 63);
-        A0 += a2[u].x * fs;
-        A1 += a2[u].y * fs;
+        A0 += b2[u].x * fs;
+        A1 += b2[u].y * fs;
       }
     }
     const uint32_t o = (uint32_t)ri_f32_to_bf16(A0 / L) | ((uint32_t)ri_f32_to_bf16(A1 / L) << 16);
