@@ -137,138 +137,162 @@ __global__ void km_zero_kernel(int32_t* a, size_t n) {
   for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) a[i] = 0;
 }
 
-__global__ __launch_bounds__(256) void km_count_kernel(const int32_t* __restrict__ assign,
-                                                       int32_t* __restrict__ counts, int N, int nc) {
-  const int p = blockIdx.y;
-  const int n = blockIdx.x * 256 + threadIdx.x;
-  if (n < N) atomicAdd(&counts[(size_t)p * nc + assign[(size_t)p * N + n]], 1);
+// Inverted lists are a stable sort of the token ids by cluster id: one or two least-significant-
+// digit counting passes of at most 9 bits.  A pass is three launches: per-chunk digit histograms
+// (one wave per chunk of KM_SORT_CHUNK tokens, wave-private LDS counters), an exclusive scan of
+// the [digit][chunk] table per problem, and a scatter in which every wave walks its chunk in
+// token order, ranks equal digits inside each 64-token round with ballots and keeps running
+// positions in LDS.  Stability makes every list ascending without any per-list sort, and no
+// global atomics are involved, so the result does not depend on scheduling.
+#define KM_SORT_CHUNK 1024
+#define KM_SORT_ROUNDS (KM_SORT_CHUNK / 64)
+#define KM_SORT_MAX_BINS 512
+
+__device__ __forceinline__ void km_wave_lds_sync() {
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 }
 
-// one workgroup per problem: offsets = exclusive prefix of counts; cursor = copy of offsets
-__global__ __launch_bounds__(1024) void km_scan_kernel(const int32_t* __restrict__ counts,
-                                                       int32_t* __restrict__ offsets,
-                                                       int32_t* __restrict__ cursor, int nc) {
+// chunk_hist[p][digit][chunk] = tokens of the chunk whose key has that digit
+__global__ __launch_bounds__(256) void km_sort_hist_kernel(const int32_t* __restrict__ keys,
+                                                           int32_t* __restrict__ chunk_hist, int N, int nchunks,
+                                                           int shift, int bits) {
+  __shared__ int32_t sh[4][KM_SORT_MAX_BINS];
+  const int p = blockIdx.y;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int chunk = blockIdx.x * 4 + wave;
+  const int bins = 1 << bits;
+  if (chunk >= nchunks) return;
+  int32_t* h = sh[wave];
+  for (int b = lane; b < bins; b += 64) h[b] = 0;
+  km_wave_lds_sync();
+  const int base = chunk * KM_SORT_CHUNK;
+  int32_t k[KM_SORT_ROUNDS];
+#pragma unroll
+  for (int r = 0; r < KM_SORT_ROUNDS; ++r) {
+    const int i = base + r * 64 + lane;
+    k[r] = (i < N) ? keys[(size_t)p * N + i] : -1;
+  }
+#pragma unroll
+  for (int r = 0; r < KM_SORT_ROUNDS; ++r)
+    if (base + r * 64 + lane < N) atomicAdd(&h[(k[r] >> shift) & (bins - 1)], 1);
+  km_wave_lds_sync();
+  for (int b = lane; b < bins; b += 64) chunk_hist[((size_t)p * bins + b) * nchunks + chunk] = h[b];
+}
+
+// in-place exclusive prefix sum over the n = bins * nchunks entries of each problem
+__global__ __launch_bounds__(1024) void km_sort_scan_kernel(int32_t* __restrict__ chunk_hist, int n) {
   __shared__ int32_t sh_w[16];
   __shared__ int32_t sh_carry;
-  const int p = blockIdx.x;
+  int32_t* a = chunk_hist + (size_t)blockIdx.x * n;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   if (threadIdx.x == 0) sh_carry = 0;
   __syncthreads();
-  for (int base = 0; base < nc; base += 1024) {
-    const int c = base + threadIdx.x;
-    const int32_t v = (c < nc) ? counts[(size_t)p * nc + c] : 0;
-    int32_t inc = v;
+  for (int base = 0; base < n; base += 4096) {
+    const int i0 = base + threadIdx.x * 4;
+    int32_t v[4], run = 0;
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      v[u] = (i0 + u < n) ? a[i0 + u] : 0;
+      run += v[u];
+    }
+    int32_t inc = run;
 #pragma unroll
     for (int d = 1; d < 64; d <<= 1) {
-      const int32_t n = __shfl_up(inc, d);
-      if (lane >= d) inc += n;
+      const int32_t o = __shfl_up(inc, d);
+      if (lane >= d) inc += o;
     }
     if (lane == 63) sh_w[wave] = inc;
     __syncthreads();
     int32_t woff = 0, tot = 0;
 #pragma unroll
     for (int w = 0; w < 16; ++w) {
-      const int32_t s = sh_w[w];
-      if (w < wave) woff += s;
-      tot += s;
+      const int32_t x = sh_w[w];
+      if (w < wave) woff += x;
+      tot += x;
     }
-    const int32_t ex = sh_carry + woff + inc - v;
-    if (c < nc) {
-      offsets[(size_t)p * (nc + 1) + c] = ex;
-      cursor[(size_t)p * nc + c] = ex;
+    int32_t ex = sh_carry + woff + inc - run;
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      if (i0 + u < n) a[i0 + u] = ex;
+      ex += v[u];
     }
     __syncthreads();
     if (threadIdx.x == 0) sh_carry += tot;
     __syncthreads();
   }
-  if (threadIdx.x == 0) offsets[(size_t)p * (nc + 1) + nc] = sh_carry;
 }
 
-__global__ __launch_bounds__(256) void km_scatter_kernel(const int32_t* __restrict__ assign,
-                                                         int32_t* __restrict__ cursor,
-                                                         int32_t* __restrict__ members, int N, int nc) {
+// toks == nullptr: token id = position (first pass); out_keys == nullptr: last pass
+__global__ __launch_bounds__(256) void km_sort_scatter_kernel(const int32_t* __restrict__ keys,
+                                                              const int32_t* __restrict__ toks,
+                                                              const int32_t* __restrict__ chunk_hist,
+                                                              int32_t* __restrict__ out_keys,
+                                                              int32_t* __restrict__ out_toks, int N, int nchunks,
+                                                              int shift, int bits) {
+  __shared__ int32_t sh[4][KM_SORT_MAX_BINS];
   const int p = blockIdx.y;
-  const int n = blockIdx.x * 256 + threadIdx.x;
-  if (n < N) {
-    const int pos = atomicAdd(&cursor[(size_t)p * nc + assign[(size_t)p * N + n]], 1);
-    members[(size_t)p * N + pos] = n;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int chunk = blockIdx.x * 4 + wave;
+  const int bins = 1 << bits;
+  if (chunk >= nchunks) return;
+  int32_t* run = sh[wave];
+  for (int b = lane; b < bins; b += 64) run[b] = chunk_hist[((size_t)p * bins + b) * nchunks + chunk];
+  const int base = chunk * KM_SORT_CHUNK;
+  int32_t k[KM_SORT_ROUNDS], t[KM_SORT_ROUNDS];
+#pragma unroll
+  for (int r = 0; r < KM_SORT_ROUNDS; ++r) {
+    const int i = base + r * 64 + lane;
+    k[r] = (i < N) ? keys[(size_t)p * N + i] : 0;
+    t[r] = (i < N && toks) ? toks[(size_t)p * N + i] : i;
   }
-}
-
-// Ascending sort inside each list.  One wave per cluster for lists of <= 64 entries; longer
-// lists are queued and sorted by whole workgroups.
-__global__ __launch_bounds__(256) void km_sort_small_kernel(const int32_t* __restrict__ counts,
-                                                            const int32_t* __restrict__ offsets,
-                                                            int32_t* __restrict__ members,
-                                                            int32_t* __restrict__ big_list,
-                                                            int32_t* __restrict__ big_count, int N, int nc) {
-  const int p = blockIdx.y;
-  const int c = blockIdx.x * 4 + (threadIdx.x >> 6);
-  const int lane = threadIdx.x & 63;
-  if (c >= nc) return;
-  const int s = counts[(size_t)p * nc + c];
-  if (s <= 1) return;
-  if (s > 64) {
-    if (lane == 0) {
-      const int k = atomicAdd(&big_count[p], 1);
-      big_list[(size_t)p * nc + k] = c;
+  km_wave_lds_sync();
+  const uint64_t below = (1ull << lane) - 1ull;
+#pragma unroll
+  for (int r = 0; r < KM_SORT_ROUNDS; ++r) {
+    const bool valid = base + r * 64 + lane < N;
+    const int bin = (k[r] >> shift) & (bins - 1);
+    uint64_t peers = __ballot(valid);  // lanes of this round with the same digit
+    for (int b = 0; b < bits; ++b) {
+      const bool bit = (bin >> b) & 1;
+      const uint64_t m = __ballot(valid && bit);
+      peers &= bit ? m : ~m;
     }
-    return;
+    const int start = run[bin];
+    km_wave_lds_sync();  // every lane has read the running position before the leader advances it
+    if (valid) {
+      const int pos = start + __popcll(peers & below);
+      if (lane == 63 - __clzll((long long)peers)) run[bin] = start + __popcll(peers);
+      out_toks[(size_t)p * N + pos] = t[r];
+      if (out_keys) out_keys[(size_t)p * N + pos] = k[r];
+    }
+    km_wave_lds_sync();
   }
-  int32_t* base = members + (size_t)p * N + offsets[(size_t)p * (nc + 1) + c];
-  const int32_t x = (lane < s) ? base[lane] : 0x7fffffff;
-  int rank = 0;
-  for (int k = 0; k < s; ++k) rank += (__shfl(x, k) < x);
-  if (lane < s) base[rank] = x;
 }
 
-#define KM_BIG_LDS 8192
-__global__ __launch_bounds__(1024) void km_sort_big_kernel(const int32_t* __restrict__ counts,
-                                                           const int32_t* __restrict__ offsets,
-                                                           int32_t* __restrict__ members,
-                                                           const int32_t* __restrict__ big_list,
-                                                           const int32_t* __restrict__ big_count, int N, int nc) {
-  __shared__ int32_t sh[KM_BIG_LDS];
+// CSR offsets from the sorted members: position i starts every cluster in (key[i-1], key[i]]
+__global__ __launch_bounds__(256) void km_bounds_kernel(const int32_t* __restrict__ assign,
+                                                        const int32_t* __restrict__ members,
+                                                        int32_t* __restrict__ offsets, int N, int nc) {
   const int p = blockIdx.y;
-  const int nbig = big_count[p];
-  for (int k = blockIdx.x; k < nbig; k += gridDim.x) {
-    const int c = big_list[(size_t)p * nc + k];
-    const int s = counts[(size_t)p * nc + c];
-    int32_t* g = members + (size_t)p * N + offsets[(size_t)p * (nc + 1) + c];
-    const bool in_lds = s <= KM_BIG_LDS;
-    int32_t* a = in_lds ? sh : g;
-    if (in_lds)
-      for (int i = threadIdx.x; i < s; i += 1024) sh[i] = g[i];
-    __syncthreads();
-    int P2 = 1;
-    while (P2 < s) P2 <<= 1;
-    // bitonic network with ascending comparators only, so entries past s act as +inf
-    for (int kk = 2; kk <= P2; kk <<= 1) {
-      for (int i = threadIdx.x; i < s; i += 1024) {
-        const int l = i ^ (kk - 1);
-        if (l > i && l < s) {
-          const int32_t x = a[i], y = a[l];
-          if (x > y) { a[i] = y; a[l] = x; }
-        }
-      }
-      __threadfence_block();
-      __syncthreads();
-      for (int j = kk >> 2; j > 0; j >>= 1) {
-        for (int i = threadIdx.x; i < s; i += 1024) {
-          const int l = i ^ j;
-          if (l > i && l < s) {
-            const int32_t x = a[i], y = a[l];
-            if (x > y) { a[i] = y; a[l] = x; }
-          }
-        }
-        __threadfence_block();
-        __syncthreads();
-      }
-    }
-    if (in_lds)
-      for (int i = threadIdx.x; i < s; i += 1024) g[i] = sh[i];
-    __syncthreads();
-  }
+  const int i = blockIdx.x * 256 + threadIdx.x;
+  if (i >= N) return;
+  const int32_t* as = assign + (size_t)p * N;
+  const int32_t* mem = members + (size_t)p * N;
+  int32_t* off = offsets + (size_t)p * (nc + 1);
+  const int c = min(max(as[mem[i]], 0), nc - 1);
+  const int cprev = (i > 0) ? min(max(as[mem[i - 1]], 0), nc - 1) : -1;
+  for (int k = cprev + 1; k <= c; ++k) off[k] = i;
+  if (i == N - 1)
+    for (int k = c + 1; k <= nc; ++k) off[k] = N;
+}
+
+__global__ __launch_bounds__(256) void km_counts_kernel(const int32_t* __restrict__ offsets,
+                                                        int32_t* __restrict__ counts, int nc) {
+  const int p = blockIdx.y;
+  const int c = blockIdx.x * 256 + threadIdx.x;
+  if (c < nc) counts[(size_t)p * nc + c] = offsets[(size_t)p * (nc + 1) + c + 1] - offsets[(size_t)p * (nc + 1) + c];
 }
 
 // ------------------------------------------------------------------------------------
@@ -458,10 +482,12 @@ extern "C" int ri_kmeans_assign(const void* data, const void* centroids, int32_t
   return RI_OK;
 }
 
+static int km_sort_chunks(int N) { return (N + KM_SORT_CHUNK - 1) / KM_SORT_CHUNK; }
+
 extern "C" size_t ri_kmeans_workspace_bytes(int P, int N, int nc) {
   if (P <= 0 || N <= 0 || nc <= 0) return 0;
-  // cursor [P, nc] + big_list [P, nc] + big_count [P]
-  return ((size_t)P * nc * 2 + (size_t)P) * sizeof(int32_t);
+  // digit table [P, 512, chunks] + one (key, token) staging pair [P, N] for the two-pass case
+  return ((size_t)P * KM_SORT_MAX_BINS * km_sort_chunks(N) + 2 * (size_t)P * N) * sizeof(int32_t);
 }
 
 extern "C" int ri_kmeans_build_lists(const int32_t* assign, int32_t* counts, int32_t* offsets,
@@ -470,25 +496,38 @@ extern "C" int ri_kmeans_build_lists(const int32_t* assign, int32_t* counts, int
   if (!assign || !counts || !offsets || !members || !workspace) return RI_ERR_ARG;
   int rc = km_check(P, N, nc);
   if (rc) return rc;
+  if (nc > (1 << 18)) return RI_ERR_ARG;  // two passes of at most 9 bits
   if (workspace_bytes < ri_kmeans_workspace_bytes(P, N, nc)) return RI_ERR_WORKSPACE;
   hipStream_t s = (hipStream_t)stream;
-  int32_t* cursor = (int32_t*)workspace;
-  int32_t* big_list = cursor + (size_t)P * nc;
-  int32_t* big_count = big_list + (size_t)P * nc;
-  km_zero_kernel<<<256, 256, 0, s>>>(counts, (size_t)P * nc);
+  const int nchunks = km_sort_chunks(N);
+  int32_t* chunk_hist = (int32_t*)workspace;
+  int32_t* tmp_key = chunk_hist + (size_t)P * KM_SORT_MAX_BINS * nchunks;
+  int32_t* tmp_tok = tmp_key + (size_t)P * N;
+  int total_bits = 1;
+  while ((1 << total_bits) < nc) ++total_bits;
+  const int lo_bits = total_bits <= 9 ? total_bits : (total_bits + 1) / 2;
+  const int hi_bits = total_bits - lo_bits;
+  const dim3 cgrid((nchunks + 3) / 4, P);
+  // pass over the low digit (the only one when the ids fit 9 bits)
+  km_sort_hist_kernel<<<cgrid, 256, 0, s>>>(assign, chunk_hist, N, nchunks, 0, lo_bits);
   RI_HIP_CHECK_LAUNCH();
-  km_zero_kernel<<<1, 256, 0, s>>>(big_count, (size_t)P);
+  km_sort_scan_kernel<<<P, 1024, 0, s>>>(chunk_hist, (1 << lo_bits) * nchunks);
   RI_HIP_CHECK_LAUNCH();
-  const dim3 tok_grid((N + 255) / 256, P);
-  km_count_kernel<<<tok_grid, 256, 0, s>>>(assign, counts, N, nc);
+  km_sort_scatter_kernel<<<cgrid, 256, 0, s>>>(assign, nullptr, chunk_hist, hi_bits ? tmp_key : nullptr,
+                                               hi_bits ? tmp_tok : members, N, nchunks, 0, lo_bits);
   RI_HIP_CHECK_LAUNCH();
-  km_scan_kernel<<<P, 1024, 0, s>>>(counts, offsets, cursor, nc);
+  if (hi_bits) {
+    km_sort_hist_kernel<<<cgrid, 256, 0, s>>>(tmp_key, chunk_hist, N, nchunks, lo_bits, hi_bits);
+    RI_HIP_CHECK_LAUNCH();
+    km_sort_scan_kernel<<<P, 1024, 0, s>>>(chunk_hist, (1 << hi_bits) * nchunks);
+    RI_HIP_CHECK_LAUNCH();
+    km_sort_scatter_kernel<<<cgrid, 256, 0, s>>>(tmp_key, tmp_tok, chunk_hist, nullptr, members, N, nchunks,
+                                                 lo_bits, hi_bits);
+    RI_HIP_CHECK_LAUNCH();
+  }
+  km_bounds_kernel<<<dim3((N + 255) / 256, P), 256, 0, s>>>(assign, members, offsets, N, nc);
   RI_HIP_CHECK_LAUNCH();
-  km_scatter_kernel<<<tok_grid, 256, 0, s>>>(assign, cursor, members, N, nc);
-  RI_HIP_CHECK_LAUNCH();
-  km_sort_small_kernel<<<dim3((nc + 3) / 4, P), 256, 0, s>>>(counts, offsets, members, big_list, big_count, N, nc);
-  RI_HIP_CHECK_LAUNCH();
-  km_sort_big_kernel<<<dim3(16, P), 1024, 0, s>>>(counts, offsets, members, big_list, big_count, N, nc);
+  km_counts_kernel<<<dim3((nc + 255) / 256, P), 256, 0, s>>>(offsets, counts, nc);
   RI_HIP_CHECK_LAUNCH();
   return RI_OK;
 }
