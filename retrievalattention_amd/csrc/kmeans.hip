@@ -7,9 +7,15 @@
 typedef float f32x16_t __attribute__((ext_vector_type(16)));
 
 #define KM_CT 64          // centroid rows per LDS tile (two 32-row MFMA halves)
-#define KM_TT 4           // 32-token MFMA columns per wave: 128 tokens held in registers
-#define KM_WG_TOKENS (4 * 32 * KM_TT)
 #define KM_ROW_U16 136    // padded LDS row (272 bytes) to spread ds_read_b128 over the banks
+#ifndef KM_TT
+#define KM_TT 4           // 32-token MFMA columns per wave, held in registers
+#endif
+#ifndef KM_WAVES
+#define KM_WAVES 4        // waves per workgroup sharing one centroid tile
+#endif
+#define KM_WG_TOKENS (KM_WAVES * 32 * KM_TT)
+#define KM_PIECES ((KM_CT * 16 + KM_WAVES * 64 - 1) / (KM_WAVES * 64))  // 16-byte tile pieces per thread
 
 // first data row of problem p: problems are `seg` consecutive N-row slices of each head
 __device__ __forceinline__ size_t km_row0(int p, int seg, int64_t head_rows, int N) {
@@ -17,18 +23,20 @@ __device__ __forceinline__ size_t km_row0(int p, int seg, int64_t head_rows, int
 }
 
 // ------------------------------------------------------------------------------------
-// assign: grid (ceil(N/512), P), 256 threads; wave = 128 tokens (four 32-token MFMA columns,
-// four independent accumulator chains) held in registers for the whole kernel.  Centroid tiles of 64 rows go through two LDS
-// buffers shared by the four waves: the next tile's global loads are issued before the MFMAs
-// of the current one and stored to the other buffer after them, one barrier per tile.
+// assign: grid (ceil(N / KM_WG_TOKENS), P), KM_WAVES waves; a wave keeps KM_TT columns of 32
+// tokens in registers for the whole kernel (KM_TT independent accumulator chains).  Centroid
+// tiles of 64 rows go through two LDS buffers shared by all waves of the workgroup: the next
+// tile's global loads are issued before the MFMAs of the current one and stored to the other
+// buffer after them, one barrier per tile.  (4 tokens columns x 4 waves measured fastest on
+// the full-size pass against 2x4, 2x8, 2x12, 3x8 with clocks warmed up and runs interleaved.)
 // MFMA 32x32x16: A = centroid rows, B = token columns; accumulator i of lane l is
 // row (i/4)*8 + (l/32)*4 + i%4, column l%32.  nc is a multiple of 32; the last tile may hold
 // one half only.
 // ------------------------------------------------------------------------------------
-__global__ __launch_bounds__(256) void km_assign_kernel(const uint16_t* __restrict__ data,
-                                                        const uint16_t* __restrict__ cent,
-                                                        int32_t* __restrict__ assign, int N, int nc, int seg,
-                                                        int64_t head_rows) {
+__global__ __launch_bounds__(KM_WAVES * 64) void km_assign_kernel(const uint16_t* __restrict__ data,
+                                                                  const uint16_t* __restrict__ cent,
+                                                                  int32_t* __restrict__ assign, int N, int nc,
+                                                                  int seg, int64_t head_rows) {
   __shared__ __attribute__((aligned(16))) uint16_t sh_c[2][KM_CT][KM_ROW_U16];
   const int p = blockIdx.y;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -36,15 +44,25 @@ __global__ __launch_bounds__(256) void km_assign_kernel(const uint16_t* __restri
   const int t0 = blockIdx.x * KM_WG_TOKENS + wave * (32 * KM_TT);
   const uint16_t* dp = data + km_row0(p, seg, head_rows, N) * RI_DIM;
   const uint16_t* cp = cent + (size_t)p * nc * RI_DIM;
-  // this thread's four 16-byte pieces of a tile: rows prow + 16 u, piece ppiece
-  const int prow = threadIdx.x >> 4, ppiece = threadIdx.x & 15;
 
-  uint4 pf[4];
+  // this thread's 16-byte pieces of a tile: piece index threadIdx.x + u * threads -> (row, column piece)
+  uint4 pf[KM_PIECES];
+  auto tile_load = [&](int ct) {
 #pragma unroll
-  for (int u = 0; u < 4; ++u) {
-    const int row = prow + 16 * u;
-    pf[u] = (row < nc) ? ri_ld16(cp + (size_t)row * RI_DIM + ppiece * 8) : ri_zero16();
-  }
+    for (int u = 0; u < KM_PIECES; ++u) {
+      const int idx = threadIdx.x + u * (KM_WAVES * 64);
+      const int row = ct + (idx >> 4);
+      pf[u] = (idx < KM_CT * 16 && row < nc) ? ri_ld16(cp + (size_t)row * RI_DIM + (idx & 15) * 8) : ri_zero16();
+    }
+  };
+  auto tile_store = [&](int buf) {
+#pragma unroll
+    for (int u = 0; u < KM_PIECES; ++u) {
+      const int idx = threadIdx.x + u * (KM_WAVES * 64);
+      if (idx < KM_CT * 16) *reinterpret_cast<uint4*>(&sh_c[buf][idx >> 4][(idx & 15) * 8]) = pf[u];
+    }
+  };
+  tile_load(0);
   uint4 b[KM_TT][8];
 #pragma unroll
   for (int tt = 0; tt < KM_TT; ++tt) {
@@ -53,8 +71,7 @@ __global__ __launch_bounds__(256) void km_assign_kernel(const uint16_t* __restri
 #pragma unroll
     for (int kk = 0; kk < 8; ++kk) b[tt][kk] = (tok < N) ? ri_ld16(q + kk * 16) : ri_zero16();
   }
-#pragma unroll
-  for (int u = 0; u < 4; ++u) *reinterpret_cast<uint4*>(&sh_c[0][prow + 16 * u][ppiece * 8]) = pf[u];
+  tile_store(0);
   __syncthreads();
 
   float best[KM_TT];
@@ -67,13 +84,7 @@ __global__ __launch_bounds__(256) void km_assign_kernel(const uint16_t* __restri
   int buf = 0;
   for (int ct = 0; ct < nc; ct += KM_CT, buf ^= 1) {
     const int nxt = ct + KM_CT;
-    if (nxt < nc) {
-#pragma unroll
-      for (int u = 0; u < 4; ++u) {
-        const int row = nxt + prow + 16 * u;
-        pf[u] = (row < nc) ? ri_ld16(cp + (size_t)row * RI_DIM + ppiece * 8) : ri_zero16();
-      }
-    }
+    if (nxt < nc) tile_load(nxt);
 #pragma unroll
     for (int half = 0; half < 2; ++half) {
       if (ct + half * 32 < nc) {  // uniform: only the last tile can lack its second half
@@ -111,10 +122,7 @@ __global__ __launch_bounds__(256) void km_assign_kernel(const uint16_t* __restri
         }
       }
     }
-    if (nxt < nc) {
-#pragma unroll
-      for (int u = 0; u < 4; ++u) *reinterpret_cast<uint4*>(&sh_c[buf ^ 1][prow + 16 * u][ppiece * 8]) = pf[u];
-    }
+    if (nxt < nc) tile_store(buf ^ 1);
     __syncthreads();
   }
 #pragma unroll
@@ -476,7 +484,7 @@ extern "C" int ri_kmeans_assign(const void* data, const void* centroids, int32_t
   int rc = km_check(P, N, nc);
   if (rc) return rc;
   if (nc % 32 != 0 || seg <= 0 || P % seg != 0) return RI_ERR_ARG;
-  km_assign_kernel<<<dim3((N + KM_WG_TOKENS - 1) / KM_WG_TOKENS, P), 256, 0, (hipStream_t)stream>>>(
+  km_assign_kernel<<<dim3((N + KM_WG_TOKENS - 1) / KM_WG_TOKENS, P), KM_WAVES * 64, 0, (hipStream_t)stream>>>(
       (const uint16_t*)data, (const uint16_t*)centroids, assign, N, nc, seg, head_rows);
   RI_HIP_CHECK_LAUNCH();
   return RI_OK;
