@@ -250,7 +250,7 @@ __device__ __forceinline__ void combine_group(const AttendParams& P, int g, int 
   if (threadIdx.x == 0 && P.valid_lengths) P.valid_lengths[g] = P.lenA + lenB;
 }
 
-#define ATT_DESC_MAX 512  // rows of one wave whose descriptors are staged in LDS at a time
+#define ATT_DESC_MAX 128  // rows of one wave whose descriptors are staged in LDS at a time
 
 // PF = chunks (of 16 rows) in flight per wave: the loads of chunk j+PF are issued before chunk j
 // is computed
@@ -560,7 +560,7 @@ static int launch_attend(AttendParams& P, int BG, int gs, hipStream_t s) {
   const dim3 grid(S, BG);
   P.fuse = fuse_default();
   switch (gs_pad_of(gs)) {
-    case 4: attend_kernel<4, 3><<<grid, 256, 0, s>>>(P); break;
+    case 4: attend_kernel<4, 2><<<grid, 256, 0, s>>>(P); break;
     case 8: attend_kernel<8, 2><<<grid, 256, 0, s>>>(P); break;
     default: attend_kernel<16, 2><<<grid, 256, 0, s>>>(P); break;
   }
@@ -578,7 +578,8 @@ static int launch_attend(AttendParams& P, int BG, int gs, hipStream_t s) {
 
 // Split plan: about two workgroups per compute unit in total (an even load over the 256 CUs,
 // all resident at once), at least 128 rows per workgroup, the budget shared between the
-// key/value rows and the estimation rows in proportion to their counts.
+// key/value rows and the estimation rows in proportion to their cost (a key/value row counts
+// twice: K and V rows and the QK product against one value-sum row).
 static void plan_splits(int64_t kv_rows, int64_t es_rows, int BG, int* S_kv, int* S_es) {
   const int target_wgs = 512;
   int per_group = target_wgs / BG;
@@ -594,7 +595,7 @@ static void plan_splits(int64_t kv_rows, int64_t es_rows, int BG, int* S_kv, int
     return;
   }
   if (per_group < 2) per_group = 2;
-  int kv = (int)((kv_rows * per_group + rows / 2) / rows);
+  int kv = (int)((kv_rows * 2 * per_group + (kv_rows * 2 + es_rows) / 2) / (kv_rows * 2 + es_rows));
   if (kv < 1) kv = 1;
   if (kv > per_group - 1) kv = per_group - 1;
   *S_kv = kv;
