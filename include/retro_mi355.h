@@ -93,6 +93,15 @@ int ri_score_select(const void* q, const void* centroids, const uint8_t* mask,
                     int page, int max_pages, float scale, void* workspace,
                     size_t workspace_bytes, ri_stream_t stream);
 
+/* Scores only: logits[g, j, c] = scale * <q[g,j,:], centroids[g,c,:]> in fp32, no selection.
+ * Used when the zones of a layer were chosen ahead of time from a predicted query
+ * (use_cluster_estimation, cache_hub/retroinfer_cache.py:582-595) and the estimation zone must be
+ * scored with the layer's true query (the reference does that by gathering the zone's centroids
+ * and running weighted_flash_decoding over them, :598-617).
+ * workspace: ri_score_select_workspace_bytes(BG, gs, nc). */
+int ri_score_logits(const void* q, const void* centroids, float* logits, int BG, int gs, int nc,
+                    float scale, void* workspace, size_t workspace_bytes, ri_stream_t stream);
+
 /* ------------------------------------------------------------------------------------
  * (4) Weighted flash decoding
  * ---------------------------------------------------------------------------------- */

@@ -28,15 +28,16 @@ def cluster_store(keys, values, lists, size):
 
 
 def decode_step(q, steady_k, steady_v, static_len, centroids, value_sum, mask, size_i32, size_bf16, store_k,
-                store_v, start, nprobe, es, page, max_pages, logits=None):
+                store_v, start, nprobe, es, page, max_pages, logits=None, zone_logits=None):
     """One layer's decode attention for all groups.
     q [BG, gs, D]; steady_* [BG, >=static_len, D]; centroids/value_sum [BG, nc, D]; mask, size_* [BG, nc];
     store_* list of per-group [rows, D]; start [BG, nc].  `logits` lets a test substitute the scores the
-    kernels produced.  Returns (out bf16 [BG, gs, D], aux)."""
+    kernels produced.  `zone_logits`: scores of another (predicted) query that choose the zones while the
+    estimation zone is still scored by q (next-layer cluster estimation, retroinfer_cache.py:582-617).  Returns (out bf16 [BG, gs, D], aux)."""
     BG, gs, D = q.shape
     scale = 1.0 / math.sqrt(D)
     x = scoring.logits_fp32(q, centroids, scale) if logits is None else logits
-    _, _, _, soft = scoring.softmax_from_logits(x)
+    _, _, _, soft = scoring.softmax_from_logits(x if zone_logits is None else zone_logits)
     dist = scoring.dist_from_softmax(soft, mask)
     ret, est = scoring.select(dist, nprobe, es)
     kept, offs = scoring.retrieval_layout(ret, size_i32, page, max_pages)

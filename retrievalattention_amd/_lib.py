@@ -19,6 +19,7 @@ SIGNATURES = {
     "ri_batch_gemm_softmax": (I, [P, P, P, P, P, P, I, I, I, I, F, F, P]),
     "ri_score_select_workspace_bytes": (SZ, [I, I, I]),
     "ri_score_select": (I, [P, P, P, P, P, P, P, P, P, P, P, P, I, P, I, I, I, I, I, I, I, F, P, SZ, P]),
+    "ri_score_logits": (I, [P, P, P, I, I, I, F, P, SZ, P]),
     "ri_flash_decoding_workspace_bytes": (SZ, [I, I]),
     "ri_weighted_flash_decoding": (I, [P, P, P, P, P, P, P, P, P, I, I, I, I64, F, P, SZ, P]),
     "ri_wave_attention_workspace_bytes": (SZ, [I, I]),

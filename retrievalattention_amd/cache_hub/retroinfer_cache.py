@@ -170,9 +170,12 @@ class retroinfer_cache(KV_Cache):
         self.est_ids = [i32(BG, max(self.es_cluster_num, 1)) for _ in range(2)]
         self.valid_lengths = [i32(BG) for _ in range(2)]
         if self.kv_residency == "device":
-            self.ret_tok_off = i32(BG, self.nprobe + 1)
-            self.row_src = i32(BG, self.buffer_size * self.page_size)
-            self.meta = i32(BG, 4)
+            # token layout of the retrieval zone; a second set when the next layer's zones are chosen
+            # while this layer's are still in use
+            sets = 2 if self.use_cluster_estimation else 1
+            self.layouts = [(i32(BG, self.nprobe + 1), i32(BG, self.buffer_size * self.page_size), i32(BG, 4))
+                            for _ in range(sets)]
+            self.ret_tok_off, self.row_src, self.meta = self.layouts[0]
         else:
             shape = (BG, self.execution_stride, 1, D)
             self.execution_buffer_keys = [torch.zeros(shape, dtype=self.dtype, device=d0) for _ in range(2)]
@@ -321,17 +324,17 @@ class retroinfer_cache(KV_Cache):
         return None, None
 
     # ------------------------------------------------------------------ decode
-    def _select(self, queries, layer, buf, with_layout):
+    def _select(self, queries, layer, buf, with_layout, layout=0):
         BG, gs, D = self.batch_groups, self.group_size, self.head_dim
         q = queries.view(BG, gs, D)
         es = self.es_cluster_num
         dev_mode = with_layout and self.kv_residency == "device"
+        ret_tok_off, row_src, meta = self.layouts[layout] if dev_mode else (None, None, None)
         kernels.score_select(
             q, self.centroids[layer], self.centroids_mask[layer],
             self.cluster_size_i32[layer] if dev_mode else None, self.cluster_start[layer] if dev_mode else None,
             self.logits, None, self.cI[buf], self.ret_ids[buf], self.est_ids[buf] if es > 0 else None,
-            self.ret_tok_off if dev_mode else None, self.row_src if dev_mode else None,
-            self.meta if dev_mode else None, self.nprobe, es, self.page_size, self.buffer_size, self.RSQRT_DIM)
+            ret_tok_off, row_src, meta, self.nprobe, es, self.page_size, self.buffer_size, self.RSQRT_DIM)
 
     def compute(self, queries, layer_idx, queries_next=None):
         """Decode attention of one layer (reference: retroinfer_cache.py:549-697).
@@ -435,8 +438,26 @@ class retroinfer_cache(KV_Cache):
 
     def _compute_device_estimated(self, queries, layer_idx, queries_next, static_len, buf, nbuf, search_here,
                                   search_next):
-        """Device residency with next-layer cluster estimation: zones come from the query the
-        previous layer predicted, scores of the estimation zone from the true query."""
-        raise NotImplementedError(
-            "use_cluster_estimation with kv_residency='device' is not available: a device-resident "
-            "store has no transfer to hide; construct the cache with use_cluster_estimation=False")
+        """Device residency with next-layer cluster estimation (reference: retroinfer_cache.py:565,
+        582-595): from the third layer on the zones come from the query the previous layer
+        predicted; the estimation zone is scored with the true query, the retrieval zone is
+        attended exactly.  A device-resident store has no transfer to hide, so this mode exists for
+        behavioural parity, not speed: the next layer's zones are chosen after this layer's attention."""
+        BG, gs, D = self.batch_groups, self.group_size, self.head_dim
+        es = self.es_cluster_num
+        q = queries.view(BG, gs, D)
+        if search_here:
+            self._select(queries, layer_idx, buf, True, layout=buf)
+        elif es > 0:
+            kernels.score_logits(q, self.centroids[layer_idx], self.logits, self.RSQRT_DIM)
+        ret_tok_off, row_src, meta = self.layouts[buf]
+        out = torch.empty((BG, gs, D), dtype=self.dtype, device=queries.device)
+        kernels.wave_attention(
+            q, self.steady_zone_keys[layer_idx], self.steady_zone_values[layer_idx], static_len,
+            self.list_keys[layer_idx], self.list_values[layer_idx], row_src, meta,
+            self.est_ids[buf] if es > 0 else None, self.logits if es > 0 else None, self.value_sum[layer_idx],
+            self.cluster_size[layer_idx], out, self.valid_lengths[buf], es, self.RSQRT_DIM)
+        if search_next:
+            self._select(queries_next, layer_idx + 1, nbuf, True, layout=nbuf)
+        return out.view(self.batch_size, 1, self.num_heads, D)
+

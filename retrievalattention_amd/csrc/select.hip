@@ -402,3 +402,14 @@ extern "C" int ri_score_select(const void* q, const void* centroids, const uint8
   RI_HIP_CHECK_LAUNCH();
   return RI_OK;
 }
+
+extern "C" int ri_score_logits(const void* q, const void* centroids, float* logits, int BG, int gs, int nc,
+                               float scale, void* workspace, size_t workspace_bytes, ri_stream_t stream) {
+  if (!q || !centroids || !logits || !workspace) return RI_ERR_ARG;
+  if (BG <= 0 || gs <= 0 || gs > 16 || nc <= 0 || (nc % 4) != 0) return RI_ERR_ARG;
+  if (workspace_bytes < ri_score_select_workspace_bytes(BG, gs, nc)) return RI_ERR_WORKSPACE;
+  const int ntiles = (nc + RI_SCORE_TILE - 1) / RI_SCORE_TILE;
+  float* tmax = (float*)workspace;
+  float* tsum = (float*)((char*)workspace + align256((size_t)BG * ntiles * gs * sizeof(float)));
+  return ri_launch_score(q, centroids, logits, tmax, tsum, BG, gs, nc, scale, (hipStream_t)stream);
+}

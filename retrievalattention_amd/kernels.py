@@ -244,6 +244,15 @@ def score_select(q, centroids, mask, cluster_size_i32, cluster_start, logits, di
           "score_select")
 
 
+def score_logits(q, centroids, logits, scale, slot=0):
+    """logits [BG, gs, nc] fp32 = scale * q . centroids^T, no selection."""
+    BG, gs, D = q.shape
+    nc = centroids.shape[1]
+    ws = _workspace(lib().ri_score_select_workspace_bytes(BG, gs, nc), q.device, f"score{slot}")
+    check(lib().ri_score_logits(_p(q), _p(centroids), _p(logits), BG, gs, nc, float(scale), _p(ws), ws.numel(),
+                                _stream()), "score_logits")
+
+
 def wave_attention(q, steady_k, steady_v, static_len, store_k, store_v, row_src, meta, est_ids, logits,
                    value_sum, cluster_size_bf16, out, valid_lengths, es, scale, slot=0):
     """Attention over steady zone + retrieved clusters (read in place) + estimation zone.

@@ -19,7 +19,7 @@ def _close(got, ref):
 
 
 def _make_cache(dev, residency, layers, B, Hkv, gs, ctx, n_centroids, n_segment, nprobe, es, new=8,
-                cache_cluster_num=None):
+                cache_cluster_num=None, use_cluster_estimation=False):
     from retrievalattention_amd.cache_hub import retroinfer_cache
     return retroinfer_cache(
         valid_start=[0] * B, layer_num=layers, batch_size=B, max_length=ctx + new, num_key_value_heads=Hkv,
@@ -27,7 +27,7 @@ def _make_cache(dev, residency, layers, B, Hkv, gs, ctx, n_centroids, n_segment,
         max_new_length=new, static_pattern_start=4, static_pattern_end=64, core=4, n_centroids=n_centroids,
         n_segment=n_segment, nprobe=nprobe, max_compute_cluster_num=nprobe + es, cache_unit_size=8,
         cache_cluster_num=cache_cluster_num if cache_cluster_num is not None else 3 * nprobe, num_gpus=1,
-        model_size=8, kv_residency=residency)
+        model_size=8, use_cluster_estimation=use_cluster_estimation, kv_residency=residency)
 
 
 def _prefill(cache, K, V, layers, B):
@@ -161,3 +161,60 @@ def test_host_and_device_residency_agree_and_cache_warms(dev):
         assert torch.equal(cd.valid_lengths[0].cpu(), ch.valid_lengths[0].cpu())
         hits.append(int(ch.hit_num_units[0].sum()))
     assert hits[0] == 0 and hits[1] > 0 and hits[2] >= hits[1]
+
+
+@pytest.mark.parametrize("residency", ["device", "host"])
+def test_next_layer_cluster_estimation(dev, residency):
+    """use_cluster_estimation (reference: retroinfer_cache.py:565, 582-595): layers 0 and 1 choose their
+    zones from their own query; every later layer uses the zones the previous layer chose from a
+    predicted query, scores its estimation zone with the true query and attends the retrieval zone
+    exactly.  Checked against the oracle with the same split between zone query and true query."""
+    layers, B, Hkv, gs, ctx = 4, 2, 2, 4, 4096 + 68
+    nc, nprobe, es = 256, 8, 60
+    cache = _make_cache(dev, residency, layers, B, Hkv, gs, ctx, nc, 1, nprobe, es, use_cluster_estimation=True)
+    K, V = _gen(layers, B, Hkv, gs, ctx, 256, dev, 11)
+    _prefill(cache, K, V, layers, B)
+    BG = B * Hkv
+    g = torch.Generator().manual_seed(12)
+    q_true = [torch.randn(B, 1, Hkv * gs, 128, generator=g).to(torch.bfloat16) for _ in range(layers)]
+    # the prediction for layer l (made at layer l-1) is off by a fair amount: zones differ from the true ones
+    q_pred = [(q.float() + 0.5 * torch.randn(q.shape, generator=g)).to(torch.bfloat16) for q in q_true]
+    differs = 0
+    for l in range(layers):
+        kn = torch.randn(B, 1, Hkv, 128, generator=g).to(torch.bfloat16)
+        vn = torch.randn(B, 1, Hkv, 128, generator=g).to(torch.bfloat16)
+        cache.decode_update_kv_cache(kn.to(dev), vn.to(dev), l)
+        nxt = q_pred[l + 1].to(dev) if l + 1 < layers else None
+        out = cache.compute(q_true[l].to(dev), l, nxt)
+        torch.cuda.synchronize()
+        static_len = cache.static_pattern_total if l == layers - 1 else cache.static_pattern_total + 1
+        if l == layers - 1:
+            static_len = cache.static_pattern_total
+        size_bf = cache.cluster_size[l].cpu()
+        size_i = size_bf.float().to(torch.int32)
+        rows = size_i.sum(1)
+        lk, lv = cache.list_keys[l].view(BG, -1, 128), cache.list_values[l].view(BG, -1, 128)
+        sk = [lk[gi, :int(rows[gi])].cpu() for gi in range(BG)]
+        sv = [lv[gi, :int(rows[gi])].cpu() for gi in range(BG)]
+        start = torch.cumsum(size_i.long(), 1) - size_i.long()
+        zone = None
+        if l >= 2:   # zones were chosen at layer l-1 from the predicted query
+            zone = scoring.logits_fp32(q_pred[l].view(BG, gs, 128), cache.centroids[l].cpu(), 1.0 / math.sqrt(128))
+        ref, aux = pipeline.decode_step(
+            q_true[l].view(BG, gs, 128), cache.steady_zone_keys[l].view(BG, -1, 128).cpu(),
+            cache.steady_zone_values[l].view(BG, -1, 128).cpu(), static_len, cache.centroids[l].cpu(),
+            cache.value_sum[l].cpu(), cache.centroids_mask[l].cpu(), size_i, size_bf, sk, sv, start, nprobe, es, 8,
+            cache.buffer_size, zone_logits=zone)
+        _close(out.cpu().view(BG, gs, 128), ref)
+        buf = l % 2
+        cI = cache.cI[buf].cpu()
+        check_zone_sets(aux["dist"], cI[:, :nprobe], cI[:, nprobe:], aux["ret"], aux["est"], nprobe, es, band=2.0)
+        if l >= 2:   # the predicted zones are not the true query's zones (otherwise the test shows nothing)
+            _, aux_true = pipeline.decode_step(
+                q_true[l].view(BG, gs, 128), cache.steady_zone_keys[l].view(BG, -1, 128).cpu(),
+                cache.steady_zone_values[l].view(BG, -1, 128).cpu(), static_len, cache.centroids[l].cpu(),
+                cache.value_sum[l].cpu(), cache.centroids_mask[l].cpu(), size_i, size_bf, sk, sv, start, nprobe, es, 8,
+                cache.buffer_size)
+            differs += int((aux_true["ret"] != aux["ret"]).any())
+    assert differs > 0
+
