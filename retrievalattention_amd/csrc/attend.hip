@@ -255,7 +255,7 @@ __device__ __forceinline__ void combine_group(const AttendParams& P, int g, int 
 // PF = chunks (of 16 rows) in flight per wave: the loads of chunk j+PF are issued before chunk j
 // is computed
 template <int GS_PAD, int PF>
-__global__ __launch_bounds__(256, GS_PAD == 16 ? 1 : 2) void attend_kernel(AttendParams P) {
+__global__ __launch_bounds__(256, GS_PAD == 16 ? 1 : 3) void attend_kernel(AttendParams P) {
   constexpr int NH = GS_PAD / 4;
   __shared__ __attribute__((aligned(16))) uint16_t sh_vt[4][16 * ATT_VT_STRIDE];
   __shared__ __attribute__((aligned(16))) uint16_t sh_pb[4][16 * 16];
@@ -581,7 +581,10 @@ static int launch_attend(AttendParams& P, int BG, int gs, hipStream_t s) {
 // key/value rows and the estimation rows in proportion to their cost (a key/value row counts
 // twice: K and V rows and the QK product against one value-sum row).
 static void plan_splits(int64_t kv_rows, int64_t es_rows, int BG, int* S_kv, int* S_es) {
-  const int target_wgs = 512;
+  // two workgroups per compute unit while the launch is short (latency counts); three once every
+  // workgroup has more than 512 rows to stream (throughput counts)
+  const int64_t all_rows = (kv_rows + es_rows) * BG;
+  const int target_wgs = all_rows > 512 * 512 ? 768 : 512;
   int per_group = target_wgs / BG;
   if (per_group < 1) per_group = 1;
   if (per_group > RI_MAX_SPLITS) per_group = RI_MAX_SPLITS;
