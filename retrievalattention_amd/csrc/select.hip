@@ -168,7 +168,7 @@ __global__ __launch_bounds__(SEL_THREADS) void select_kernel(
   __shared__ uint32_t sh_sel[4];  // bin of T1, entries above it, bin of T2, entries above it
   __shared__ uint32_t sh_ret[1024];
   __shared__ uint32_t sh_sorted[1024];
-  __shared__ uint32_t sh_pages, sh_tret;
+  __shared__ uint32_t sh_pages, sh_tret, sh_nkeep;
 
   const int g = blockIdx.x;
   const int tid = threadIdx.x;
@@ -189,7 +189,7 @@ __global__ __launch_bounds__(SEL_THREADS) void select_kernel(
       *reinterpret_cast<int4*>(&sh_size[c]) = *reinterpret_cast<const int4*>(cluster_size + (size_t)g * nc + c);
 #pragma unroll
   for (int i = 0; i < SEL_BPT; ++i) hist[tid * SEL_BPT + i] = 0u;
-  if (tid == 0) { sh_pages = 0; sh_tret = 0; }
+  if (tid == 0) { sh_pages = 0; sh_tret = 0; sh_nkeep = 0; }
   __syncthreads();
   // calls f(id, key) for every owned key in ascending id order
   auto for_each_key = [&](auto&& f) {
@@ -314,11 +314,22 @@ __global__ __launch_bounds__(SEL_THREADS) void select_kernel(
     // kept clusters form a prefix because the page prefix is monotone; tokens before a kept
     // cluster all belong to kept clusters
     keep = r < np && pg_run + pg <= (uint32_t)max_pages;
+    // the kept clusters are the ranks 0 .. nkeep-1: the last of them publishes the totals
     if (keep) {
-      atomicMax(&sh_pages, pg_run + pg);
-      atomicMax(&sh_tret, tok_run + sz);
+      bool next_keep = false;
+      if (r + 1 < np) {
+        const int nc_ = (int)(0xffffu - (sh_sorted[r + 1] & 0xffffu));
+        const uint32_t sz_n = (uint32_t)(sizes_in_lds ? sh_size[nc_] : cluster_size[(size_t)g * nc + nc_]);
+        next_keep = pg_run + pg + (sz_n + page - 1) / page <= (uint32_t)max_pages;
+      }
+      if (!next_keep) {
+        sh_pages = pg_run + pg;
+        sh_tret = tok_run + sz;
+        sh_nkeep = (uint32_t)r + 1u;
+      }
     }
-    nkeep = __syncthreads_count(keep);
+    __syncthreads();
+    nkeep = (int)sh_nkeep;
     T_ret = (int32_t)sh_tret;
   }
 
