@@ -244,6 +244,34 @@ int ri_kmeans_value_sum(const void* values, const int32_t* counts, const int32_t
                         const int32_t* members, void* value_sum, int P, int N, int nc,
                         void* workspace, size_t workspace_bytes, ri_stream_t stream);
 
+/* Device-side block cache manager: BufferManager::batch_access followed by
+ * BufferManager::batch_update (wave_buffer_cpu.cpp:190-257 and :102-188) in one launch, one
+ * workgroup per group, with no host round trip, for a host-resident cluster store.
+ *   ret_ids [BG, np] int32: retrieved cluster ids in rank order (from ri_score_select)
+ *   sizes, starts [BG, meta_stride] int32: tokens and first host-store row of every cluster
+ *   blk_off [BG, blk_off_stride] int32: exclusive prefix of ceil(size / block), ncl + 1 entries
+ * State, all device memory owned by the caller and only touched by this call:
+ *   stamp [BG, stamp_stride] int32 (zero-initialised: nothing resident), blk_ids
+ *   [BG, blk_ids_stride] int32 (cache block ids of resident clusters at blk_off),
+ *   free_list [BG, capacity] int32 (initialised 0..capacity-1), free_count [BG] (= capacity),
+ *   epoch [BG] (= 0).
+ * Output lists [BG, buffer_size] int32 and counts [BG], in the layout ri_gather_copy_and_concat
+ * and ri_gather_copy_and_scatter read: hit (cache block id, size, token offset), miss (host row,
+ * size, token offset), update (execution-buffer token offset, size, cache block id).
+ * Policy: the walk over the ranks stops at the first cluster whose blocks do not fit
+ * buffer_size; the longest prefix of the misses that fits `capacity` is admitted; victims are
+ * whole clusters, least recently touched step first, ascending id inside a step, never one
+ * touched in this call.  np <= 1023, ncl <= 65536. */
+int ri_lru_access_update(const int32_t* ret_ids, const int32_t* sizes, const int32_t* starts,
+                         int meta_stride, const int32_t* blk_off, int blk_off_stride, int32_t* stamp,
+                         int stamp_stride, int32_t* blk_ids, int blk_ids_stride, int32_t* free_list,
+                         int32_t* free_count, int32_t* epoch, int32_t* hit_ids, int32_t* hit_sizes,
+                         int32_t* hit_cumsum, int32_t* hit_num, int32_t* miss_ids,
+                         int32_t* miss_sizes, int32_t* miss_cumsum, int32_t* miss_num,
+                         int32_t* upd_buf, int32_t* upd_sizes, int32_t* upd_cache, int32_t* upd_num,
+                         int BG, int np, int ncl, int buffer_size, int capacity, int block,
+                         ri_stream_t stream);
+
 /* Device-side replacement of WaveBufferCPU::organize_kv (wave_buffer_cpu.cpp:545-567):
  * out[p, i, :] = in[p, members[p, i], :] — K/V rows permuted into cluster-contiguous order. */
 int ri_permute_rows(const void* in, const int32_t* members, void* out, int P, int N,

@@ -6,6 +6,7 @@ update); the copy functions are the loop oracles of
 library/retroinfer/test/test_gather_copy.py (:110-127, :190-194, :233-237).
 Block ids: the reference takes them from an unordered_set (iteration order unspecified,
 :153-156); this model hands out the lowest free id last released first, like the library.
+DeviceLruModel restates the policy of the device-side manager, which is this build's own.
 """
 import torch
 
@@ -82,6 +83,100 @@ class LruModel:
         self.hit_keys, self.miss_keys = [], []
         return upd
 
+
+
+class DeviceLruModel:
+    """The block cache policy of the device-side manager (csrc/lru.hip), one group, plain Python.
+    Same access walk and admission prefix as LruModel; recency is the number of the last step that
+    touched a cluster; victims are whole clusters, oldest step first (ages of 255 steps and more
+    count alike), ascending id inside the boundary age, never one touched in the current step, and
+    an admission the victims cannot cover is cut short.  Freed ids are appended to the free list
+    in ascending cluster id; admitted clusters take ids off the end of the list in rank order."""
+    AGES = 256
+
+    def __init__(self, sizes, block, capacity, buffer_size):
+        self.block, self.capacity, self.buffer_size = block, capacity, buffer_size
+        self.sizes = [int(s) for s in sizes]
+        self.start, row = [], 0
+        for s_ in self.sizes:
+            self.start.append(row)
+            row += s_
+        self.nblk = [(s_ + block - 1) // block for s_ in self.sizes]
+        self.stamp = [0] * len(self.sizes)
+        self.blocks = {}                       # resident cluster -> block ids
+        self.free = list(range(capacity))
+        self.epoch = 0
+
+    def _blocks(self, c):
+        n = self.nblk[c]
+        return [self.block] * (n - 1) + [self.sizes[c] - (n - 1) * self.block] if n else []
+
+    def step(self, ids):
+        """Returns (hit, miss, update) lists of (index, size, offset) triples like LruModel."""
+        E = self.epoch + 1
+        hit, miss, hits, misses = [], [], [], []
+        pages = hs = ms = 0
+        for c in ids:
+            c = int(c)
+            if c < 0 or c >= len(self.sizes):
+                continue
+            pages += self.nblk[c]
+            if pages > self.buffer_size:
+                break
+            if self.nblk[c] == 0:
+                continue
+            if self.stamp[c] != 0:
+                hits.append(c)
+                for bid, sz in zip(self.blocks[c], self._blocks(c)):
+                    hit.append((bid, sz, hs)); hs += sz
+            else:
+                misses.append((c, ms))
+                row = self.start[c]
+                for sz in self._blocks(c):
+                    miss.append((row, sz, ms)); ms += sz; row += self.block
+        for c in hits:
+            self.stamp[c] = E
+        admit, need = [], 0
+        for c, off in misses:
+            if need + self.nblk[c] > self.capacity:
+                break
+            need += self.nblk[c]; admit.append((c, off))
+        to_free = need - len(self.free)
+        if to_free > 0:
+            age = lambda c: min(E - self.stamp[c], self.AGES - 1)
+            cand = [c for c in range(len(self.sizes)) if self.stamp[c] not in (0, E)]
+            hist = [0] * self.AGES
+            for c in cand:
+                hist[age(c)] += self.nblk[c]
+            acc, cut = 0, -1
+            for a in range(self.AGES - 1, 0, -1):
+                if acc + hist[a] >= to_free:
+                    cut = a
+                    break
+                acc += hist[a]
+            rem, run = to_free - acc, 0
+            for c in cand:                      # ascending id
+                out = cut < 0 or age(c) > cut
+                if age(c) == cut:
+                    out = run < rem
+                    run += self.nblk[c]
+                if out:
+                    self.free.extend(self.blocks.pop(c))
+                    self.stamp[c] = 0
+        F = len(self.free)
+        upd, taken = [], 0
+        for c, off in admit:
+            if taken + self.nblk[c] > F:
+                break
+            ids_c = [self.free[F - 1 - (taken + j)] for j in range(self.nblk[c])]
+            for j, (b, sz) in enumerate(zip(ids_c, self._blocks(c))):
+                upd.append((b, sz, off + j * self.block))
+            self.blocks[c] = ids_c
+            self.stamp[c] = E
+            taken += self.nblk[c]
+        del self.free[F - taken:]
+        self.epoch = E
+        return hit, miss, upd
 
 def gather_copy_vectors(src_k, src_v, src_m, idx, copy_start, copy_num):
     """test_gather_copy.py:233-237."""

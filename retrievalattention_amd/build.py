@@ -12,7 +12,7 @@ from concurrent.futures import ThreadPoolExecutor
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libretro_mi355.so")
-HIP_SOURCES = ["capi.hip", "score.hip", "select.hip", "attend.hip", "gather.hip", "kmeans.hip"]
+HIP_SOURCES = ["capi.hip", "score.hip", "select.hip", "attend.hip", "gather.hip", "kmeans.hip", "lru.hip"]
 CPP_SOURCES = ["wavebuf.cpp"]
 ARCH = "gfx950"
 # -ffp-contract=off: products and sums round separately unless the source says fmaf, which

@@ -1,0 +1,245 @@
+// Device-side block cache manager for a host-resident cluster store (gfx950).
+//
+// Does on the GPU, in one launch and without a host round trip, what the reference does on CPU
+// worker threads between the top-k search and the gather:
+//   BufferManager::batch_access  (library/retroinfer/retroinfer_kernels/src/wave_buffer_cpu.cpp:190-257)
+//     walk the retrieved clusters in rank order, stop when their blocks no longer fit the
+//     execution buffer, emit the hit list (cache block ids) and the miss list (host rows);
+//   BufferManager::batch_update  (wave_buffer_cpu.cpp:102-188)
+//     touch the hits, admit the longest prefix of the misses that fits the cache, evict
+//     least-recently-used clusters until enough blocks are free, hand out block ids, emit the
+//     admission list for the scatter kernel.
+// The lists have the layout the copy kernels of gather.hip read.
+//
+// Recency is kept per cluster as the number of the last step that touched it.  Eviction takes
+// whole clusters, oldest step first and ascending cluster id inside the boundary step, until the
+// request is covered; clusters touched in the current step are never evicted, so an admission
+// that cannot be covered is cut short instead.  (The reference keeps a linked list in touch
+// order; which of several equally old clusters goes first is the only observable difference,
+// and nothing downstream depends on it: hits and misses deliver the same bytes.)
+#include "ri_common.h"
+
+#define LRU_THREADS 1024
+#define LRU_WAVES (LRU_THREADS / 64)
+#define LRU_AGES 256
+
+struct LruParams {
+  const int32_t* ret_ids;   // [BG, np] cluster ids in rank order
+  const int32_t* sizes;     // [BG, meta_stride] tokens per cluster
+  const int32_t* starts;    // [BG, meta_stride] first row of the cluster in the host store
+  const int32_t* blk_off;   // [BG, blk_off_stride] exclusive prefix of ceil(size / block)
+  int32_t* stamp;           // [BG, stamp_stride] 0 = not resident, else last step that touched it
+  int32_t* blk_ids;         // [BG, blk_ids_stride] cache block ids of resident clusters, at blk_off
+  int32_t* free_list;       // [BG, capacity] free block ids, the first free_count are valid
+  int32_t* free_count;      // [BG]
+  int32_t* epoch;           // [BG] step counter
+  int32_t *hit_ids, *hit_sizes, *hit_cumsum, *hit_num;
+  int32_t *miss_ids, *miss_sizes, *miss_cumsum, *miss_num;
+  int32_t *upd_buf, *upd_sizes, *upd_cache, *upd_num;
+  int np, ncl, meta_stride, blk_off_stride, stamp_stride, blk_ids_stride, buffer_size, capacity, block;
+};
+
+// exclusive prefix sums of N values over the 1024 threads; totals in tot
+template <int N>
+__device__ __forceinline__ void lru_scan(const int (&v)[N], int (&pre)[N], int (&tot)[N], int* sh) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  int inc[N];
+#pragma unroll
+  for (int k = 0; k < N; ++k) {
+    inc[k] = v[k];
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+      const int o = __shfl_up(inc[k], d);
+      if (lane >= d) inc[k] += o;
+    }
+    if (lane == 63) sh[k * LRU_WAVES + wave] = inc[k];
+  }
+  __syncthreads();
+#pragma unroll
+  for (int k = 0; k < N; ++k) {
+    int woff = 0, t = 0;
+#pragma unroll
+    for (int w = 0; w < LRU_WAVES; ++w) {
+      const int x = sh[k * LRU_WAVES + w];
+      if (w < wave) woff += x;
+      t += x;
+    }
+    pre[k] = woff + inc[k] - v[k];
+    tot[k] = t;
+  }
+  __syncthreads();
+}
+
+__global__ __launch_bounds__(LRU_THREADS) void lru_kernel(LruParams P) {
+  __shared__ int sh_scan[4 * LRU_WAVES];
+  __shared__ int sh_hist[LRU_AGES];
+  __shared__ int sh_cut[2];  // boundary age, blocks freed by strictly older clusters
+  const int g = blockIdx.x;
+  const int tid = threadIdx.x;
+  const int block = P.block;
+  const int32_t* sizes = P.sizes + (size_t)g * P.meta_stride;
+  const int32_t* starts = P.starts + (size_t)g * P.meta_stride;
+  const int32_t* boff = P.blk_off + (size_t)g * P.blk_off_stride;
+  int32_t* stamp = P.stamp + (size_t)g * P.stamp_stride;
+  int32_t* bids = P.blk_ids + (size_t)g * P.blk_ids_stride;
+  int32_t* flist = P.free_list + (size_t)g * P.capacity;
+  const size_t lo = (size_t)g * P.buffer_size;
+  const int E = P.epoch[g] + 1;
+  const int F0 = P.free_count[g];
+
+  // ---- access: thread r looks at the cluster of rank r ----
+  int c = -1, nb = 0, sz = 0;
+  if (tid < P.np) {
+    c = P.ret_ids[(size_t)g * P.np + tid];
+    if (c < 0 || c >= P.ncl) {
+      c = -1;
+    } else {
+      sz = sizes[c];
+      nb = (sz + block - 1) / block;
+    }
+  }
+  int v1[1] = {nb}, p1[1], t1[1];
+  lru_scan<1>(v1, p1, t1, sh_scan);
+  // the walk stops at the first cluster whose blocks no longer fit: everything after it is dropped
+  const bool keep = c >= 0 && nb > 0 && p1[0] + nb <= P.buffer_size;
+  const bool hit = keep && stamp[c] != 0;
+  const bool miss = keep && !hit;
+  int v4[4] = {hit ? nb : 0, hit ? sz : 0, miss ? nb : 0, miss ? sz : 0}, p4[4], t4[4];
+  lru_scan<4>(v4, p4, t4, sh_scan);
+  // the longest prefix of the misses whose blocks fit the whole cache may be admitted
+  bool adm = miss && p4[2] + nb <= P.capacity;
+  int va[1] = {adm ? nb : 0}, pa[1], ta[1];
+  lru_scan<1>(va, pa, ta, sh_scan);
+  const int need = ta[0];
+
+  if (hit) {
+    const int32_t* ids = bids + boff[c];
+    for (int j = 0; j < nb; ++j) {
+      P.hit_ids[lo + p4[0] + j] = ids[j];
+      P.hit_sizes[lo + p4[0] + j] = (j == nb - 1) ? sz - (nb - 1) * block : block;
+      P.hit_cumsum[lo + p4[0] + j] = p4[1] + j * block;
+    }
+    stamp[c] = E;
+  }
+  if (miss) {
+    const int row = starts[c];
+    for (int j = 0; j < nb; ++j) {
+      P.miss_ids[lo + p4[2] + j] = row + j * block;
+      P.miss_sizes[lo + p4[2] + j] = (j == nb - 1) ? sz - (nb - 1) * block : block;
+      P.miss_cumsum[lo + p4[2] + j] = p4[3] + j * block;
+    }
+  }
+  if (tid == 0) {
+    P.hit_num[g] = t4[0];
+    P.miss_num[g] = t4[2];
+  }
+  if (tid < LRU_AGES) sh_hist[tid] = 0;
+  __syncthreads();  // the hits carry this step's stamp before anybody looks for victims
+
+  // ---- eviction: free (need - F0) blocks from the oldest clusters ----
+  const int to_free = need - F0;  // uniform
+  int F = F0;
+  if (to_free > 0) {
+    // thread t owns the ids [t*K, t*K + K): id order inside the boundary age comes out of a prefix sum
+    const int K = (P.ncl + LRU_THREADS - 1) / LRU_THREADS;
+    const int c0 = tid * K, c1 = min(P.ncl, c0 + K);
+    for (int cc = c0; cc < c1; ++cc) {
+      const int st = stamp[cc];
+      if (st != 0 && st != E) atomicAdd(&sh_hist[min(E - st, LRU_AGES - 1)], boff[cc + 1] - boff[cc]);
+    }
+    __syncthreads();
+    if (tid == 0) {
+      int acc = 0, cut = -1;
+      for (int a = LRU_AGES - 1; a >= 1; --a) {
+        if (acc + sh_hist[a] >= to_free) { cut = a; break; }
+        acc += sh_hist[a];
+      }
+      sh_cut[0] = cut;  // -1: even every untouched cluster does not cover the request
+      sh_cut[1] = acc;
+    }
+    __syncthreads();
+    const int cut = sh_cut[0];
+    const int rem = to_free - sh_cut[1];  // blocks still wanted from the boundary age
+    int tie = 0;
+    for (int cc = c0; cc < c1; ++cc) {
+      const int st = stamp[cc];
+      if (st != 0 && st != E && min(E - st, LRU_AGES - 1) == cut) tie += boff[cc + 1] - boff[cc];
+    }
+    int vt[1] = {tie}, pt[1], tt[1];
+    lru_scan<1>(vt, pt, tt, sh_scan);
+    int run = pt[0], ev = 0;
+    uint64_t ev_bits = 0;  // K <= 64 ids per thread
+    for (int cc = c0; cc < c1; ++cc) {
+      const int st = stamp[cc];
+      if (st == 0 || st == E) continue;
+      const int age = min(E - st, LRU_AGES - 1);
+      const int nbc = boff[cc + 1] - boff[cc];
+      bool out = cut < 0 || age > cut;
+      if (age == cut) {
+        out = run < rem;
+        run += nbc;
+      }
+      if (out) {
+        ev_bits |= 1ull << (cc - c0);
+        ev += nbc;
+      }
+    }
+    int ve[1] = {ev}, pe[1], te[1];
+    lru_scan<1>(ve, pe, te, sh_scan);
+    int w = F0 + pe[0];
+    for (int cc = c0; cc < c1; ++cc) {
+      if (!((ev_bits >> (cc - c0)) & 1ull)) continue;
+      const int nbc = boff[cc + 1] - boff[cc];
+      for (int j = 0; j < nbc; ++j) flist[w++] = bids[boff[cc] + j];
+      stamp[cc] = 0;
+    }
+    F = F0 + te[0];
+    __syncthreads();  // the freed ids are in the list before they are handed out
+  }
+
+  // ---- admission: block ids come off the end of the free list in rank order ----
+  adm = adm && pa[0] + nb <= F;  // cut short if the untouched clusters did not cover the request
+  int vb[1] = {adm ? nb : 0}, pb[1], tb[1];
+  lru_scan<1>(vb, pb, tb, sh_scan);
+  if (adm) {
+    int32_t* ids = bids + boff[c];
+    for (int j = 0; j < nb; ++j) {
+      const int id = flist[F - 1 - (pa[0] + j)];
+      ids[j] = id;
+      P.upd_cache[lo + pa[0] + j] = id;
+      P.upd_sizes[lo + pa[0] + j] = (j == nb - 1) ? sz - (nb - 1) * block : block;
+      P.upd_buf[lo + pa[0] + j] = p4[3] + j * block;  // admitted misses lead the miss list
+    }
+    stamp[c] = E;
+  }
+  if (tid == 0) {
+    P.upd_num[g] = tb[0];
+    P.free_count[g] = F - tb[0];
+    P.epoch[g] = E;
+  }
+}
+
+extern "C" int ri_lru_access_update(const int32_t* ret_ids, const int32_t* sizes, const int32_t* starts,
+                                    int meta_stride, const int32_t* blk_off, int blk_off_stride, int32_t* stamp,
+                                    int stamp_stride, int32_t* blk_ids, int blk_ids_stride, int32_t* free_list,
+                                    int32_t* free_count, int32_t* epoch, int32_t* hit_ids, int32_t* hit_sizes,
+                                    int32_t* hit_cumsum, int32_t* hit_num, int32_t* miss_ids, int32_t* miss_sizes,
+                                    int32_t* miss_cumsum, int32_t* miss_num, int32_t* upd_buf, int32_t* upd_sizes,
+                                    int32_t* upd_cache, int32_t* upd_num, int BG, int np, int ncl, int buffer_size,
+                                    int capacity, int block, ri_stream_t stream) {
+  if (!ret_ids || !sizes || !starts || !blk_off || !stamp || !blk_ids || !free_list || !free_count || !epoch ||
+      !hit_ids || !hit_sizes || !hit_cumsum || !hit_num || !miss_ids || !miss_sizes || !miss_cumsum || !miss_num ||
+      !upd_buf || !upd_sizes || !upd_cache || !upd_num)
+    return RI_ERR_ARG;
+  if (BG <= 0 || np <= 0 || np > LRU_THREADS - 1 || ncl <= 0 || ncl > 64 * LRU_THREADS || buffer_size <= 0 ||
+      capacity <= 0 || block <= 0)
+    return RI_ERR_ARG;
+  if (meta_stride < ncl || blk_off_stride < ncl + 1 || stamp_stride < ncl || blk_ids_stride <= 0) return RI_ERR_ARG;
+  LruParams P = {ret_ids, sizes, starts, blk_off, stamp, blk_ids, free_list, free_count, epoch,
+                 hit_ids, hit_sizes, hit_cumsum, hit_num, miss_ids, miss_sizes, miss_cumsum, miss_num,
+                 upd_buf, upd_sizes, upd_cache, upd_num,
+                 np, ncl, meta_stride, blk_off_stride, stamp_stride, blk_ids_stride, buffer_size, capacity, block};
+  lru_kernel<<<BG, LRU_THREADS, 0, (hipStream_t)stream>>>(P);
+  RI_HIP_CHECK_LAUNCH();
+  return RI_OK;
+}

@@ -281,6 +281,38 @@ def buffer_attention(q, buf_k, buf_v, cache_seqlens, est_ids, logits, value_sum,
                                     float(scale), _p(ws), ws.numel(), _stream()), "buffer_attention")
 
 
+class DeviceLru:
+    """State of the device-side block cache manager of one layer (ri_lru_access_update)."""
+
+    def __init__(self, BG, max_clusters, max_blocks, capacity, buffer_size, block, device):
+        i32 = lambda *s: torch.zeros(s, dtype=torch.int32, device=device)
+        self.BG, self.capacity, self.buffer_size, self.block = BG, capacity, buffer_size, block
+        self.stamp = i32(BG, max_clusters)
+        self.blk_off = i32(BG, max_clusters + 1)
+        self.blk_ids = i32(BG, max_blocks)
+        self.free_list = torch.arange(capacity, dtype=torch.int32, device=device).repeat(BG, 1).contiguous()
+        self.free_count = torch.full((BG,), capacity, dtype=torch.int32, device=device)
+        self.epoch = i32(BG)
+
+    def set_sizes(self, sizes_i32):
+        """sizes_i32 [BG, ncl]: recompute the block offsets (offsets of existing clusters do not move
+        when clusters are appended)."""
+        nb = (sizes_i32.to(torch.int64) + self.block - 1) // self.block
+        ncl = sizes_i32.shape[1]
+        self.blk_off[:, 1:ncl + 1] = torch.cumsum(nb, 1).to(torch.int32)
+        assert int(self.blk_off[:, ncl].max()) <= self.blk_ids.shape[1]
+
+    def access_update(self, ret_ids, sizes, starts, lists):
+        """lists: the 12 tensors hit (ids, sizes, cumsum, num), miss (...), update (buf, sizes, cache, num)."""
+        BG, np_ = ret_ids.shape
+        ncl = sizes.shape[1]
+        check(lib().ri_lru_access_update(
+            _p(ret_ids), _p(sizes), _p(starts), sizes.stride(0), _p(self.blk_off), self.blk_off.shape[1],
+            _p(self.stamp), self.stamp.shape[1], _p(self.blk_ids), self.blk_ids.shape[1], _p(self.free_list),
+            _p(self.free_count), _p(self.epoch), *[_p(t) for t in lists], BG, np_, ncl, self.buffer_size,
+            self.capacity, self.block, _stream()), "lru_access_update")
+
+
 def kmeans_assign(data, centroids, assign, P, N, nc, seg, head_rows):
     check(lib().ri_kmeans_assign(_p(data), _p(centroids), _p(assign), P, N, nc, seg, head_rows, _stream()),
           "kmeans_assign")

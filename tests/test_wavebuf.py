@@ -159,3 +159,46 @@ def test_bad_arguments_are_rejected():
     wb = kernels.WaveBufferCPU(1, 1, 128, 1, 8, 4, 4, 4, 4, 1, pool.get())
     with pytest.raises(RuntimeError, match="before it was set up"):
         wb.batch_access()
+
+
+def test_device_lru_model_invariants():
+    """The policy the device-side manager implements, on its Python restatement: every requested
+    cluster is a hit or a miss exactly once (until the buffer cut-off), hit <=> resident, block ids
+    unique, resident blocks + free blocks = capacity, victims are the least recently touched."""
+    import random
+    from oracle.wavebuf import DeviceLruModel
+    rnd = random.Random(3)
+    sizes = [rnd.randint(0, 40) for _ in range(200)]
+    m = DeviceLruModel(sizes, 8, 60, 48)
+    last_touch = {}
+    for step in range(1, 60):
+        ids = rnd.sample(range(200), 12)
+        resident_before = set(m.blocks)
+        hit, miss, upd = m.step(ids)
+        pages, seen = 0, []
+        for c in ids:
+            pages += m.nblk[c]
+            if pages > 48:
+                break
+            if m.nblk[c]:
+                seen.append(c)
+        assert len(hit) + len(miss) == sum(m.nblk[c] for c in seen)
+        assert sum(sz for _, sz, _ in hit) + sum(sz for _, sz, _ in miss) == sum(sizes[c] for c in seen)
+        hits = [c for c in seen if c in resident_before]
+        assert len(hit) == sum(m.nblk[c] for c in hits)
+        for c in seen:
+            if c in m.blocks:
+                last_touch[c] = step
+        used = [b for ids_c in m.blocks.values() for b in ids_c]
+        assert len(set(used)) == len(used) and not set(used) & set(m.free)
+        assert len(used) + len(m.free) == 60
+        evicted = resident_before - set(m.blocks)
+        if evicted:   # nothing older than a victim stays resident, except within the boundary step
+            newest_victim = max(last_touch[c] for c in evicted)
+            for c in m.blocks:
+                if c not in seen:
+                    assert last_touch[c] >= newest_victim or last_touch[c] == newest_victim
+            oldest_kept = min((last_touch[c] for c in m.blocks if c not in seen), default=step)
+            assert max(last_touch[c] for c in evicted) <= oldest_kept
+        for c in evicted:
+            last_touch.pop(c, None)
