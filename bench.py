@@ -44,7 +44,7 @@ def log(*a):
     print(*a, file=sys.stderr, flush=True)
 
 
-def build_cache(cfg, L, dev, residency="device"):
+def build_cache(cfg, L, dev, residency="device", block_cache="device"):
     from retrievalattention_amd import synth
     from retrievalattention_amd.cache_hub import retroinfer_cache
     B, Hkv, gs, N = cfg["B"], cfg["Hkv"], cfg["gs"], cfg["N"]
@@ -57,7 +57,8 @@ def build_cache(cfg, L, dev, residency="device"):
         num_heads=Hkv * gs, head_dim=128, dtype=torch.bfloat16, layer_mapping={str(l): "cuda:0" for l in range(L)},
         max_new_length=new, static_pattern_start=synth.STEADY_START, static_pattern_end=synth.STEADY_END, core=8,
         n_centroids=cfg["nc"], n_segment=cfg["S"], nprobe=nprobe, max_compute_cluster_num=nprobe + es,
-        cache_unit_size=8, cache_cluster_num=3 * nprobe, num_gpus=1, model_size=0, kv_residency=residency)
+        cache_unit_size=8, cache_cluster_num=3 * nprobe, num_gpus=1, model_size=0, kv_residency=residency,
+        block_cache=block_cache)
     queries = []
     t0 = time.time()
     for l in range(L):
@@ -188,12 +189,23 @@ def bench_host(args, cfg, cache, queries, L, nprobe, es, static_len):
         step(l)
     torch.cuda.synchronize()
     t_cold = (time.perf_counter() - t0) / L
+    use_graph = cache.block_cache == "device" and not args.no_graph
+    if use_graph:   # the device-side manager has no host round trip: the whole step replays as a HIP graph
+        graphs = []
+        for l in range(L):
+            gr = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(gr):
+                step(l)
+            graphs.append(gr)
+        run = lambda i: graphs[i % L].replay()
+    else:
+        run = lambda i: step(i % L)
     for i in range(args.warmup):
-        step(i % L)
+        run(i)
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     for i in range(args.steps):
-        step(i % L)
+        run(i)
     torch.cuda.synchronize()
     t_warm = (time.perf_counter() - t0) / args.steps
     miss = sum(int(cache.miss_num_units[l].sum()) for l in range(L))
@@ -205,7 +217,8 @@ def bench_host(args, cfg, cache, queries, L, nprobe, es, static_len):
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
         "config": {"workload": f"{args.config}: {cfg['desc']}; clustered K/V in pinned host memory, block cache of "
                                f"{cache.cache_size if hasattr(cache, 'cache_size') else '?'} blocks per group, "
-                               f"nprobe {nprobe}, estimation zone {es}, {L} layers, eager launches, warm = same "
+                               f"block cache manager on the {cache.block_cache}, nprobe {nprobe}, estimation zone {es}, {L} layers, "
+                               f"{'HIP graph replay' if use_graph else 'eager launches'}, warm = same "
                                f"queries repeated", "batch": B, "context_tokens": cfg["N"],
                    "layers_for_tokens_per_s": cfg["L"], "warm_hit_blocks": hit, "warm_miss_blocks": miss},
         "roofline": None, "cpu_baseline": None}))
@@ -223,6 +236,9 @@ def main():
     ap.add_argument("--residency", default="device", choices=["device", "host"],
                     help="host: clustered K/V in pinned host memory behind the block cache (staged operator path, "
                          "eager launches; reports the cold first pass and the warm steady state)")
+    ap.add_argument("--block-cache", default="device", choices=["device", "host"],
+                    help="with --residency host: block cache manager as a kernel (HIP graph replays) or the "
+                         "reference's worker threads (eager launches)")
     ap.add_argument("--no-kmeans", action="store_true", help="skip the prefill clustering measurement")
     ap.add_argument("--copy-probe", action="store_true",
                     help="also run 8 device copies of 256 MiB (a known-size kernel to scale rocprofv3 byte counters by)")
@@ -244,7 +260,7 @@ def main():
             b.copy_(a)
         torch.cuda.synchronize()
         del a, b
-    cache, queries, nprobe, es = build_cache(cfg, L, dev, args.residency)
+    cache, queries, nprobe, es = build_cache(cfg, L, dev, args.residency, args.block_cache)
     static_len = cache.static_pattern_total  # 4 + 64 + the token being decoded (already counted)
     if args.residency == "host":
         return bench_host(args, cfg, cache, queries, L, nprobe, es, static_len)

@@ -37,7 +37,8 @@ class retroinfer_cache(KV_Cache):
     def __init__(self, valid_start, layer_num, batch_size, max_length, num_key_value_heads, num_heads,
                  head_dim, dtype, layer_mapping, max_new_length, static_pattern_start, static_pattern_end, core,
                  n_centroids, n_segment, nprobe, max_compute_cluster_num, cache_unit_size, cache_cluster_num,
-                 num_gpus, model_size, use_cluster_estimation=False, kv_residency="auto"):
+                 num_gpus, model_size, use_cluster_estimation=False, kv_residency="auto",
+                 block_cache="device"):
         super().__init__(layer_num, batch_size, max_length, num_key_value_heads, num_heads, head_dim, dtype,
                          layer_mapping, num_gpus, model_size)
         if head_dim != 128 or dtype != torch.bfloat16:
@@ -53,6 +54,11 @@ class retroinfer_cache(KV_Cache):
         self.page_size = cache_unit_size
         self.core = core
         self.use_cluster_estimation = use_cluster_estimation
+        if block_cache not in ("device", "host"):
+            raise ValueError("block_cache must be 'device' or 'host'")
+        # who runs the block cache of a host-resident store: a kernel (no host round trip per step) or
+        # the reference's worker threads (WaveBufferCPU.batch_access / sync)
+        self.block_cache = block_cache
 
         self.input_length = self.max_length - max_new_length
         self.max_new_length = min(max_new_length - 1, THRESHOLD_LENGTH)  # one token comes out of prefill
@@ -100,6 +106,10 @@ class retroinfer_cache(KV_Cache):
             self.offload_update_keys = _pinned((BG, THRESHOLD_LENGTH, D), dtype)
             self.offload_update_values = _pinned((BG, THRESHOLD_LENGTH, D), dtype)
 
+        # per cluster: first row in the (device or host) store and token count
+        self.cluster_start = [zeros((BG, n_centroids), torch.int32, dev(l)) for l in L]
+        self.cluster_size_i32 = [zeros((BG, n_centroids), torch.int32, dev(l)) for l in L]
+        self.store_rows = [[0] * BG for _ in L]  # rows of the store in use, per group
         if self.kv_residency == "device":
             self._init_device_store()
         else:
@@ -121,13 +131,10 @@ class retroinfer_cache(KV_Cache):
         shape = (self.batch_size, self.kv_head, self.list_stride, D)
         self.list_keys = [torch.zeros(shape, dtype=self.dtype, device=dev(l)) for l in L]
         self.list_values = [torch.zeros(shape, dtype=self.dtype, device=dev(l)) for l in L]
-        # per cluster: first row in the store and token count
-        self.cluster_start = [torch.zeros((BG, self.n_centroids), dtype=torch.int32, device=dev(l)) for l in L]
-        self.cluster_size_i32 = [torch.zeros((BG, self.n_centroids), dtype=torch.int32, device=dev(l)) for l in L]
-        self.store_rows = [[0] * BG for _ in L]  # rows of the store in use, per group
 
     def _init_wave_buffer(self):
         dev = lambda ldx: self.layer_mapping[str(ldx)]
+        zeros = lambda shape, dt, d: torch.zeros(shape, dtype=dt, device=d)
         BG, D = self.batch_groups, self.head_dim
         L = range(self.layer_num)
         self.thread_pool = kernels.ThreadPool(self.core)
@@ -141,13 +148,28 @@ class retroinfer_cache(KV_Cache):
             setattr(self, nm, [_pinned((BG, self.buffer_size), torch.int32, 0) for _ in L])
         for nm in ("hit_num_units", "miss_num_units", "update_num_units"):
             setattr(self, nm, [_pinned((BG,), torch.int32, 0) for _ in L])
+        self._host_lists = None
+        if self.block_cache == "device":
+            # the worker-thread manager keeps its (unused) pinned lists; the copy kernels read these instead
+            self._host_lists = {nm: getattr(self, nm) for nm in names + ["hit_num_units", "miss_num_units",
+                                                                         "update_num_units"]}
+            for nm in names:
+                setattr(self, nm, [zeros((BG, self.buffer_size), torch.int32, dev(l)) for l in L])
+            for nm in ("hit_num_units", "miss_num_units", "update_num_units"):
+                setattr(self, nm, [zeros((BG,), torch.int32, dev(l)) for l in L])
+            max_blocks = self.list_stride // self.page_size + self.n_centroids + self.n_centroids_new + 1
+            self.device_lru = [kernels.DeviceLru(BG, self.n_centroids + self.n_centroids_new, max_blocks,
+                                                 self.cache_size, self.buffer_size, self.page_size, dev(l)) for l in L]
         self.cluster_ids = [_pinned((BG, self.nprobe), torch.int64, 0) for _ in range(2)]
         for l in L:
+            hl = self._host_lists if self._host_lists is not None else {nm: getattr(self, nm) for nm in names + [
+                "hit_num_units", "miss_num_units", "update_num_units"]}
             self.wave_buffer[l].set_indices(
-                self.hit_unit_idices[l], self.hit_unit_sizes[l], self.hit_unit_sizes_cumsum[l], self.hit_num_units[l],
-                self.miss_unit_idices[l], self.miss_unit_sizes[l], self.miss_unit_sizes_cumsum[l],
-                self.miss_num_units[l], self.update_buffer_indices[l], self.update_unit_sizes[l],
-                self.update_cache_indices[l], self.update_num_units[l], self.cluster_ids[l % 2])
+                hl["hit_unit_idices"][l], hl["hit_unit_sizes"][l], hl["hit_unit_sizes_cumsum"][l],
+                hl["hit_num_units"][l], hl["miss_unit_idices"][l], hl["miss_unit_sizes"][l],
+                hl["miss_unit_sizes_cumsum"][l], hl["miss_num_units"][l], hl["update_buffer_indices"][l],
+                hl["update_unit_sizes"][l], hl["update_cache_indices"][l], hl["update_num_units"][l],
+                self.cluster_ids[l % 2])
         self.cache_keys = [torch.zeros((self.batch_size, self.kv_head, self.cache_size, self.page_size, D),
                                        dtype=self.dtype, device=dev(l)) for l in L]
         self.cache_values = [torch.zeros_like(self.cache_keys[l]) for l in L]
@@ -194,6 +216,9 @@ class retroinfer_cache(KV_Cache):
         torch.cuda.synchronize()
         if self.kv_residency == "host":
             self.wave_buffer[self.layer_num - 1].construction_sync()
+            if self.block_cache == "device":
+                for l in range(self.layer_num):
+                    self.device_lru[l].set_sizes(self.cluster_size_i32[l])
         self.clusters_cpu = self.cluster_size_cpu = None
         self.temp_keys = self.temp_values = None
 
@@ -239,16 +264,18 @@ class retroinfer_cache(KV_Cache):
         self.centroids_mask[layer_idx][rows].copy_(km.counts == 0)
         self.cluster_size[layer_idx][rows].copy_(km.counts.to(self.dtype))
 
+        # clusters sit in the store in id order, tokens ascending inside (device: permute below; host:
+        # WaveBufferCPU's organisation)
+        self.cluster_start[layer_idx][rows].copy_(km.offsets[:, :self.n_centroids])
+        self.cluster_size_i32[layer_idx][rows].copy_(km.counts)
+        for h in range(H):
+            self.store_rows[layer_idx][batch_idx * H + h] = valid_length
         if self.kv_residency == "device":
             # cluster-contiguous store built on the device (stands in for organize_kv on the host)
             lk = self.list_keys[layer_idx][batch_idx]
             lv = self.list_values[layer_idx][batch_idx]
             kernels.permute_rows(self.temp_keys, km.members, lk, H, valid_length, valid_length, self.list_stride)
             kernels.permute_rows(self.temp_values, km.members, lv, H, valid_length, valid_length, self.list_stride)
-            self.cluster_start[layer_idx][rows].copy_(km.offsets[:, :self.n_centroids])
-            self.cluster_size_i32[layer_idx][rows].copy_(km.counts)
-            for h in range(H):
-                self.store_rows[layer_idx][batch_idx * H + h] = valid_length
         else:
             self.cluster_size_cpu = km.counts.cpu().contiguous()
             self.clusters_cpu = csr_to_dense(km.counts, km.offsets, km.members).cpu().contiguous()
@@ -291,21 +318,23 @@ class retroinfer_cache(KV_Cache):
             self.value_sum[ldx] = torch.cat((self.value_sum[ldx], km.value_sum), dim=1)
             self.centroids_mask[ldx] = torch.cat((self.centroids_mask[ldx], km.counts == 0), dim=1)
             self.cluster_size[ldx] = torch.cat((self.cluster_size[ldx], km.counts.to(self.dtype)), dim=1)
+            base = self.store_rows[ldx][0]
+            self.cluster_start[ldx] = torch.cat((self.cluster_start[ldx], km.offsets[:, :ncu] + base), dim=1)
+            self.cluster_size_i32[ldx] = torch.cat((self.cluster_size_i32[ldx], km.counts), dim=1)
+            self.store_rows[ldx] = [base + THRESHOLD_LENGTH] * BG
             if self.kv_residency == "device":
-                base = self.store_rows[ldx][0]
                 assert base + THRESHOLD_LENGTH <= self.list_stride, "cluster store is full"
                 lk = self.list_keys[ldx].view(BG, self.list_stride, D)[:, base:]
                 lv = self.list_values[ldx].view(BG, self.list_stride, D)[:, base:]
                 kernels.permute_rows(uk, km.members, lk, BG, THRESHOLD_LENGTH, THRESHOLD_LENGTH, self.list_stride)
                 kernels.permute_rows(uv, km.members, lv, BG, THRESHOLD_LENGTH, THRESHOLD_LENGTH, self.list_stride)
-                self.cluster_start[ldx] = torch.cat((self.cluster_start[ldx], km.offsets[:, :ncu] + base), dim=1)
-                self.cluster_size_i32[ldx] = torch.cat((self.cluster_size_i32[ldx], km.counts), dim=1)
-                self.store_rows[ldx] = [base + THRESHOLD_LENGTH] * BG
             else:
                 self.copyevents[dkey].synchronize()
                 self.wave_buffer[ldx].update_kv(self.offload_update_keys, self.offload_update_values,
                                                 csr_to_dense(km.counts, km.offsets, km.members).cpu().contiguous(),
                                                 km.counts.cpu().contiguous())
+                if self.block_cache == "device":
+                    self.device_lru[ldx].set_sizes(self.cluster_size_i32[ldx])
         torch.cuda.set_device(self.layer_mapping[str(0)])
         self.n_centroids += ncu
         self.logits = torch.zeros((BG, self.group_size, self.n_centroids), dtype=torch.float32,
@@ -366,8 +395,22 @@ class retroinfer_cache(KV_Cache):
     # staged path: the reference's sequence of operators, one call each
     def _search(self, queries, layer, buf):
         self._select(queries, layer, buf, False)
-        if self.kv_residency == "host":
+        if self.kv_residency == "host" and self.block_cache == "host":
             self.cluster_ids[buf].copy_(self.cI[buf][:, :self.nprobe])  # blocking copy into pinned memory
+
+    def _lists(self, layer):
+        return [self.hit_unit_idices[layer], self.hit_unit_sizes[layer], self.hit_unit_sizes_cumsum[layer],
+                self.hit_num_units[layer], self.miss_unit_idices[layer], self.miss_unit_sizes[layer],
+                self.miss_unit_sizes_cumsum[layer], self.miss_num_units[layer], self.update_buffer_indices[layer],
+                self.update_unit_sizes[layer], self.update_cache_indices[layer], self.update_num_units[layer]]
+
+    def _access(self, layer, buf):
+        """Hit / miss / admission lists of the clusters chosen for `layer` (in buffer `buf`)."""
+        if self.block_cache == "device":
+            self.device_lru[layer].access_update(self.ret_ids[buf], self.cluster_size_i32[layer],
+                                                 self.cluster_start[layer], self._lists(layer))
+        else:
+            self.wave_buffer[layer].batch_access()
 
     def _assemble(self, layer, buf, static_len):
         if self.kv_residency == "host":
@@ -405,9 +448,9 @@ class retroinfer_cache(KV_Cache):
         else:
             es_out = es_lse = None
         if search_here:
-            self.wave_buffer[layer_idx].batch_access()
+            self._access(layer_idx, buf)
         if search_next:
-            self.wave_buffer[layer_idx + 1].batch_access()
+            self._access(layer_idx + 1, nbuf)
         if search_here:
             self._assemble(layer_idx, buf, static_len)
         if search_next:
@@ -428,7 +471,8 @@ class retroinfer_cache(KV_Cache):
             attn = kernels.weighted_flash_decoding(
                 q4, self.execution_buffer_keys[buf], self.execution_buffer_values[buf], previous_out=es_out,
                 previous_lse=es_lse, cache_seqlens=self.valid_lengths[buf])
-        self.wave_buffer[layer_idx].sync()
+        if self.block_cache == "host":
+            self.wave_buffer[layer_idx].sync()
         kernels.gather_copy_and_scatter(
             self.execution_buffer_keys[buf], self.cache_keys[layer_idx], self.execution_buffer_values[buf],
             self.cache_values[layer_idx], self.update_buffer_indices[layer_idx], self.update_unit_sizes[layer_idx],

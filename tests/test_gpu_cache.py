@@ -21,13 +21,18 @@ def _close(got, ref):
 def _make_cache(dev, residency, layers, B, Hkv, gs, ctx, n_centroids, n_segment, nprobe, es, new=8,
                 cache_cluster_num=None, use_cluster_estimation=False):
     from retrievalattention_amd.cache_hub import retroinfer_cache
+    # "host-cpu": host-resident store with the reference's worker-thread block cache manager;
+    # "host": the same store with the device-side manager
+    block_cache = "host" if residency == "host-cpu" else "device"
+    residency = "host" if residency == "host-cpu" else residency
     return retroinfer_cache(
         valid_start=[0] * B, layer_num=layers, batch_size=B, max_length=ctx + new, num_key_value_heads=Hkv,
         num_heads=Hkv * gs, head_dim=128, dtype=torch.bfloat16, layer_mapping={str(l): "cuda:0" for l in range(layers)},
         max_new_length=new, static_pattern_start=4, static_pattern_end=64, core=4, n_centroids=n_centroids,
         n_segment=n_segment, nprobe=nprobe, max_compute_cluster_num=nprobe + es, cache_unit_size=8,
         cache_cluster_num=cache_cluster_num if cache_cluster_num is not None else 3 * nprobe, num_gpus=1,
-        model_size=8, use_cluster_estimation=use_cluster_estimation, kv_residency=residency)
+        model_size=8, use_cluster_estimation=use_cluster_estimation, kv_residency=residency,
+        block_cache=block_cache)
 
 
 def _prefill(cache, K, V, layers, B):
@@ -49,7 +54,7 @@ def _gen(layers, B, Hkv, gs, ctx, nmix, dev, seed):
     return K, V
 
 
-@pytest.mark.parametrize("residency", ["device", "host"])
+@pytest.mark.parametrize("residency", ["device", "host", "host-cpu"])
 def test_decode_matches_oracle(dev, residency):
     """Prefill + three decode steps; every compute() is compared with the oracle's decode step
     run on the index the cache actually holds."""
@@ -135,14 +140,15 @@ def test_full_retrieval_equals_dense_attention(dev):
     _close(out.view(Hkv, gs, 128), ref)
 
 
-def test_host_and_device_residency_agree_and_cache_warms(dev):
+@pytest.mark.parametrize("host_kind", ["host", "host-cpu"])
+def test_host_and_device_residency_agree_and_cache_warms(dev, host_kind):
     """Same inputs through both residencies: identical selections, outputs within tolerance;
     repeated queries turn misses into hits in the LRU block cache."""
     layers, B, Hkv, gs, ctx = 1, 2, 2, 7, 3072 + 68
     nc, nprobe, es = 192, 6, 40
     K, V = _gen(layers, B, Hkv, gs, ctx, 192, dev, 5)
     cd = _make_cache(dev, "device", layers, B, Hkv, gs, ctx, nc, 1, nprobe, es)
-    ch = _make_cache(dev, "host", layers, B, Hkv, gs, ctx, nc, 1, nprobe, es)
+    ch = _make_cache(dev, host_kind, layers, B, Hkv, gs, ctx, nc, 1, nprobe, es)
     _prefill(cd, K, V, layers, B)
     _prefill(ch, K, V, layers, B)
     assert torch.equal(cd.centroids[0], ch.centroids[0])
@@ -161,9 +167,34 @@ def test_host_and_device_residency_agree_and_cache_warms(dev):
         assert torch.equal(cd.valid_lengths[0].cpu(), ch.valid_lengths[0].cpu())
         hits.append(int(ch.hit_num_units[0].sum()))
     assert hits[0] == 0 and hits[1] > 0 and hits[2] >= hits[1]
+    if host_kind == "host":
+        # device-side manager: what sits in the block cache is what the store holds for those clusters
+        lru, BG = ch.device_lru[0], B * Hkv
+        size = ch.cluster_size_i32[0].cpu()
+        start = ch.cluster_start[0].cpu()
+        stamp, boff, bids = lru.stamp.cpu(), lru.blk_off.cpu(), lru.blk_ids.cpu()
+        ck = ch.cache_keys[0].view(BG, -1, 8, 128).cpu()
+        cv = ch.cache_values[0].view(BG, -1, 8, 128).cpu()
+        lk, lv = ch.list_keys[0].view(BG, -1, 128), ch.list_values[0].view(BG, -1, 128)
+        checked = 0
+        for gi in range(BG):
+            used = []
+            for c in torch.nonzero(stamp[gi, :nc]).flatten().tolist():
+                n = int(size[gi, c])
+                ids = bids[gi, int(boff[gi, c]):int(boff[gi, c + 1])].tolist()
+                used += ids
+                got_k = ck[gi, ids].reshape(-1, 128)[:n]
+                got_v = cv[gi, ids].reshape(-1, 128)[:n]
+                r0 = int(start[gi, c])
+                assert torch.equal(got_k, lk[gi, r0:r0 + n]) and torch.equal(got_v, lv[gi, r0:r0 + n])
+                checked += 1
+            free = lru.free_list[gi, :int(lru.free_count[gi])].tolist()
+            assert len(set(used)) == len(used) and not set(used) & set(free)
+            assert len(used) + len(free) == ch.cache_size
+        assert checked > 0
 
 
-@pytest.mark.parametrize("residency", ["device", "host"])
+@pytest.mark.parametrize("residency", ["device", "host", "host-cpu"])
 def test_next_layer_cluster_estimation(dev, residency):
     """use_cluster_estimation (reference: retroinfer_cache.py:565, 582-595): layers 0 and 1 choose their
     zones from their own query; every later layer uses the zones the previous layer chose from a
