@@ -14,9 +14,17 @@ Every function cites the reference file:line it follows.  How each one is pinned
                                   (:110-127, :190-194, :233-237), bit-exact
   wavebuf.LruModel                brute-force list model + invariants (hit <=> resident, capacity,
                                   unique block ids, least-recently-touched eviction)
+  wavebuf.DeviceLruModel          the policy of the device-side block cache manager, which is this
+                                  build's own (the reference manages the cache on CPU threads):
+                                  invariants (every requested cluster once, hit <=> resident, unique
+                                  block ids, blocks conserved, victims not newer than survivors)
   kmeans.*                        brute force on tiny inputs in fp64, plus invariants (partition of
                                   the tokens, centroid*size = sum of keys, empty cluster keeps its
-                                  centroid, float32 init formula, remainder tokens)
+                                  centroid, float32 init formula, remainder tokens); the fixed
+                                  summation order of kmeans.cluster_sums (blocks of 256 tokens) by a
+                                  plain-loop restatement
+  pipeline.decode_step            composition of the above; with zone_logits, next-layer cluster
+                                  estimation (zones from a predicted query, retroinfer_cache.py:582-617)
   attention.weighted_flash_decoding   PARITY UNPINNED against the reference: the callee
                                   (github.com/Starmys/flash-attention, branch "weighted") is not in
                                   the reference tree and has no test there.  Semantics are inferred
