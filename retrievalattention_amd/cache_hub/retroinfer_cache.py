@@ -215,10 +215,12 @@ class retroinfer_cache(KV_Cache):
         """End of prefill (reference: retroinfer_cache.py:336-365)."""
         torch.cuda.synchronize()
         if self.kv_residency == "host":
-            self.wave_buffer[self.layer_num - 1].construction_sync()
-            if self.block_cache == "device":
+            if self.block_cache == "host":
+                self.wave_buffer[self.layer_num - 1].construction_sync()
+            else:
                 for l in range(self.layer_num):
                     self.device_lru[l].set_sizes(self.cluster_size_i32[l])
+                self.stage_keys = self.stage_values = None
         self.clusters_cpu = self.cluster_size_cpu = None
         self.temp_keys = self.temp_values = None
 
@@ -236,7 +238,10 @@ class retroinfer_cache(KV_Cache):
         rows = slice(batch_idx * H, (batch_idx + 1) * H)
         dkey = self.layer_mapping[str(layer_idx)]
 
-        if self.kv_residency == "host":
+        # host store filled by the worker threads (reference flow) or by a device permutation + one copy
+        cpu_organise = self.kv_residency == "host" and self.block_cache == "host"
+        dev_organise = self.kv_residency == "host" and self.block_cache == "device"
+        if cpu_organise:
             # the previous construction must have consumed the shared offload buffers
             prev = layer_idx - 1 if layer_idx > 0 else (self.layer_num - 1 if batch_idx > 0 else None)
             if prev is not None:
@@ -244,7 +249,7 @@ class retroinfer_cache(KV_Cache):
 
         self.temp_keys = key_states[0, vs + sps:seq_len - spe].transpose(0, 1).contiguous()      # [H, N, D]
         self.temp_values = value_states[0, vs + sps:seq_len - spe].transpose(0, 1).contiguous()
-        if self.kv_residency == "host":
+        if cpu_organise:
             self.mainevents[dkey].record()
             with torch.cuda.stream(self.copystream):
                 self.mainevents[dkey].wait()
@@ -276,6 +281,25 @@ class retroinfer_cache(KV_Cache):
             lv = self.list_values[layer_idx][batch_idx]
             kernels.permute_rows(self.temp_keys, km.members, lk, H, valid_length, valid_length, self.list_stride)
             kernels.permute_rows(self.temp_values, km.members, lv, H, valid_length, valid_length, self.list_stride)
+        elif dev_organise:
+            # the same permutation on the device into a staging buffer, then one copy per tensor into
+            # the pinned store on the copy stream (no host-side re-organisation, no dense cluster lists)
+            self.copyevents[dkey].synchronize()   # the previous copy has left the staging buffers
+            if getattr(self, "stage_keys", None) is None or self.stage_keys.device != self.temp_keys.device:
+                n_in = self.input_length - self.static_pattern_total
+                self.stage_keys = torch.empty((H, n_in, self.head_dim), dtype=self.dtype, device=self.temp_keys.device)
+                self.stage_values = torch.empty_like(self.stage_keys)
+            n_st = self.stage_keys.shape[1]
+            kernels.permute_rows(self.temp_keys, km.members, self.stage_keys, H, valid_length, valid_length, n_st)
+            kernels.permute_rows(self.temp_values, km.members, self.stage_values, H, valid_length, valid_length, n_st)
+            self.mainevents[dkey].record()
+            with torch.cuda.stream(self.copystream):
+                self.mainevents[dkey].wait()
+                self.list_keys[layer_idx][batch_idx, :, :valid_length].copy_(self.stage_keys[:, :valid_length],
+                                                                             non_blocking=True)
+                self.list_values[layer_idx][batch_idx, :, :valid_length].copy_(self.stage_values[:, :valid_length],
+                                                                               non_blocking=True)
+                self.copyevents[dkey].record()
         else:
             self.cluster_size_cpu = km.counts.cpu().contiguous()
             self.clusters_cpu = csr_to_dense(km.counts, km.offsets, km.members).cpu().contiguous()
@@ -287,7 +311,7 @@ class retroinfer_cache(KV_Cache):
     def sync(self, layer_idx, batch_idx):
         """After the prefill attention of (layer, sequence): hand the offloaded K/V to the host
         re-organisation (reference: retroinfer_cache.py:443-458).  Nothing to do on the device."""
-        if self.kv_residency == "host":
+        if self.kv_residency == "host" and self.block_cache == "host":
             self.copyevents[self.layer_mapping[str(layer_idx)]].synchronize()
             self.wave_buffer[layer_idx].async_construction(self.clusters_cpu, self.cluster_size_cpu, batch_idx)
 
@@ -305,7 +329,7 @@ class retroinfer_cache(KV_Cache):
             uv = self.steady_zone_values[ldx][:, :, lo:hi].clone().reshape(BG, THRESHOLD_LENGTH, D).contiguous()
             for zone in (self.steady_zone_keys, self.steady_zone_values):   # slide the local window
                 zone[ldx][:, :, sps:sps + spe] = zone[ldx][:, :, hi:hi + spe].clone()
-            if self.kv_residency == "host":
+            if self.kv_residency == "host" and self.block_cache == "host":
                 self.mainevents[dkey].record()
                 with torch.cuda.stream(self.copystream):
                     self.mainevents[dkey].wait()
@@ -328,13 +352,19 @@ class retroinfer_cache(KV_Cache):
                 lv = self.list_values[ldx].view(BG, self.list_stride, D)[:, base:]
                 kernels.permute_rows(uk, km.members, lk, BG, THRESHOLD_LENGTH, THRESHOLD_LENGTH, self.list_stride)
                 kernels.permute_rows(uv, km.members, lv, BG, THRESHOLD_LENGTH, THRESHOLD_LENGTH, self.list_stride)
+            elif self.block_cache == "device":
+                assert base + THRESHOLD_LENGTH <= self.list_stride, "cluster store is full"
+                pk, pv = torch.empty_like(uk), torch.empty_like(uv)
+                kernels.permute_rows(uk, km.members, pk, BG, THRESHOLD_LENGTH, THRESHOLD_LENGTH, THRESHOLD_LENGTH)
+                kernels.permute_rows(uv, km.members, pv, BG, THRESHOLD_LENGTH, THRESHOLD_LENGTH, THRESHOLD_LENGTH)
+                self.list_keys[ldx].view(BG, self.list_stride, D)[:, base:base + THRESHOLD_LENGTH].copy_(pk)
+                self.list_values[ldx].view(BG, self.list_stride, D)[:, base:base + THRESHOLD_LENGTH].copy_(pv)
+                self.device_lru[ldx].set_sizes(self.cluster_size_i32[ldx])
             else:
                 self.copyevents[dkey].synchronize()
                 self.wave_buffer[ldx].update_kv(self.offload_update_keys, self.offload_update_values,
                                                 csr_to_dense(km.counts, km.offsets, km.members).cpu().contiguous(),
                                                 km.counts.cpu().contiguous())
-                if self.block_cache == "device":
-                    self.device_lru[ldx].set_sizes(self.cluster_size_i32[ldx])
         torch.cuda.set_device(self.layer_mapping[str(0)])
         self.n_centroids += ncu
         self.logits = torch.zeros((BG, self.group_size, self.n_centroids), dtype=torch.float32,

@@ -249,3 +249,54 @@ def test_next_layer_cluster_estimation(dev, residency):
             differs += int((aux_true["ret"] != aux["ret"]).any())
     assert differs > 0
 
+
+
+@pytest.mark.parametrize("residency", ["device", "host", "host-cpu"])
+def test_index_growth_after_1024_generated_tokens(dev, residency):
+    """Decode-time index update (reference: retroinfer_cache.py:462-546): once the steady zone holds
+    1024 tokens beyond its 4 + 64, they are clustered into 64 new centroids and appended to the index
+    and the store; the last 64 stay as the local window.  Checked: the appended store rows are exactly
+    the folded tokens, and decoding afterwards matches the oracle on the grown index."""
+    layers, B, Hkv, gs, ctx = 1, 2, 2, 4, 2048 + 68
+    nc, nprobe, es, new = 128, 8, 40, 1100
+    cache = _make_cache(dev, residency, layers, B, Hkv, gs, ctx, nc, 1, nprobe, es, new=new)
+    K, V = _gen(layers, B, Hkv, gs, ctx, 128, dev, 21)
+    _prefill(cache, K, V, layers, B)
+    BG, N = B * Hkv, ctx - 68
+    g = torch.Generator().manual_seed(22)
+    gk = torch.randn(B, 1030, Hkv, 128, generator=g).to(torch.bfloat16)
+    gv = torch.randn(B, 1030, Hkv, 128, generator=g).to(torch.bfloat16)
+    q = torch.randn(B, 1, Hkv * gs, 128, generator=g).to(torch.bfloat16).to(dev)
+    for t in range(1030):
+        cache.decode_update_kv_cache(gk[:, t:t + 1].to(dev), gv[:, t:t + 1].to(dev), 0)
+        if t in (0, 700):          # keep the block cache busy before the index grows
+            cache.compute(q, 0)
+    torch.cuda.synchronize()
+    assert cache.n_centroids == nc + 64 and cache.centroids[0].shape[1] == nc + 64
+    assert cache.static_pattern_total == 4 + 64 + (1030 - 1024)   # the fold happened on the 1025th call
+    lk, lv = cache.list_keys[0].view(BG, -1, 128), cache.list_values[0].view(BG, -1, 128)
+    for b in range(B):
+        for h in range(Hkv):
+            gi = b * Hkv + h
+            folded_k = torch.cat([K[0][b][0, ctx - 64:, h].cpu(), gk[b, :960, h]])      # prompt tail + first 960 generated
+            folded_v = torch.cat([V[0][b][0, ctx - 64:, h].cpu(), gv[b, :960, h]])
+            got_k, got_v = lk[gi, N:N + 1024].cpu(), lv[gi, N:N + 1024].cpu()
+            assert torch.equal(torch.sort(got_k.float().sum(1)).values, torch.sort(folded_k.float().sum(1)).values)
+            assert torch.equal(torch.sort(got_v.float().sum(1)).values, torch.sort(folded_v.float().sum(1)).values)
+    size_i = cache.cluster_size_i32[0].cpu()
+    assert bool((size_i[:, nc:].sum(1) == 1024).all()) and bool((size_i.sum(1) == N + 1024).all())
+    out = cache.compute(q, 0)
+    torch.cuda.synchronize()
+    sk = [lk[gi, :N + 1024].cpu() for gi in range(BG)]
+    sv = [lv[gi, :N + 1024].cpu() for gi in range(BG)]
+    start = torch.cumsum(size_i.long(), 1) - size_i.long()
+    assert torch.equal(start.int(), cache.cluster_start[0].cpu())
+    static_len = cache.static_pattern_total
+    ref, aux = pipeline.decode_step(
+        q.cpu().view(BG, gs, 128), cache.steady_zone_keys[0].view(BG, -1, 128).cpu(),
+        cache.steady_zone_values[0].view(BG, -1, 128).cpu(), static_len, cache.centroids[0].cpu(),
+        cache.value_sum[0].cpu(), cache.centroids_mask[0].cpu(), size_i, cache.cluster_size[0].cpu(), sk, sv, start,
+        nprobe, es, 8, cache.buffer_size)
+    _close(out.cpu().view(BG, gs, 128), ref)
+    cI = cache.cI[0].cpu()
+    check_zone_sets(aux["dist"], cI[:, :nprobe], cI[:, nprobe:], aux["ret"], aux["est"], nprobe, es, band=2.0)
