@@ -58,7 +58,6 @@ struct AttendParams {
   int S_kv;
   int S_es;
   int gs;
-  int fuse;  // 1: the last workgroup of a group merges; 0: a separate combine launch does
   float scale;
   // epilogue
   const uint16_t* prev_out;  // [BG, gs, 128] or null
@@ -178,20 +177,16 @@ __device__ __forceinline__ void wave_rows(int total, int nwaves, int wid, int* r
 // Merges the S split partials of group g (and the optional previous result) and writes the
 // output: wave w of the calling workgroup takes heads w, w+4, ...; lanes first cover the splits
 // (statistics), then two dims each.
-// COHERENT: the partials were written by other workgroups of the same launch; they are read with
+// The partials were written by other workgroups of the same launch; they are read with
 // device-scope loads (which go past this compute unit's non-coherent cache lines) instead of
 // an acquire fence that would drop the whole cache.
-template <bool COHERENT>
 __device__ __forceinline__ float2 ri_ld_partial(const float* p) {
-  if (COHERENT) {
-    const uint64_t v = __hip_atomic_load(reinterpret_cast<const uint64_t*>(p), __ATOMIC_RELAXED,
-                                         __HIP_MEMORY_SCOPE_AGENT);
-    return make_float2(__uint_as_float((uint32_t)v), __uint_as_float((uint32_t)(v >> 32)));
-  }
-  return *reinterpret_cast<const float2*>(p);
+  const uint64_t v = __hip_atomic_load(reinterpret_cast<const uint64_t*>(p), __ATOMIC_RELAXED,
+                                       __HIP_MEMORY_SCOPE_AGENT);
+  return make_float2(__uint_as_float((uint32_t)v), __uint_as_float((uint32_t)(v >> 32)));
 }
 
-template <int GS_PAD, bool COHERENT>
+template <int GS_PAD>
 __device__ __forceinline__ void combine_group(const AttendParams& P, int g, int S, int lenB) {
   const int gs = P.gs;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -202,11 +197,11 @@ __device__ __forceinline__ void combine_group(const AttendParams& P, int g, int 
     // first CB_PRE splits' numerators; their latencies overlap instead of adding up
     constexpr int CB_PRE = 24;
     float2 ms = make_float2(-INFINITY, 0.f);
-    if (lane < S) ms = ri_ld_partial<COHERENT>(ml + (size_t)lane * GS_PAD * 2);
+    if (lane < S) ms = ri_ld_partial(ml + (size_t)lane * GS_PAD * 2);
     float2 a2[CB_PRE];
 #pragma unroll
     for (int u = 0; u < CB_PRE; ++u)
-      a2[u] = (u < S) ? ri_ld_partial<COHERENT>(pa + (size_t)u * GS_PAD * RI_DIM) : make_float2(0.f, 0.f);
+      a2[u] = (u < S) ? ri_ld_partial(pa + (size_t)u * GS_PAD * RI_DIM) : make_float2(0.f, 0.f);
     const float pl = P.prev_lse ? P.prev_lse[(size_t)g * gs + j] : -INFINITY;
     uint32_t po = 0u;
     if (P.prev_lse) po = *reinterpret_cast<const uint32_t*>(P.prev_out + ((size_t)g * gs + j) * RI_DIM + 2 * lane);
@@ -234,7 +229,7 @@ __device__ __forceinline__ void combine_group(const AttendParams& P, int g, int 
       float2 b2[8];
 #pragma unroll
       for (int u = 0; u < 8; ++u)
-        b2[u] = (s0 + u < S) ? ri_ld_partial<COHERENT>(pa + (size_t)(s0 + u) * GS_PAD * RI_DIM)
+        b2[u] = (s0 + u < S) ? ri_ld_partial(pa + (size_t)(s0 + u) * GS_PAD * RI_DIM)
                              : make_float2(0.f, 0.f);
 #pragma unroll
       for (int u = 0; u < 8; ++u) {
@@ -486,23 +481,15 @@ __global__ __launch_bounds__(256, GS_PAD == 16 ? 1 : 3) void attend_kernel(Atten
       l += sh_l[w][j] * f;
     }
     const size_t o = ((size_t)g * S + split) * GS_PAD + j;
-    if (P.fuse) {  // device-coherent stores: another workgroup of this launch reads them
-      __hip_atomic_store(&P.part_acc[o * RI_DIM + d], a, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      if (d == 0) {
-        __hip_atomic_store(&P.part_ml[o * 2], M, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        __hip_atomic_store(&P.part_ml[o * 2 + 1], l, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      }
-    } else {
-      P.part_acc[o * RI_DIM + d] = a;
-      if (d == 0) {
-        P.part_ml[o * 2] = M;
-        P.part_ml[o * 2 + 1] = l;
-      }
+    // device-coherent stores: another workgroup of this launch reads them
+    __hip_atomic_store(&P.part_acc[o * RI_DIM + d], a, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (d == 0) {
+      __hip_atomic_store(&P.part_ml[o * 2], M, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      __hip_atomic_store(&P.part_ml[o * 2 + 1], l, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
   }
 
   // ---------------- last workgroup of the group merges all splits ----------------
-  if (!P.fuse) return;
   // The partial went out with device-coherent stores; once they have completed the arrival is
   // announced.  The last workgroup to arrive reads every partial with device-coherent loads.
   __builtin_amdgcn_s_waitcnt(0);
@@ -511,16 +498,8 @@ __global__ __launch_bounds__(256, GS_PAD == 16 ? 1 : 3) void attend_kernel(Atten
     sh_last = (__hip_atomic_fetch_add(&P.counters[g], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == S - 1);
   __syncthreads();
   if (!sh_last) return;
-  combine_group<GS_PAD, true>(P, g, S, lenB);
+  combine_group<GS_PAD>(P, g, S, lenB);
   if (threadIdx.x == 0) P.counters[g] = 0;  // ready for the next launch
-}
-
-// separate merge pass: grid (BG), 256 threads
-template <int GS_PAD>
-__global__ __launch_bounds__(256) void combine_kernel(AttendParams P) {
-  const int g = blockIdx.x;
-  const int lenB = P.lenB_ptr ? P.lenB_ptr[(size_t)g * P.lenB_ptr_stride] : P.lenB_const;
-  combine_group<GS_PAD, false>(P, g, P.S_kv + P.S_es, lenB);
 }
 
 // ------------------------------------------------------------------------------------
@@ -546,33 +525,15 @@ static void carve_workspace(AttendParams& P, void* workspace, int BG, int gp) {
   P.part_acc = P.part_ml + (size_t)BG * RI_MAX_SPLITS * gp * 2;
 }
 
-static int fuse_default() {
-  static int v = -1;
-  if (v < 0) {
-    const char* e = getenv("RI_ATTN_FUSE");
-    v = e ? atoi(e) : 1;
-  }
-  return v;
-}
-
 static int launch_attend(AttendParams& P, int BG, int gs, hipStream_t s) {
   const int S = P.S_kv + P.S_es;
   const dim3 grid(S, BG);
-  P.fuse = fuse_default();
   switch (gs_pad_of(gs)) {
     case 4: attend_kernel<4, 2><<<grid, 256, 0, s>>>(P); break;
     case 8: attend_kernel<8, 2><<<grid, 256, 0, s>>>(P); break;
     default: attend_kernel<16, 2><<<grid, 256, 0, s>>>(P); break;
   }
   RI_HIP_CHECK_LAUNCH();
-  if (!P.fuse) {
-    switch (gs_pad_of(gs)) {
-      case 4: combine_kernel<4><<<BG, 256, 0, s>>>(P); break;
-      case 8: combine_kernel<8><<<BG, 256, 0, s>>>(P); break;
-      default: combine_kernel<16><<<BG, 256, 0, s>>>(P); break;
-    }
-    RI_HIP_CHECK_LAUNCH();
-  }
   return RI_OK;
 }
 
