@@ -61,6 +61,7 @@ def test_batch_gemm_softmax_matches_reference_test(dev):
     (2, 8, 16384, 294, 3801, 3),  # config-5 shape
     (3, 1, 64, 1, 0, 4),          # smallest: one probe, no estimation zone
     (2, 16, 1000, 20, 980, 5),    # nc not a multiple of 256, zones cover every cluster
+    (1, 4, 32768, 300, 3000, 6),  # more clusters than the select kernel stages in LDS
 ])
 def test_score_select(dev, BG, gs, nc, nprobe, es, seed):
     from retrievalattention_amd import kernels
