@@ -181,7 +181,7 @@ def bench_host(args, cfg, cache, queries, L, nprobe, es, static_len):
     B = cfg["B"]
 
     def step(l):
-        return cache._compute_staged(queries[l], l, None, static_len, l % 2, (l + 1) % 2, True, False)
+        return cache._compute(queries[l], l, None, static_len)
 
     torch.cuda.synchronize()
     t0 = time.perf_counter()
@@ -208,8 +208,8 @@ def bench_host(args, cfg, cache, queries, L, nprobe, es, static_len):
         run(i)
     torch.cuda.synchronize()
     t_warm = (time.perf_counter() - t0) / args.steps
-    miss = sum(int(cache.miss_num_units[l].sum()) for l in range(L))
-    hit = sum(int(cache.hit_num_units[l].sum()) for l in range(L))
+    stats = [cache.block_cache_stats(l) for l in range(L)]
+    hit, miss = sum(s_[0] for s_ in stats), sum(s_[1] for s_ in stats)
     print(json.dumps({
         "metric": "decode tokens/s at 128K ctx (attention only, B / (L * t_layer_step)); us/layer-step and % HBM roofline alongside",
         "value": B / (cfg["L"] * t_warm), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,

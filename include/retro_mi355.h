@@ -261,7 +261,12 @@ int ri_kmeans_value_sum(const void* values, const int32_t* counts, const int32_t
  * Policy: the walk over the ranks stops at the first cluster whose blocks do not fit
  * buffer_size; the longest prefix of the misses that fits `capacity` is admitted; victims are
  * whole clusters, least recently touched step first, ascending id inside a step, never one
- * touched in this call.  np <= 1023, ncl <= 65536. */
+ * touched in this call.  np <= 1023, ncl <= 65536.
+ * With row_src [BG, row_src_stride] and meta [BG, 4] (both or neither): for attention in place over
+ * one tensor that holds the `capacity` cache blocks first and the staging rows of the misses from row
+ * stage_row0 on, row_src receives the row of every retrieved token (hits: block id * block + i;
+ * misses: stage_row0 + their offset in the miss list), meta {clusters kept, tokens, blocks, 0} as
+ * ri_score_select writes it, and the hit count is reported as 0 (nothing to copy). */
 int ri_lru_access_update(const int32_t* ret_ids, const int32_t* sizes, const int32_t* starts,
                          int meta_stride, const int32_t* blk_off, int blk_off_stride, int32_t* stamp,
                          int stamp_stride, int32_t* blk_ids, int blk_ids_stride, int32_t* free_list,
@@ -269,6 +274,7 @@ int ri_lru_access_update(const int32_t* ret_ids, const int32_t* sizes, const int
                          int32_t* hit_cumsum, int32_t* hit_num, int32_t* miss_ids,
                          int32_t* miss_sizes, int32_t* miss_cumsum, int32_t* miss_num,
                          int32_t* upd_buf, int32_t* upd_sizes, int32_t* upd_cache, int32_t* upd_num,
+                         int32_t* row_src, int row_src_stride, int stage_row0, int32_t* meta,
                          int BG, int np, int ncl, int buffer_size, int capacity, int block,
                          ri_stream_t stream);
 

@@ -94,8 +94,10 @@ class DeviceLruModel:
     in ascending cluster id; admitted clusters take ids off the end of the list in rank order."""
     AGES = 256
 
-    def __init__(self, sizes, block, capacity, buffer_size):
+    def __init__(self, sizes, block, capacity, buffer_size, stage_row0=None):
         self.block, self.capacity, self.buffer_size = block, capacity, buffer_size
+        self.stage_row0 = stage_row0           # set: also keep the row table for attention in place
+        self.rows = []
         self.sizes = [int(s) for s in sizes]
         self.start, row = [], 0
         for s_ in self.sizes:
@@ -116,6 +118,7 @@ class DeviceLruModel:
         E = self.epoch + 1
         hit, miss, hits, misses = [], [], [], []
         pages = hs = ms = 0
+        self.rows = []
         for c in ids:
             c = int(c)
             if c < 0 or c >= len(self.sizes):
@@ -129,8 +132,11 @@ class DeviceLruModel:
                 hits.append(c)
                 for bid, sz in zip(self.blocks[c], self._blocks(c)):
                     hit.append((bid, sz, hs)); hs += sz
+                    self.rows += [bid * self.block + i for i in range(sz)]
             else:
                 misses.append((c, ms))
+                if self.stage_row0 is not None:
+                    self.rows += [self.stage_row0 + ms + i for i in range(self.sizes[c])]
                 row = self.start[c]
                 for sz in self._blocks(c):
                     miss.append((row, sz, ms)); ms += sz; row += self.block

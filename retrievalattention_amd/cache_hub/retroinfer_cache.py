@@ -170,7 +170,11 @@ class retroinfer_cache(KV_Cache):
                 hl["miss_unit_sizes_cumsum"][l], hl["miss_num_units"][l], hl["update_buffer_indices"][l],
                 hl["update_unit_sizes"][l], hl["update_cache_indices"][l], hl["update_num_units"][l],
                 self.cluster_ids[l % 2])
-        self.cache_keys = [torch.zeros((self.batch_size, self.kv_head, self.cache_size, self.page_size, D),
+        # with the device-side manager the staging blocks of the misses sit behind the cache blocks in the
+        # same tensor, so that attention can read hits in place and staged misses through one row table
+        self.cache_blocks = self.cache_size + (self.buffer_size if self.block_cache == "device" else 0)
+        self.cache_stride = self.cache_blocks
+        self.cache_keys = [torch.zeros((self.batch_size, self.kv_head, self.cache_blocks, self.page_size, D),
                                        dtype=self.dtype, device=dev(l)) for l in L]
         self.cache_values = [torch.zeros_like(self.cache_keys[l]) for l in L]
         n_in = self.input_length - self.static_pattern_total
@@ -191,14 +195,14 @@ class retroinfer_cache(KV_Cache):
         self.ret_ids = [i32(BG, self.nprobe) for _ in range(2)]
         self.est_ids = [i32(BG, max(self.es_cluster_num, 1)) for _ in range(2)]
         self.valid_lengths = [i32(BG) for _ in range(2)]
-        if self.kv_residency == "device":
+        if self.kv_residency == "device" or self.block_cache == "device":
             # token layout of the retrieval zone; a second set when the next layer's zones are chosen
             # while this layer's are still in use
             sets = 2 if self.use_cluster_estimation else 1
             self.layouts = [(i32(BG, self.nprobe + 1), i32(BG, self.buffer_size * self.page_size), i32(BG, 4))
                             for _ in range(sets)]
             self.ret_tok_off, self.row_src, self.meta = self.layouts[0]
-        else:
+        if self.kv_residency != "device":
             shape = (BG, self.execution_stride, 1, D)
             self.execution_buffer_keys = [torch.zeros(shape, dtype=self.dtype, device=d0) for _ in range(2)]
             self.execution_buffer_values = [torch.zeros(shape, dtype=self.dtype, device=d0) for _ in range(2)]
@@ -398,15 +402,21 @@ class retroinfer_cache(KV_Cache):
     def compute(self, queries, layer_idx, queries_next=None):
         """Decode attention of one layer (reference: retroinfer_cache.py:549-697).
         queries [batch, 1, heads, dim] on the device; returns the same shape."""
-        BG, gs, D = self.batch_groups, self.group_size, self.head_dim
         last = layer_idx == self.layer_num - 1
         static_len = self.static_pattern_total if last else self.static_pattern_total + 1
+        return self._compute(queries, layer_idx, queries_next, static_len)
+
+    def _compute(self, queries, layer_idx, queries_next, static_len):
+        """compute() for a given number of steady-zone tokens."""
         buf, nbuf = layer_idx % 2, (layer_idx + 1) % 2
         search_here = layer_idx < 2 or not self.use_cluster_estimation
         search_next = (self.use_cluster_estimation and 0 < layer_idx < self.layer_num - 1
                        and queries_next is not None)
         if self.kv_residency == "device" and not self.use_cluster_estimation:
             return self._compute_device(queries, layer_idx, static_len, buf)
+        if self.kv_residency == "host" and self.block_cache == "device":
+            return self._compute_host_in_place(queries, layer_idx, queries_next, static_len, buf, nbuf, search_here,
+                                               search_next)
         return self._compute_staged(queries, layer_idx, queries_next, static_len, buf, nbuf, search_here,
                                     search_next)
 
@@ -420,6 +430,75 @@ class retroinfer_cache(KV_Cache):
             static_len, self.list_keys[layer_idx], self.list_values[layer_idx], self.row_src, self.meta,
             self.est_ids[buf] if es > 0 else None, self.logits if es > 0 else None, self.value_sum[layer_idx],
             self.cluster_size[layer_idx], out, self.valid_lengths[buf], es, self.RSQRT_DIM)
+        return out.view(self.batch_size, 1, self.num_heads, D)
+
+    def block_cache_stats(self, layer_idx):
+        """(hit blocks, miss blocks) of the layer's last look-up, summed over the groups (host residency)."""
+        miss = int(self.miss_num_units[layer_idx].sum())
+        if self.block_cache == "device":
+            lay = (layer_idx % 2) if self.use_cluster_estimation else 0
+            return int(self.layouts[lay][2][:, 2].sum()) - miss, miss
+        return int(self.hit_num_units[layer_idx].sum()), miss
+
+    # host-resident store, block cache managed on the device: hits are read in place from the cache
+    # blocks, misses are staged behind them in the same tensor, both through one row table
+    def _access_in_place(self, layer, buf):
+        lay = buf if self.use_cluster_estimation else 0
+        _, row_src, meta = self.layouts[lay]
+        self.device_lru[layer].access_update(self.ret_ids[buf], self.cluster_size_i32[layer], self.cluster_start[layer],
+                                             self._lists(layer), row_src=row_src,
+                                             stage_row0=self.cache_size * self.page_size, meta=meta)
+
+    def _stage_misses(self, layer, buf):
+        BG, D = self.batch_groups, self.head_dim
+        rows = self.cache_blocks * self.page_size
+        stage_k = self.cache_keys[layer].view(BG, rows, D)[:, self.cache_size * self.page_size:]
+        stage_v = self.cache_values[layer].view(BG, rows, D)[:, self.cache_size * self.page_size:]
+        kernels.gather_copy_and_concat(
+            self.steady_zone_keys[layer], self.list_keys[layer], self.cache_keys[layer], stage_k,
+            self.steady_zone_values[layer], self.list_values[layer], self.cache_values[layer], stage_v,
+            self.miss_unit_idices[layer], self.miss_unit_sizes[layer], self.miss_unit_sizes_cumsum[layer],
+            self.miss_num_units[layer], self.hit_unit_idices[layer], self.hit_unit_sizes[layer],
+            self.hit_unit_sizes_cumsum[layer], self.hit_num_units[layer], self.valid_lengths[buf], BG,
+            self.static_stride, self.list_stride, self.cache_stride, rows, self.buffer_size, 0)
+        return stage_k, stage_v
+
+    def _compute_host_in_place(self, queries, layer_idx, queries_next, static_len, buf, nbuf, search_here,
+                               search_next):
+        BG, gs, D = self.batch_groups, self.group_size, self.head_dim
+        es = self.es_cluster_num
+        q = queries.view(BG, gs, D)
+        rows = self.cache_blocks * self.page_size
+        if search_here:
+            self._select(queries, layer_idx, buf, False)
+            self._access_in_place(layer_idx, buf)
+            self._stage_misses(layer_idx, buf)
+        else:
+            if es > 0:   # zones came from the predicted query: the estimation zone is scored by the true one
+                kernels.score_logits(q, self.centroids[layer_idx], self.logits, self.RSQRT_DIM)
+            torch.cuda.current_stream().wait_stream(self.copystream)   # misses staged during the previous layer
+        _, row_src, meta = self.layouts[buf if self.use_cluster_estimation else 0]
+        out = torch.empty((BG, gs, D), dtype=self.dtype, device=queries.device)
+        ck = self.cache_keys[layer_idx].view(BG, rows, D)
+        cv = self.cache_values[layer_idx].view(BG, rows, D)
+        kernels.wave_attention(
+            q, self.steady_zone_keys[layer_idx], self.steady_zone_values[layer_idx], static_len, ck, cv, row_src, meta,
+            self.est_ids[buf] if es > 0 else None, self.logits if es > 0 else None, self.value_sum[layer_idx],
+            self.cluster_size[layer_idx], out, self.valid_lengths[buf], es, self.RSQRT_DIM)
+        # admission: staged blocks of the admitted misses into the cache blocks handed out for them
+        stage0 = self.cache_size * self.page_size
+        kernels.gather_copy_and_scatter(
+            ck[:, stage0:], self.cache_keys[layer_idx], cv[:, stage0:], self.cache_values[layer_idx],
+            self.update_buffer_indices[layer_idx], self.update_unit_sizes[layer_idx],
+            self.update_cache_indices[layer_idx], self.update_num_units[layer_idx], BG, rows, self.cache_stride,
+            self.buffer_size, 0)
+        if search_next:
+            self._select(queries_next, layer_idx + 1, nbuf, False)
+            self._access_in_place(layer_idx + 1, nbuf)
+            cur = torch.cuda.current_stream()
+            self.copystream.wait_stream(cur)
+            with torch.cuda.stream(self.copystream):
+                self._stage_misses(layer_idx + 1, nbuf)
         return out.view(self.batch_size, 1, self.num_heads, D)
 
     # staged path: the reference's sequence of operators, one call each

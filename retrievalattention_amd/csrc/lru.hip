@@ -36,6 +36,11 @@ struct LruParams {
   int32_t *hit_ids, *hit_sizes, *hit_cumsum, *hit_num;
   int32_t *miss_ids, *miss_sizes, *miss_cumsum, *miss_num;
   int32_t *upd_buf, *upd_sizes, *upd_cache, *upd_num;
+  // optional row table for attention in place: row of every retrieved token in a tensor that holds the
+  // cache blocks first and the staging area of the misses behind them; then no hit list is emitted
+  int32_t* row_src;  // [BG, row_src_stride] or null
+  int32_t* meta;     // [BG, 4]: {clusters kept, tokens, blocks, 0} or null
+  int row_src_stride, stage_row0;
   int np, ncl, meta_stride, blk_off_stride, stamp_stride, blk_ids_stride, buffer_size, capacity, block;
 };
 
@@ -74,6 +79,7 @@ __global__ __launch_bounds__(LRU_THREADS) void lru_kernel(LruParams P) {
   __shared__ int sh_scan[4 * LRU_WAVES];
   __shared__ int sh_hist[LRU_AGES];
   __shared__ int sh_cut[2];  // boundary age, blocks freed by strictly older clusters
+  __shared__ int sh_off[LRU_THREADS], sh_src[LRU_THREADS];
   const int g = blockIdx.x;
   const int tid = threadIdx.x;
   const int block = P.block;
@@ -104,20 +110,48 @@ __global__ __launch_bounds__(LRU_THREADS) void lru_kernel(LruParams P) {
   const bool keep = c >= 0 && nb > 0 && p1[0] + nb <= P.buffer_size;
   const bool hit = keep && stamp[c] != 0;
   const bool miss = keep && !hit;
-  int v4[4] = {hit ? nb : 0, hit ? sz : 0, miss ? nb : 0, miss ? sz : 0}, p4[4], t4[4];
+  int v4[4] = {hit ? nb : 0, keep ? sz : 0, miss ? nb : 0, miss ? sz : 0}, p4[4], t4[4];
   lru_scan<4>(v4, p4, t4, sh_scan);
+  // p4[1]: tokens of kept clusters of lower rank (position in the row table); the hit list's own
+  // token offsets are only needed without a row table
+  int hit_tok = 0;
+  if (!P.row_src) {
+    int vh[1] = {hit ? sz : 0}, ph[1], th[1];
+    lru_scan<1>(vh, ph, th, sh_scan);
+    hit_tok = ph[0];
+  }
   // the longest prefix of the misses whose blocks fit the whole cache may be admitted
   bool adm = miss && p4[2] + nb <= P.capacity;
   int va[1] = {adm ? nb : 0}, pa[1], ta[1];
   lru_scan<1>(va, pa, ta, sh_scan);
   const int need = ta[0];
 
+  const bool rows = P.row_src != nullptr;
+  if (rows) {
+    // row table: every thread takes tokens t, t + 1024, ... and finds the rank that owns them by
+    // bisection over the token offsets of the ranks (clusters that were dropped have no tokens)
+    sh_off[tid] = p4[1];
+    sh_src[tid] = hit ? -(boff[c] + 1) : P.stage_row0 + p4[3];  // hits: where their block ids are
+    __syncthreads();
+    int32_t* table = P.row_src + (size_t)g * P.row_src_stride;
+    for (int t = tid; t < t4[1]; t += LRU_THREADS) {
+      int lo_r = 0, hi_r = LRU_THREADS;  // first rank whose offset exceeds t
+      while (lo_r < hi_r) {
+        const int mid = (lo_r + hi_r) >> 1;
+        if (sh_off[mid] > t) hi_r = mid; else lo_r = mid + 1;
+      }
+      const int r = lo_r - 1, i = t - sh_off[r], src = sh_src[r];
+      table[t] = src < 0 ? bids[-src - 1 + i / block] * block + i % block : src + i;
+    }
+  }
   if (hit) {
     const int32_t* ids = bids + boff[c];
-    for (int j = 0; j < nb; ++j) {
-      P.hit_ids[lo + p4[0] + j] = ids[j];
-      P.hit_sizes[lo + p4[0] + j] = (j == nb - 1) ? sz - (nb - 1) * block : block;
-      P.hit_cumsum[lo + p4[0] + j] = p4[1] + j * block;
+    if (!rows) {
+      for (int j = 0; j < nb; ++j) {
+        P.hit_ids[lo + p4[0] + j] = ids[j];
+        P.hit_sizes[lo + p4[0] + j] = (j == nb - 1) ? sz - (nb - 1) * block : block;
+        P.hit_cumsum[lo + p4[0] + j] = hit_tok + j * block;
+      }
     }
     stamp[c] = E;
   }
@@ -130,8 +164,17 @@ __global__ __launch_bounds__(LRU_THREADS) void lru_kernel(LruParams P) {
     }
   }
   if (tid == 0) {
-    P.hit_num[g] = t4[0];
+    P.hit_num[g] = rows ? 0 : t4[0];
     P.miss_num[g] = t4[2];
+  }
+  if (P.meta) {
+    const int nkept = __syncthreads_count(keep);
+    if (tid == 0) {
+      P.meta[g * 4 + 0] = nkept;
+      P.meta[g * 4 + 1] = t4[1];
+      P.meta[g * 4 + 2] = t4[0] + t4[2];
+      P.meta[g * 4 + 3] = 0;
+    }
   }
   if (tid < LRU_AGES) sh_hist[tid] = 0;
   __syncthreads();  // the hits carry this step's stamp before anybody looks for victims
@@ -225,7 +268,8 @@ extern "C" int ri_lru_access_update(const int32_t* ret_ids, const int32_t* sizes
                                     int32_t* free_count, int32_t* epoch, int32_t* hit_ids, int32_t* hit_sizes,
                                     int32_t* hit_cumsum, int32_t* hit_num, int32_t* miss_ids, int32_t* miss_sizes,
                                     int32_t* miss_cumsum, int32_t* miss_num, int32_t* upd_buf, int32_t* upd_sizes,
-                                    int32_t* upd_cache, int32_t* upd_num, int BG, int np, int ncl, int buffer_size,
+                                    int32_t* upd_cache, int32_t* upd_num, int32_t* row_src, int row_src_stride,
+                                    int stage_row0, int32_t* meta, int BG, int np, int ncl, int buffer_size,
                                     int capacity, int block, ri_stream_t stream) {
   if (!ret_ids || !sizes || !starts || !blk_off || !stamp || !blk_ids || !free_list || !free_count || !epoch ||
       !hit_ids || !hit_sizes || !hit_cumsum || !hit_num || !miss_ids || !miss_sizes || !miss_cumsum || !miss_num ||
@@ -235,9 +279,10 @@ extern "C" int ri_lru_access_update(const int32_t* ret_ids, const int32_t* sizes
       capacity <= 0 || block <= 0)
     return RI_ERR_ARG;
   if (meta_stride < ncl || blk_off_stride < ncl + 1 || stamp_stride < ncl || blk_ids_stride <= 0) return RI_ERR_ARG;
+  if (row_src && (!meta || row_src_stride < buffer_size * block || stage_row0 < capacity * block)) return RI_ERR_ARG;
   LruParams P = {ret_ids, sizes, starts, blk_off, stamp, blk_ids, free_list, free_count, epoch,
                  hit_ids, hit_sizes, hit_cumsum, hit_num, miss_ids, miss_sizes, miss_cumsum, miss_num,
-                 upd_buf, upd_sizes, upd_cache, upd_num,
+                 upd_buf, upd_sizes, upd_cache, upd_num, row_src, meta, row_src_stride, stage_row0,
                  np, ncl, meta_stride, blk_off_stride, stamp_stride, blk_ids_stride, buffer_size, capacity, block};
   lru_kernel<<<BG, LRU_THREADS, 0, (hipStream_t)stream>>>(P);
   RI_HIP_CHECK_LAUNCH();

@@ -302,14 +302,16 @@ class DeviceLru:
         self.blk_off[:, 1:ncl + 1] = torch.cumsum(nb, 1).to(torch.int32)
         assert int(self.blk_off[:, ncl].max()) <= self.blk_ids.shape[1]
 
-    def access_update(self, ret_ids, sizes, starts, lists):
-        """lists: the 12 tensors hit (ids, sizes, cumsum, num), miss (...), update (buf, sizes, cache, num)."""
+    def access_update(self, ret_ids, sizes, starts, lists, row_src=None, stage_row0=0, meta=None):
+        """lists: the 12 tensors hit (ids, sizes, cumsum, num), miss (...), update (buf, sizes, cache, num).
+        row_src / meta: row table for attention in place (hits are then not listed for copying)."""
         BG, np_ = ret_ids.shape
         ncl = sizes.shape[1]
         check(lib().ri_lru_access_update(
             _p(ret_ids), _p(sizes), _p(starts), sizes.stride(0), _p(self.blk_off), self.blk_off.shape[1],
             _p(self.stamp), self.stamp.shape[1], _p(self.blk_ids), self.blk_ids.shape[1], _p(self.free_list),
-            _p(self.free_count), _p(self.epoch), *[_p(t) for t in lists], BG, np_, ncl, self.buffer_size,
+            _p(self.free_count), _p(self.epoch), *[_p(t) for t in lists], _p(row_src),
+            0 if row_src is None else row_src.shape[1], stage_row0, _p(meta), BG, np_, ncl, self.buffer_size,
             self.capacity, self.block, _stream()), "lru_access_update")
 
 
