@@ -150,6 +150,7 @@ class ThreadPool:
     """wave_buffer_cpu.cpp:17-35."""
 
     def __init__(self, num_threads):
+        self._destroy = lib().ri_threadpool_destroy   # bound now: module globals may be gone at interpreter exit
         self._h = lib().ri_threadpool_create(int(num_threads))
         if not self._h:
             raise RuntimeError("ri_threadpool_create failed")
@@ -160,7 +161,7 @@ class ThreadPool:
     def __del__(self):
         h, self._h = getattr(self, "_h", None), None
         if h:
-            lib().ri_threadpool_destroy(h)
+            self._destroy(h)
 
 
 class WaveBufferCPU:
@@ -171,6 +172,7 @@ class WaveBufferCPU:
                  buffer_size, capacity, threads, pool):
         self._pool = pool
         self._keep = {}
+        self._destroy = lib().ri_wavebuf_destroy
         self._h = lib().ri_wavebuf_create(batch_size, group_num, dim, nprobe, block_size, n_centroids,
                                           final_n_centroids, buffer_size, capacity, threads, pool._h)
         if not self._h:
@@ -179,7 +181,7 @@ class WaveBufferCPU:
     def __del__(self):
         h, self._h = getattr(self, "_h", None), None
         if h:
-            lib().ri_wavebuf_destroy(h)
+            self._destroy(h)
 
     def set_indices(self, hit_block_ids, hit_block_sizes, hit_block_sizes_cumsum, hit_block_nums,
                     miss_block_ids, miss_block_sizes, miss_block_sizes_cumsum, miss_block_nums,
