@@ -43,9 +43,11 @@ def weighted_flash_decoding(q, k, v, weight=None, previous_out=None, previous_ls
 
 
 def estimation(logits, est_ids, value_sum, cluster_size_bf16):
-    """Estimation-zone partial from the scoring logits (SURVEY appendix A.4 semantics of the
-    call at cache_hub/retroinfer_cache.py:611-617): scores are the cluster logits, values the
-    cluster value sums, denominator weights the bf16 cluster sizes.
+    """Estimation-zone partial from the scoring logits (the call at
+    cache_hub/retroinfer_cache.py:611-617, semantics inferred from its operands): scores are the
+    cluster logits s_i = q.c_i / sqrt(D), values the cluster value sums, the denominator weights
+    e^{s_i} by the bf16 cluster sizes: out = sum_i e^{s_i} VS_i / sum_i w_i e^{s_i},
+    lse = log sum_i w_i e^{s_i}.
     logits [BG, gs, nc] fp32, est_ids [BG, es].  Returns (es_out fp64 [BG, gs, D], lse fp64)."""
     BG, gs, nc = logits.shape
     D = value_sum.shape[-1]
