@@ -323,8 +323,9 @@ def main():
     def attend(l, slot):
         kernels.wave_attention(
             queries[l].view(BG, gs, 128), cache.steady_zone_keys[l], cache.steady_zone_values[l], static_len,
-            cache.list_keys[l], cache.list_values[l], cache.row_src, cache.meta, cache.est_ids[slot], cache.logits,
-            cache.value_sum[l], cache.cluster_size[l], out_tmp, cache.valid_lengths[slot], es, cache.RSQRT_DIM)
+            cache.list_keys[l], cache.list_values[l], None, cache.meta, cache.est_ids[slot], cache.logits,
+            cache.value_sum[l], cache.cluster_size[l], out_tmp, cache.valid_lengths[slot], es, cache.RSQRT_DIM,
+            ret_tok_off=cache.ret_tok_off, ret_start=cache.ret_start)
 
     for i in range(n_k + 8):
         l, slot = i % L, i % 2

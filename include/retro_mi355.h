@@ -43,7 +43,7 @@ enum {
 const char* ri_status_string(int status);
 int ri_last_hip_error(void);
 /* ABI version: bumped when a signature changes. */
-int ri_abi_version(void);
+int ri_abi_version(void);   /* 2 */
 /* Launches an empty kernel on `stream`: lets a caller measure the per-dispatch overhead that
  * event timings of back-to-back launches include.  No counterpart in the reference. */
 int ri_null_launch(ri_stream_t stream);
@@ -81,14 +81,17 @@ int ri_batch_gemm_softmax(const void* A, const void* B, void* D, float* Norm, fl
  *   ret_tok_off[BG, np+1] int32: exclusive token prefix of the retrieval clusters after
  *              the reference's buffer cut-off (stop before the first cluster whose pages
  *              push the running total over max_pages; wave_buffer_cpu.cpp:207-216)
- *   row_src    [BG, row_src_stride] int32: store row of every retrieved token, or NULL
+ *              (entries from the last kept rank on hold the retrieved token count)
+ *   ret_start  [BG, np] int32 or NULL: first store row of the cluster of every rank
+ *   row_src    [BG, row_src_stride] int32: store row of every retrieved token, or NULL (the
+ *              attention can work from ret_tok_off + ret_start instead, which is cheaper to write)
  *   meta       [BG, 4] int32: {clusters kept, retrieved tokens, pages used, 0}
  * workspace: ri_score_select_workspace_bytes(BG, gs, nc) bytes of device memory. */
 size_t ri_score_select_workspace_bytes(int BG, int gs, int nc);
 int ri_score_select(const void* q, const void* centroids, const uint8_t* mask,
                     const int32_t* cluster_size_i32, const int32_t* cluster_start,
                     float* logits, void* dist, int64_t* cI, int32_t* ret_ids,
-                    int32_t* est_ids, int32_t* ret_tok_off, int32_t* row_src,
+                    int32_t* est_ids, int32_t* ret_tok_off, int32_t* ret_start, int32_t* row_src,
                     int row_src_stride, int32_t* meta, int BG, int gs, int nc, int np, int es,
                     int page, int max_pages, float scale, void* workspace,
                     size_t workspace_bytes, ri_stream_t stream);
@@ -134,7 +137,9 @@ int ri_weighted_flash_decoding(const void* q, const void* k, const void* v, cons
  * the row table instead of staging them in an execution buffer.
  *   steady_k/v [BG, steady_stride, 128]: first static_len rows attended
  *   store_k/v  [BG, store_stride, 128]: cluster-contiguous K/V
- *   row_src, meta, est_ids, logits: as written by ri_score_select
+ *   row_src [BG, row_src_stride]: store row of every retrieved token; or NULL with ret_tok_off
+ *   [BG, np+1] and ret_start [BG, np]: rank r's tokens are the store rows ret_start[r] + i
+ *   meta, est_ids, logits: as written by ri_score_select (or meta by ri_lru_access_update)
  *   value_sum [BG, nc, 128] bf16, cluster_size_bf16 [BG, nc] bf16 (estimation weights)
  *   es may be 0 (no estimation zone).  out [BG, gs, 128] bf16; valid_lengths [BG] int32 or
  *   NULL receives static_len + retrieved tokens (what gather_copy_and_concat reports).
@@ -143,7 +148,8 @@ size_t ri_wave_attention_workspace_bytes(int BG, int gs);
 int ri_wave_attention(const void* q, const void* steady_k, const void* steady_v,
                       int64_t steady_stride, int static_len, const void* store_k,
                       const void* store_v, int64_t store_stride, const int32_t* row_src,
-                      int row_src_stride, const int32_t* meta, const int32_t* est_ids,
+                      int row_src_stride, const int32_t* ret_tok_off, const int32_t* ret_start, int np,
+                      const int32_t* meta, const int32_t* est_ids,
                       const float* logits, const void* value_sum,
                       const void* cluster_size_bf16, void* out, int32_t* valid_lengths,
                       int BG, int gs, int nc, int es, float scale, void* workspace,

@@ -18,12 +18,12 @@ SIGNATURES = {
     "ri_null_launch": (I, [P]),
     "ri_batch_gemm_softmax": (I, [P, P, P, P, P, P, I, I, I, I, F, F, P]),
     "ri_score_select_workspace_bytes": (SZ, [I, I, I]),
-    "ri_score_select": (I, [P, P, P, P, P, P, P, P, P, P, P, P, I, P, I, I, I, I, I, I, I, F, P, SZ, P]),
+    "ri_score_select": (I, [P] * 13 + [I, P, I, I, I, I, I, I, I, F, P, SZ, P]),
     "ri_score_logits": (I, [P, P, P, I, I, I, F, P, SZ, P]),
     "ri_flash_decoding_workspace_bytes": (SZ, [I, I]),
     "ri_weighted_flash_decoding": (I, [P, P, P, P, P, P, P, P, P, I, I, I, I64, F, P, SZ, P]),
     "ri_wave_attention_workspace_bytes": (SZ, [I, I]),
-    "ri_wave_attention": (I, [P, P, P, I64, I, P, P, I64, P, I, P, P, P, P, P, P, P, I, I, I, I, F, P, SZ, P]),
+    "ri_wave_attention": (I, [P, P, P, I64, I, P, P, I64, P, I, P, P, I, P, P, P, P, P, P, P, I, I, I, I, F, P, SZ, P]),
     "ri_buffer_attention": (I, [P, P, P, I64, P, I, P, P, P, P, P, I, I, I, I, F, P, SZ, P]),
     "ri_lru_access_update": (I, [P, P, P, I, P, I, P, I, P, I, P, P, P] + [P] * 12 + [P, I, I, P] + [I] * 6 + [P]),
     "ri_gather_copy_vectors": (I, [P, P, P, P, P, P, P, I, I, I, I, I, I, P]),

@@ -191,7 +191,12 @@ class retroinfer_cache(KV_Cache):
         BG, D, gs = self.batch_groups, self.head_dim, self.group_size
         i32 = lambda *s: torch.zeros(s, dtype=torch.int32, device=d0)
         self.logits = torch.zeros((BG, gs, self.n_centroids), dtype=torch.float32, device=d0)
-        self.cI = [torch.zeros((BG, self.max_compute_cluster_num), dtype=torch.int64, device=d0) for _ in range(2)]
+        # int64 id lists [BG, nprobe + es] as the reference keeps them: real tensors on the staged
+        # operator path (gather_copy_vectors and the host id copy read them), views put together from the
+        # int32 lists on demand elsewhere
+        staged = self.kv_residency == "host" and self.block_cache == "host"
+        self._cI = [torch.zeros((BG, self.max_compute_cluster_num), dtype=torch.int64, device=d0)
+                    for _ in range(2)] if staged else None
         self.ret_ids = [i32(BG, self.nprobe) for _ in range(2)]
         self.est_ids = [i32(BG, max(self.es_cluster_num, 1)) for _ in range(2)]
         self.valid_lengths = [i32(BG) for _ in range(2)]
@@ -199,9 +204,12 @@ class retroinfer_cache(KV_Cache):
             # token layout of the retrieval zone; a second set when the next layer's zones are chosen
             # while this layer's are still in use
             sets = 2 if self.use_cluster_estimation else 1
-            self.layouts = [(i32(BG, self.nprobe + 1), i32(BG, self.buffer_size * self.page_size), i32(BG, 4))
+            # device residency: rank tables (token prefix and first store row of every rank); host
+            # residency with the device-side manager: a row table (hits are scattered cache blocks)
+            rows = self.buffer_size * self.page_size if self.kv_residency != "device" else 1
+            self.layouts = [(i32(BG, self.nprobe + 1), i32(BG, self.nprobe), i32(BG, rows), i32(BG, 4))
                             for _ in range(sets)]
-            self.ret_tok_off, self.row_src, self.meta = self.layouts[0]
+            self.ret_tok_off, self.ret_start, self.row_src, self.meta = self.layouts[0]
         if self.kv_residency != "device":
             shape = (BG, self.execution_stride, 1, D)
             self.execution_buffer_keys = [torch.zeros(shape, dtype=self.dtype, device=d0) for _ in range(2)]
@@ -386,18 +394,31 @@ class retroinfer_cache(KV_Cache):
             self.static_pattern_total += 1
         return None, None
 
+    @property
+    def cI(self):
+        """[2] tensors [BG, nprobe + es] int64: retrieval ids in rank order, then estimation ids
+        (reference attribute: retroinfer_cache.py:573)."""
+        if self._cI is not None:
+            return self._cI
+        es = self.es_cluster_num
+        return [torch.cat((self.ret_ids[b], self.est_ids[b][:, :es]), dim=1).to(torch.int64) for b in range(2)]
+
     # ------------------------------------------------------------------ decode
     def _select(self, queries, layer, buf, with_layout, layout=0):
         BG, gs, D = self.batch_groups, self.group_size, self.head_dim
         q = queries.view(BG, gs, D)
         es = self.es_cluster_num
         dev_mode = with_layout and self.kv_residency == "device"
-        ret_tok_off, row_src, meta = self.layouts[layout] if dev_mode else (None, None, None)
+        ret_tok_off, ret_start, _, meta = self.layouts[layout] if dev_mode else (None, None, None, None)
+        # the int64 id list of the reference is only written where something reads it (the staged
+        # operator path); elsewhere cI is put together from the int32 lists on demand
+        cI = self._cI[buf] if self._cI is not None else None
         kernels.score_select(
             q, self.centroids[layer], self.centroids_mask[layer],
             self.cluster_size_i32[layer] if dev_mode else None, self.cluster_start[layer] if dev_mode else None,
-            self.logits, None, self.cI[buf], self.ret_ids[buf], self.est_ids[buf] if es > 0 else None,
-            ret_tok_off, row_src, meta, self.nprobe, es, self.page_size, self.buffer_size, self.RSQRT_DIM)
+            self.logits, None, cI, self.ret_ids[buf], self.est_ids[buf] if es > 0 else None,
+            ret_tok_off, None, meta, self.nprobe, es, self.page_size, self.buffer_size, self.RSQRT_DIM,
+            ret_start=ret_start)
 
     def compute(self, queries, layer_idx, queries_next=None):
         """Decode attention of one layer (reference: retroinfer_cache.py:549-697).
@@ -427,9 +448,10 @@ class retroinfer_cache(KV_Cache):
         es = self.es_cluster_num
         kernels.wave_attention(
             queries.view(BG, gs, D), self.steady_zone_keys[layer_idx], self.steady_zone_values[layer_idx],
-            static_len, self.list_keys[layer_idx], self.list_values[layer_idx], self.row_src, self.meta,
+            static_len, self.list_keys[layer_idx], self.list_values[layer_idx], None, self.meta,
             self.est_ids[buf] if es > 0 else None, self.logits if es > 0 else None, self.value_sum[layer_idx],
-            self.cluster_size[layer_idx], out, self.valid_lengths[buf], es, self.RSQRT_DIM)
+            self.cluster_size[layer_idx], out, self.valid_lengths[buf], es, self.RSQRT_DIM,
+            ret_tok_off=self.ret_tok_off, ret_start=self.ret_start)
         return out.view(self.batch_size, 1, self.num_heads, D)
 
     def block_cache_stats(self, layer_idx):
@@ -437,14 +459,14 @@ class retroinfer_cache(KV_Cache):
         miss = int(self.miss_num_units[layer_idx].sum())
         if self.block_cache == "device":
             lay = (layer_idx % 2) if self.use_cluster_estimation else 0
-            return int(self.layouts[lay][2][:, 2].sum()) - miss, miss
+            return int(self.layouts[lay][3][:, 2].sum()) - miss, miss
         return int(self.hit_num_units[layer_idx].sum()), miss
 
     # host-resident store, block cache managed on the device: hits are read in place from the cache
     # blocks, misses are staged behind them in the same tensor, both through one row table
     def _access_in_place(self, layer, buf):
         lay = buf if self.use_cluster_estimation else 0
-        _, row_src, meta = self.layouts[lay]
+        _, _, row_src, meta = self.layouts[lay]
         self.device_lru[layer].access_update(self.ret_ids[buf], self.cluster_size_i32[layer], self.cluster_start[layer],
                                              self._lists(layer), row_src=row_src,
                                              stage_row0=self.cache_size * self.page_size, meta=meta)
@@ -477,7 +499,7 @@ class retroinfer_cache(KV_Cache):
             if es > 0:   # zones came from the predicted query: the estimation zone is scored by the true one
                 kernels.score_logits(q, self.centroids[layer_idx], self.logits, self.RSQRT_DIM)
             torch.cuda.current_stream().wait_stream(self.copystream)   # misses staged during the previous layer
-        _, row_src, meta = self.layouts[buf if self.use_cluster_estimation else 0]
+        _, _, row_src, meta = self.layouts[buf if self.use_cluster_estimation else 0]
         out = torch.empty((BG, gs, D), dtype=self.dtype, device=queries.device)
         ck = self.cache_keys[layer_idx].view(BG, rows, D)
         cv = self.cache_values[layer_idx].view(BG, rows, D)
@@ -505,7 +527,7 @@ class retroinfer_cache(KV_Cache):
     def _search(self, queries, layer, buf):
         self._select(queries, layer, buf, False)
         if self.kv_residency == "host" and self.block_cache == "host":
-            self.cluster_ids[buf].copy_(self.cI[buf][:, :self.nprobe])  # blocking copy into pinned memory
+            self.cluster_ids[buf].copy_(self._cI[buf][:, :self.nprobe])  # blocking copy into pinned memory
 
     def _lists(self, layer):
         return [self.hit_unit_idices[layer], self.hit_unit_sizes[layer], self.hit_unit_sizes_cumsum[layer],
@@ -550,7 +572,7 @@ class retroinfer_cache(KV_Cache):
         if self.es_cluster_num > 0 and not fuse_est:
             kernels.gather_copy_vectors(
                 self.centroids[layer_idx], self.es_centroids, self.value_sum[layer_idx], self.es_value_sum,
-                self.cluster_size[layer_idx], self.es_cluster_size, self.cI[buf], BG, self.n_centroids,
+                self.cluster_size[layer_idx], self.es_cluster_size, self._cI[buf], BG, self.n_centroids,
                 self.es_cluster_num, self.max_compute_cluster_num, self.nprobe, self.es_cluster_num)
             es_out, es_lse = kernels.weighted_flash_decoding(q4, self.es_centroids, self.es_value_sum,
                                                              self.es_cluster_size, return_softmax_lse=True)
@@ -603,13 +625,14 @@ class retroinfer_cache(KV_Cache):
             self._select(queries, layer_idx, buf, True, layout=buf)
         elif es > 0:
             kernels.score_logits(q, self.centroids[layer_idx], self.logits, self.RSQRT_DIM)
-        ret_tok_off, row_src, meta = self.layouts[buf]
+        ret_tok_off, ret_start, _, meta = self.layouts[buf]
         out = torch.empty((BG, gs, D), dtype=self.dtype, device=queries.device)
         kernels.wave_attention(
             q, self.steady_zone_keys[layer_idx], self.steady_zone_values[layer_idx], static_len,
-            self.list_keys[layer_idx], self.list_values[layer_idx], row_src, meta,
+            self.list_keys[layer_idx], self.list_values[layer_idx], None, meta,
             self.est_ids[buf] if es > 0 else None, self.logits if es > 0 else None, self.value_sum[layer_idx],
-            self.cluster_size[layer_idx], out, self.valid_lengths[buf], es, self.RSQRT_DIM)
+            self.cluster_size[layer_idx], out, self.valid_lengths[buf], es, self.RSQRT_DIM,
+            ret_tok_off=ret_tok_off, ret_start=ret_start)
         if search_next:
             self._select(queries_next, layer_idx + 1, nbuf, True, layout=nbuf)
         return out.view(self.batch_size, 1, self.num_heads, D)

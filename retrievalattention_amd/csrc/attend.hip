@@ -39,6 +39,11 @@ struct AttendParams {
   int64_t strideB;
   const int32_t* row_src;
   int rs_stride;
+  // or, without a row table: rank r of np clusters covers rows [ret_off[r], ret_off[r+1]) of region B,
+  // stored contiguously from row ret_start[r] (ret_off has np + 1 entries, constant from the last kept rank on)
+  const int32_t* ret_off;
+  const int32_t* ret_start;
+  int np;
   const int32_t* lenB_ptr;  // lenB(g) = lenB_ptr ? lenB_ptr[g*lenB_ptr_stride] : lenB_const
   int lenB_ptr_stride;
   int lenB_const;
@@ -262,6 +267,7 @@ __global__ __launch_bounds__(256, GS_PAD == 16 ? 1 : 3) void attend_kernel(Atten
   __shared__ int sh_desc[4][ATT_DESC_MAX];
   __shared__ float sh_w[4][ATT_DESC_MAX];
   __shared__ int sh_last;
+  __shared__ int sh_roff[1025], sh_rst[1024];
 
   const int g = blockIdx.y;
   const int split = blockIdx.x;
@@ -288,17 +294,39 @@ __global__ __launch_bounds__(256, GS_PAD == 16 ? 1 : 3) void attend_kernel(Atten
 
   if (split < P.S_kv) {
     // ---------------- key/value rows ----------------
+    // rank tables (requested together with everything else the prologue loads: no dependent round trip)
+    const bool tab = P.ret_off != nullptr;
+    // every global load of the prologue is requested before the first of them is consumed
+    int t_off[4], t_st[4];
+    if (tab) {
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int i = threadIdx.x + u * 256;
+        t_off[u] = (i <= P.np) ? P.ret_off[(size_t)g * (P.np + 1) + i] : 0;
+        t_st[u] = (i < P.np) ? P.ret_start[(size_t)g * P.np + i] : 0;
+      }
+    }
+    // A operand: query heads through LDS (read again per chunk: registers go to the loads);
+    // row m of the MFMA holds head m % GS_PAD, zero if >= gs
+    static_assert(GS_PAD * (RI_DIM / 8) <= 256, "one piece of the query per thread");
+    {
+      const int head = threadIdx.x / (RI_DIM / 8), piece = threadIdx.x % (RI_DIM / 8);
+      uint4 qv = ri_zero16();
+      if (head < gs) qv = ri_ld16(P.q + ((size_t)g * gs + head) * RI_DIM + piece * 8);
+      if (head < GS_PAD) *reinterpret_cast<uint4*>(&sh_q[head][piece * 8]) = qv;
+    }
+    if (tab) {
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int i = threadIdx.x + u * 256;
+        if (i <= P.np) sh_roff[i] = t_off[u];
+        if (i < P.np) sh_rst[i] = t_st[u];
+      }
+    }
+    // (the row count is consumed only now: the loads above went out together with its load)
     const int total = P.lenA + lenB;
     int r0, r1;
     wave_rows(total, P.S_kv * 4, split * 4 + wave, &r0, &r1);
-
-    // A operand: query heads through LDS (read again per chunk: registers go to the loads);
-    // row m of the MFMA holds head m % GS_PAD, zero if >= gs
-    for (int i = threadIdx.x; i < GS_PAD * (RI_DIM / 8); i += 256) {
-      const int head = i / (RI_DIM / 8), piece = i % (RI_DIM / 8);
-      *reinterpret_cast<uint4*>(&sh_q[head][piece * 8]) =
-          (head < gs) ? ri_ld16(P.q + ((size_t)g * gs + head) * RI_DIM + piece * 8) : ri_zero16();
-    }
     const uint16_t* qrow = &sh_q[n % GS_PAD][h * 8];
     const uint16_t* kA = P.kA + (size_t)g * P.strideA * RI_DIM;
     const uint16_t* vA = P.vA + (size_t)g * P.strideA * RI_DIM;
@@ -308,6 +336,10 @@ __global__ __launch_bounds__(256, GS_PAD == 16 ? 1 : 3) void attend_kernel(Atten
     const uint16_t* wB = P.weightB ? P.weightB + (size_t)g * P.weight_stride : nullptr;
     const int r_first = ri_head_reg<GS_PAD>(h);
     bool q_ready = false;
+    if (tab) {  // the tables are searched while the rows are located
+      __syncthreads();
+      q_ready = true;
+    }
 
     for (int s0 = r0; s0 < r1; s0 += ATT_DESC_MAX) {
       const int s1 = min(r1, s0 + ATT_DESC_MAX);
@@ -321,7 +353,18 @@ __global__ __launch_bounds__(256, GS_PAD == 16 ? 1 : 3) void attend_kernel(Atten
             d = row | ATT_FLAG_A;
           } else {
             const int rb = row - P.lenA;
-            d = rs ? rs[rb] : rb;
+            if (tab) {
+              // the last rank whose first row is <= rb (ranks of empty clusters share a first row
+              // with the next rank, which is the one found)
+              int lo = 0, hi = P.np;
+              while (lo + 1 < hi) {
+                const int mid = (lo + hi) >> 1;
+                if (sh_roff[mid] <= rb) lo = mid; else hi = mid;
+              }
+              d = sh_rst[lo] + rb - sh_roff[lo];
+            } else {
+              d = rs ? rs[rb] : rb;
+            }
             if (wB) w = ri_bf16_to_f32(wB[rb]);
           }
         }
@@ -601,12 +644,13 @@ extern "C" int ri_weighted_flash_decoding(const void* q, const void* k, const vo
 extern "C" int ri_wave_attention(const void* q, const void* steady_k, const void* steady_v,
                                  int64_t steady_stride, int static_len, const void* store_k,
                                  const void* store_v, int64_t store_stride, const int32_t* row_src,
-                                 int row_src_stride, const int32_t* meta, const int32_t* est_ids,
+                                 int row_src_stride, const int32_t* ret_tok_off, const int32_t* ret_start, int np,
+                                 const int32_t* meta, const int32_t* est_ids,
                                  const float* logits, const void* value_sum, const void* cluster_size_bf16,
                                  void* out, int32_t* valid_lengths, int BG, int gs, int nc, int es,
                                  float scale, void* workspace, size_t workspace_bytes, ri_stream_t stream) {
-  if (!q || !steady_k || !steady_v || !store_k || !store_v || !row_src || !meta || !out || !workspace)
-    return RI_ERR_ARG;
+  if (!q || !steady_k || !steady_v || !store_k || !store_v || !meta || !out || !workspace) return RI_ERR_ARG;
+  if (!row_src && (!ret_tok_off || !ret_start || np <= 0 || np > 1023)) return RI_ERR_ARG;
   if (BG <= 0 || BG > RI_MAX_GROUPS || gs <= 0 || gs > 16 || static_len < 0 || static_len > steady_stride ||
       es < 0 || nc <= 0)
     return RI_ERR_ARG;
@@ -624,6 +668,11 @@ extern "C" int ri_wave_attention(const void* q, const void* steady_k, const void
   P.strideB = store_stride;
   P.row_src = row_src;
   P.rs_stride = row_src_stride;
+  if (!row_src) {
+    P.ret_off = ret_tok_off;
+    P.ret_start = ret_start;
+    P.np = np;
+  }
   P.lenB_ptr = meta + 1;
   P.lenB_ptr_stride = 4;
   P.est_ids = est_ids;
@@ -637,8 +686,9 @@ extern "C" int ri_wave_attention(const void* q, const void* steady_k, const void
   P.out = (uint16_t*)out;
   P.valid_lengths = valid_lengths;
   // the retrieved-token count is only known on the device: size the split for the row table
-  // capacity scaled by the usual fill (a quarter), the estimation zone by its exact size
-  plan_splits(static_len + row_src_stride / 4, es, BG, &P.S_kv, &P.S_es);
+  // capacity scaled by the usual fill (a quarter) or for 16 tokens per rank, the estimation zone by
+  // its exact size
+  plan_splits(static_len + (row_src ? row_src_stride / 4 : np * 16), es, BG, &P.S_kv, &P.S_es);
   carve_workspace(P, workspace, BG, gp);
   return launch_attend(P, BG, gs, (hipStream_t)stream);
 }

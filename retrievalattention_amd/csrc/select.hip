@@ -159,8 +159,8 @@ __device__ __forceinline__ uint32_t sel_bin(uint32_t key) {
 __global__ __launch_bounds__(SEL_THREADS) void select_kernel(
     const uint16_t* __restrict__ keys, const int32_t* __restrict__ cluster_size,
     const int32_t* __restrict__ cluster_start, int64_t* __restrict__ cI, int32_t* __restrict__ ret_ids,
-    int32_t* __restrict__ est_ids, int32_t* __restrict__ ret_tok_off, int32_t* __restrict__ row_src,
-    int row_src_stride, int32_t* __restrict__ meta, int nc, int np, int es, int page, int max_pages,
+    int32_t* __restrict__ est_ids, int32_t* __restrict__ ret_tok_off, int32_t* __restrict__ ret_start,
+    int32_t* __restrict__ row_src, int row_src_stride, int32_t* __restrict__ meta, int nc, int np, int es, int page, int max_pages,
     int sizes_in_lds) {
   extern __shared__ int32_t sh_size[];  // nc cluster sizes when sizes_in_lds
   __shared__ uint32_t hist[SEL_BINS];
@@ -218,12 +218,16 @@ __global__ __launch_bounds__(SEL_THREADS) void select_kernel(
     block_excl_scan<1>(vin, below, tot, sh_scan[0]);
     uint32_t above = tot[0] - below[0] - mine;  // entries in bins above this thread's
     const uint32_t rankA = (uint32_t)(np - 1), rankB = (uint32_t)(k2 - 1);
+    // only threads that hold keys of the retrieval zone (their bins' ranks are needed below) or one of
+    // the two threshold ranks walk their bins
+    if (mine > 0 && (above < (uint32_t)np || (above <= rankB && rankB < above + mine))) {
 #pragma unroll
-    for (int i = SEL_BPT - 1; i >= 0; --i) {
-      if (above <= rankA && rankA < above + hb[i]) { sh_sel[0] = tid * SEL_BPT + i; sh_sel[1] = above; }
-      if (above <= rankB && rankB < above + hb[i]) { sh_sel[2] = tid * SEL_BPT + i; sh_sel[3] = above; }
-      hist[tid * SEL_BPT + i] = above;
-      above += hb[i];
+      for (int i = SEL_BPT - 1; i >= 0; --i) {
+        if (above <= rankA && rankA < above + hb[i]) { sh_sel[0] = tid * SEL_BPT + i; sh_sel[1] = above; }
+        if (above <= rankB && rankB < above + hb[i]) { sh_sel[2] = tid * SEL_BPT + i; sh_sel[3] = above; }
+        hist[tid * SEL_BPT + i] = above;
+        above += hb[i];
+      }
     }
   }
   __syncthreads();
@@ -350,6 +354,7 @@ __global__ __launch_bounds__(SEL_THREADS) void select_kernel(
   }
   if (!cluster_size) return;
   if (r <= np) ret_tok_off[(size_t)g * (np + 1) + r] = (r < nkeep) ? (int32_t)tok_run : T_ret;
+  if (ret_start && r < np) ret_start[(size_t)g * np + r] = st;
   if (tid == 0) {
     meta[g * 4 + 0] = nkeep;
     meta[g * 4 + 1] = T_ret;
@@ -377,8 +382,8 @@ extern "C" size_t ri_score_select_workspace_bytes(int BG, int gs, int nc) {
 extern "C" int ri_score_select(const void* q, const void* centroids, const uint8_t* mask,
                                const int32_t* cluster_size_i32, const int32_t* cluster_start,
                                float* logits, void* dist, int64_t* cI, int32_t* ret_ids,
-                               int32_t* est_ids, int32_t* ret_tok_off, int32_t* row_src,
-                               int row_src_stride, int32_t* meta, int BG, int gs, int nc, int np,
+                               int32_t* est_ids, int32_t* ret_tok_off, int32_t* ret_start,
+                               int32_t* row_src, int row_src_stride, int32_t* meta, int BG, int gs, int nc, int np,
                                int es, int page, int max_pages, float scale, void* workspace,
                                size_t workspace_bytes, ri_stream_t stream) {
   if (!q || !centroids || !logits || !ret_ids || !workspace) return RI_ERR_ARG;
@@ -408,7 +413,8 @@ extern "C" int ri_score_select(const void* q, const void* centroids, const uint8
   // all cluster sizes fit in LDS next to the histogram up to 16384 clusters
   const int sizes_in_lds = (cluster_size_i32 && nc <= 16384) ? 1 : 0;
   select_kernel<<<BG, SEL_THREADS, sizes_in_lds ? (size_t)nc * sizeof(int32_t) : 0, s>>>(
-      keys, cluster_size_i32, cluster_start, cI, ret_ids, est_ids, ret_tok_off, row_src, row_src_stride, meta, nc,
+      keys, cluster_size_i32, cluster_start, cI, ret_ids, est_ids, ret_tok_off, ret_start, row_src, row_src_stride, meta,
+      nc,
       np, es, page, max_pages, sizes_in_lds);
   RI_HIP_CHECK_LAUNCH();
   return RI_OK;

@@ -232,16 +232,18 @@ class WaveBufferCPU:
 # fused MI355X entry points
 # ----------------------------------------------------------------------------------------
 def score_select(q, centroids, mask, cluster_size_i32, cluster_start, logits, dist, cI, ret_ids, est_ids,
-                 ret_tok_off, row_src, meta, nprobe, es, page, max_pages, scale, slot=0):
+                 ret_tok_off, row_src, meta, nprobe, es, page, max_pages, scale, slot=0, ret_start=None):
     """Centroid scoring + retrieval/estimation selection + token layout.  `slot` names the
-    scratch area: calls that may run concurrently (different streams) must use different slots."""
+    scratch area: calls that may run concurrently (different streams) must use different slots.
+    The layout goes out as a row table (row_src), as rank tables (ret_tok_off + ret_start), or both."""
     BG, gs, D = q.shape
     nc = centroids.shape[1]
     nb = lib().ri_score_select_workspace_bytes(BG, gs, nc)
     ws = _workspace(nb, q.device, f"score{slot}")
     check(lib().ri_score_select(_p(q), _p(centroids), _p(mask), _p(cluster_size_i32), _p(cluster_start),
                                 _p(logits), _p(dist), _p(cI), _p(ret_ids), _p(est_ids), _p(ret_tok_off),
-                                _p(row_src), 0 if row_src is None else row_src.shape[1], _p(meta), BG, gs, nc,
+                                _p(ret_start), _p(row_src), 0 if row_src is None else row_src.shape[1], _p(meta),
+                                BG, gs, nc,
                                 nprobe, es, page, max_pages, float(scale), _p(ws), ws.numel(), _stream()),
           "score_select")
 
@@ -256,16 +258,19 @@ def score_logits(q, centroids, logits, scale, slot=0):
 
 
 def wave_attention(q, steady_k, steady_v, static_len, store_k, store_v, row_src, meta, est_ids, logits,
-                   value_sum, cluster_size_bf16, out, valid_lengths, es, scale, slot=0):
+                   value_sum, cluster_size_bf16, out, valid_lengths, es, scale, slot=0, ret_tok_off=None,
+                   ret_start=None):
     """Attention over steady zone + retrieved clusters (read in place) + estimation zone.
-    `slot`: scratch area, one per concurrent call."""
+    The retrieved rows come from a row table (row_src) or, with row_src None, from the rank tables
+    ret_tok_off [BG, np+1] and ret_start [BG, np].  `slot`: scratch area, one per concurrent call."""
     BG, gs, D = q.shape
     nc = value_sum.shape[1]
     nb = lib().ri_wave_attention_workspace_bytes(BG, gs)
     ws = _workspace(nb, q.device, f"attn{slot}")
     check(lib().ri_wave_attention(_p(q), _p(steady_k), _p(steady_v), steady_k.shape[-2], static_len, _p(store_k),
-                                  _p(store_v), store_k.shape[-2], _p(row_src), row_src.shape[1], _p(meta),
-                                  _p(est_ids), _p(logits), _p(value_sum), _p(cluster_size_bf16), _p(out),
+                                  _p(store_v), store_k.shape[-2], _p(row_src),
+                                  0 if row_src is None else row_src.shape[1], _p(ret_tok_off), _p(ret_start),
+                                  0 if ret_start is None else ret_start.shape[1], _p(meta), _p(est_ids), _p(logits), _p(value_sum), _p(cluster_size_bf16), _p(out),
                                   _p(valid_lengths), BG, gs, nc, es, float(scale), _p(ws), ws.numel(), _stream()),
           "wave_attention")
 

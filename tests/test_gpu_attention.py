@@ -150,6 +150,19 @@ def test_wave_attention(dev, BG, gs, nc, nprobe, es, static_len, seed):
                            rows, meta, est if es else None, logits if es else None, vsum.to(dev),
                            size_bf.to(dev), out, vl, es, scale)
     torch.cuda.synchronize()
+    # the same through the rank tables (token prefix + first store row per rank) instead of the row table
+    rst = torch.empty(BG, nprobe, dtype=torch.int32, device=dev)
+    out_t = torch.empty_like(out)
+    kernels.score_select(qd, cent.to(dev), mask.to(torch.uint8).to(dev), size.to(dev), start.to(dev), logits, None,
+                         None, ret, est if es else None, off, None, meta, nprobe, es, page, max_pages, scale,
+                         ret_start=rst)
+    kernels.wave_attention(qd, steady_k.to(dev), steady_v.to(dev), static_len, store_k.to(dev), store_v.to(dev),
+                           None, meta, est if es else None, logits if es else None, vsum.to(dev),
+                           size_bf.to(dev), out_t, vl, es, scale, ret_tok_off=off, ret_start=rst)
+    torch.cuda.synchronize()
+    # (the two modes may split the rows differently: equal up to rounding, both checked against the oracle)
+    assert float((out_t.float() - out.float()).abs().max()) <= 2e-3
+    assert torch.equal(rst.cpu().long(), torch.gather(start.long(), 1, ret.cpu().long()))
     ret_c, est_c, lg = ret.cpu().long(), est.cpu()[:, :es].long(), logits.cpu()
     kept, offs = scoring.retrieval_layout(ret_c, size, page, max_pages)
     assert torch.equal(vl.cpu().long(), static_len + offs[:, -1])
@@ -167,3 +180,4 @@ def test_wave_attention(dev, BG, gs, nc, nprobe, es, static_len, seed):
             po, pl = eo.to(torch.bfloat16), el.float()   # the reference hands es_out over in bf16
         ref[b] = attention.weighted_flash_decoding(q[b:b + 1], kk, vv, None, po, pl)[0][0]
     _close(out.cpu(), ref)
+    _close(out_t.cpu(), ref)
