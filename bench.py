@@ -25,7 +25,7 @@ HBM_PEAK = 8.0e12  # bytes/s, MI355X
 # HBM bytes per attend_kernel launch from rocprofv3 counter runs of this script (FETCH_SIZE and
 # WRITE_SIZE, each scaled by what the counter reads for the known-size copy of --copy-probe);
 # the summaries are kept under profiles/.
-MEASURED_TRAFFIC = {"c2": int((31733.8 * 2.000 + 1201.0 * 1.000) * 1024)}
+MEASURED_TRAFFIC = {"c2": int((31707.4 * 2.000 + 1201.1 * 1.000) * 1024)}
 
 CONFIGS = {
     # name: batch, kv heads, group size, clustered tokens, mixture centres, centroids, segments, outliers, layers
@@ -312,6 +312,35 @@ def main():
     torch.cuda.synchronize()
     t_step = (time.perf_counter() - t0) / args.steps
 
+    # the dominant kernel's duration inside the replayed step: the same layer cycle without its launch
+    # (score_kernel + dist_kernel + select_kernel only), both cycles timed by one event pair each on the
+    # launch stream; the difference is attend_kernel plus the gap in front of it
+    t_attn_in_step = None
+    if graphs is not None:
+        sel_graphs = []
+        for l in range(L):
+            gr = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(gr):
+                cache._select(queries[l], l, l % 2, True)
+            sel_graphs.append(gr)
+        torch.cuda.synchronize()
+        e0, e1, e2 = (torch.cuda.Event(enable_timing=True) for _ in range(3))
+        best = [float("inf"), float("inf")]
+        for _ in range(3):
+            for i in range(args.warmup):
+                run(i)
+            e0.record()
+            for i in range(args.steps):
+                graphs[i % L][0].replay()
+            e1.record()
+            for i in range(args.steps):
+                sel_graphs[i % L].replay()
+            e2.record()
+            torch.cuda.synchronize()
+            best = [min(best[0], e0.elapsed_time(e1)), min(best[1], e1.elapsed_time(e2))]
+        t_attn_in_step = (best[0] - best[1]) * 1e-3 / args.steps
+        t_select_in_step = best[1] * 1e-3 / args.steps
+
     # per-kernel pass: the same layer cycle launched eagerly, one event pair around each entry point's
     # launches on the launch stream (cold caches as in the timed region: every step is another layer)
     from retrievalattention_amd import kernels, _lib
@@ -370,13 +399,19 @@ def main():
         },
     }
     # dominant kernel: attend_kernel, the one launch of ri_wave_attention (longest kernel, and the one that
-    # moves the K/V bytes).  Its event time includes the dispatch of the launch; null_launch_us is what
-    # the same event pair reads around an empty kernel.
+    # moves the K/V bytes).  Its duration is taken inside the replayed step (step cycle minus the cycle
+    # without it); an event pair around one eager launch also counts the dispatch of the launch
+    # (eager_event_us; null_launch_us is what the same pair reads around an empty kernel).
+    t_dom = t_attn_in_step if t_attn_in_step else t_attn
     result["roofline"] = {"bound": "hbm", "kernel": "attend_kernel (ri_wave_attention)",
-                          "achieved": attn_bytes / t_attn / 1e9, "peak": HBM_PEAK / 1e9, "unit": "GB/s",
-                          "frac": attn_bytes / t_attn / HBM_PEAK, "traffic": MEASURED_TRAFFIC.get(args.config),
-                          "launch_us": t_attn * 1e6, "null_launch_us": t_null * 1e6,
-                          "algorithmic_bytes": attn_bytes, "launches_timed": n_k}
+                          "achieved": attn_bytes / t_dom / 1e9, "peak": HBM_PEAK / 1e9, "unit": "GB/s",
+                          "frac": attn_bytes / t_dom / HBM_PEAK, "traffic": MEASURED_TRAFFIC.get(args.config),
+                          "launch_us": t_dom * 1e6, "eager_event_us": t_attn * 1e6, "null_launch_us": t_null * 1e6,
+                          "algorithmic_bytes": attn_bytes,
+                          "launches_timed": args.steps if t_attn_in_step else n_k}
+    if t_attn_in_step:
+        result["stages"]["score_select"]["us_in_step"] = t_select_in_step * 1e6
+        result["stages"]["wave_attention"]["us_in_step"] = t_attn_in_step * 1e6
     if not args.no_kmeans:
         result["prefill_kmeans"] = bench_kmeans(cfg, dev)
     if not args.no_cpu_baseline:
