@@ -4,7 +4,11 @@ TEST INFRASTRUCTURE ONLY.  Nothing under this package is part of the product: it
 checker that tests/, __graft_entry__.smoke() and the cpu_baseline leg of bench.py compare the
 HIP kernels against.  The product (retrievalattention_amd/) never imports it.
 
-Every function cites the reference file:line it follows.  How each one is pinned:
+Every function cites the reference file:line it follows.  The reference stores no golden vectors
+for this path; tests/golden/known_answers.json holds hand-worked known answers for every part below
+(initial tokens, a clustering followed by hand, softmax cases in closed form, ties and masked clusters
+in the selection, the buffer cut-off, a block cache trace, rational attention results), derived in
+tests/golden/make_known_answers.py without this package.  How each function is pinned:
 
   scoring.batch_gemm_softmax      the reference's own test oracle bmm -> /sqrt(d) -> softmax
                                   (library/retroinfer/test/test_batch_gemm_softmax.py:9-18, atol 1e-3)
