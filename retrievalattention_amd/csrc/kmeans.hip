@@ -5,9 +5,12 @@
 #include "ri_common.h"
 
 typedef float f32x16_t __attribute__((ext_vector_type(16)));
+typedef __attribute__((address_space(3))) void* km_lds_ptr;
+typedef const __attribute__((address_space(1))) void* km_glb_ptr;
 
-#define KM_CT 64          // centroid rows per LDS tile (two 32-row MFMA halves)
-#define KM_ROW_U16 136    // padded LDS row (272 bytes) to spread ds_read_b128 over the banks
+#ifndef KM_CT
+#define KM_CT 128         // centroid rows per LDS tile (32-row MFMA sub-tiles)
+#endif
 #ifndef KM_TT
 #define KM_TT 4           // 32-token MFMA columns per wave, held in registers
 #endif
@@ -15,7 +18,15 @@ typedef float f32x16_t __attribute__((ext_vector_type(16)));
 #define KM_WAVES 4        // waves per workgroup sharing one centroid tile
 #endif
 #define KM_WG_TOKENS (KM_WAVES * 32 * KM_TT)
-#define KM_PIECES ((KM_CT * 16 + KM_WAVES * 64 - 1) / (KM_WAVES * 64))  // 16-byte tile pieces per thread
+static_assert(KM_CT % (4 * KM_WAVES) == 0 && KM_CT % 32 == 0, "a tile is whole 1 KiB wave loads and whole sub-tiles");
+
+// 16 bytes per lane from global memory straight into LDS: lane l lands at lds_base + 16 l
+// (lds_base: byte address inside the workgroup's LDS, the same in every lane).  The wait for the
+// data is the caller's (s_waitcnt vmcnt): issued as inline assembly so that LDS reads of other
+// buffers are not made to wait for it.
+__device__ __forceinline__ void km_lds_dma16(const void* g, uint32_t lds_base) {
+  asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" : : "v"(g), "s"(lds_base) : "memory", "m0");
+}
 
 // first data row of problem p: problems are `seg` consecutive N-row slices of each head
 __device__ __forceinline__ size_t km_row0(int p, int seg, int64_t head_rows, int N) {
@@ -25,19 +36,20 @@ __device__ __forceinline__ size_t km_row0(int p, int seg, int64_t head_rows, int
 // ------------------------------------------------------------------------------------
 // assign: grid (ceil(N / KM_WG_TOKENS), P), KM_WAVES waves; a wave keeps KM_TT columns of 32
 // tokens in registers for the whole kernel (KM_TT independent accumulator chains).  Centroid
-// tiles of 64 rows go through two LDS buffers shared by all waves of the workgroup: the next
-// tile's global loads are issued before the MFMAs of the current one and stored to the other
-// buffer after them, one barrier per tile.  (4 tokens columns x 4 waves measured fastest on
-// the full-size pass against 2x4, 2x8, 2x12, 3x8 with clocks warmed up and runs interleaved.)
+// tiles of KM_CT rows go through two LDS buffers shared by all waves of the workgroup: the next
+// tile is requested from global memory straight into the other buffer (no registers, no LDS
+// stores) before the MFMAs of the current one, one wait and one barrier per tile.  (4 token
+// columns x 4 waves measured fastest on the full-size pass against 2x4, 2x8, 2x12, 3x8, and
+// 128-row tiles against 64 and 256, with clocks warmed up and runs interleaved.)
 // MFMA 32x32x16: A = centroid rows, B = token columns; accumulator i of lane l is
 // row (i/4)*8 + (l/32)*4 + i%4, column l%32.  nc is a multiple of 32; the last tile may hold
-// one half only.
+// fewer sub-tiles.
 // ------------------------------------------------------------------------------------
 __global__ __launch_bounds__(KM_WAVES * 64) void km_assign_kernel(const uint16_t* __restrict__ data,
                                                                   const uint16_t* __restrict__ cent,
                                                                   int32_t* __restrict__ assign, int N, int nc,
                                                                   int seg, int64_t head_rows) {
-  __shared__ __attribute__((aligned(16))) uint16_t sh_c[2][KM_CT][KM_ROW_U16];
+  __shared__ __attribute__((aligned(1024))) uint16_t sh_c[2][KM_CT][RI_DIM];
   const int p = blockIdx.y;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int r = lane & 31, hh = lane >> 5;
@@ -45,24 +57,24 @@ __global__ __launch_bounds__(KM_WAVES * 64) void km_assign_kernel(const uint16_t
   const uint16_t* dp = data + km_row0(p, seg, head_rows, N) * RI_DIM;
   const uint16_t* cp = cent + (size_t)p * nc * RI_DIM;
 
-  // this thread's 16-byte pieces of a tile: piece index threadIdx.x + u * threads -> (row, column piece)
-  uint4 pf[KM_PIECES];
-  auto tile_load = [&](int ct) {
+  // A tile goes from global memory straight into LDS, 16 bytes per lane and 1 KiB (four rows)
+  // per wave instruction: lane l lands at byte l * 16 of the instruction's LDS window, and which
+  // global piece it fetches is free, so the 16-byte pieces of row w are stored at piece ^ (w & 15):
+  // the 16 lanes of a ds_read_b128 phase then hit 16 different piece positions (all 64 banks once).
+  const int ld_row = lane >> 4, ld_piece = lane & 15;
+  const uint32_t sh_base = (uint32_t)(uintptr_t)(km_lds_ptr)&sh_c[0][0][0];
+  auto tile_load = [&](int ct, int buf) {
 #pragma unroll
-    for (int u = 0; u < KM_PIECES; ++u) {
-      const int idx = threadIdx.x + u * (KM_WAVES * 64);
-      const int row = ct + (idx >> 4);
-      pf[u] = (idx < KM_CT * 16 && row < nc) ? ri_ld16(cp + (size_t)row * RI_DIM + (idx & 15) * 8) : ri_zero16();
+    for (int u = 0; u < KM_CT / 4 / KM_WAVES; ++u) {
+      const int row4 = (wave + u * KM_WAVES) * 4;      // first of the four rows of this instruction
+      const int row = row4 + ld_row;
+      if (ct + row4 < nc) {  // uniform: nc is a multiple of 32
+        const uint16_t* g = cp + (size_t)(ct + row) * RI_DIM + ((ld_piece ^ (row & 15)) * 8);
+        km_lds_dma16(g, __builtin_amdgcn_readfirstlane(sh_base + (uint32_t)((buf * KM_CT + row4) * RI_DIM * 2)));
+      }
     }
   };
-  auto tile_store = [&](int buf) {
-#pragma unroll
-    for (int u = 0; u < KM_PIECES; ++u) {
-      const int idx = threadIdx.x + u * (KM_WAVES * 64);
-      if (idx < KM_CT * 16) *reinterpret_cast<uint4*>(&sh_c[buf][idx >> 4][(idx & 15) * 8]) = pf[u];
-    }
-  };
-  tile_load(0);
+  tile_load(0, 0);
   uint4 b[KM_TT][8];
 #pragma unroll
   for (int tt = 0; tt < KM_TT; ++tt) {
@@ -71,7 +83,13 @@ __global__ __launch_bounds__(KM_WAVES * 64) void km_assign_kernel(const uint16_t
 #pragma unroll
     for (int kk = 0; kk < 8; ++kk) b[tt][kk] = (tok < N) ? ri_ld16(q + kk * 16) : ri_zero16();
   }
-  tile_store(0);
+  // (the token registers are consumed here so that the compiler's own wait for their loads sits
+  // in front of the loop and not inside it, where it would also wait for the tile in flight)
+#pragma unroll
+  for (int tt = 0; tt < KM_TT; ++tt)
+#pragma unroll
+    for (int kk = 0; kk < 8; ++kk) asm volatile("" : : "v"(b[tt][kk].x));
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   __syncthreads();
 
   float best[KM_TT];
@@ -84,10 +102,10 @@ __global__ __launch_bounds__(KM_WAVES * 64) void km_assign_kernel(const uint16_t
   int buf = 0;
   for (int ct = 0; ct < nc; ct += KM_CT, buf ^= 1) {
     const int nxt = ct + KM_CT;
-    if (nxt < nc) tile_load(nxt);
+    if (nxt < nc) tile_load(nxt, buf ^ 1);
 #pragma unroll
-    for (int half = 0; half < 2; ++half) {
-      if (ct + half * 32 < nc) {  // uniform: only the last tile can lack its second half
+    for (int half = 0; half < KM_CT / 32; ++half) {
+      if (ct + half * 32 < nc) {  // uniform: only the last tile can lack sub-tiles
         f32x16_t acc[KM_TT];
 #pragma unroll
         for (int tt = 0; tt < KM_TT; ++tt)
@@ -95,7 +113,7 @@ __global__ __launch_bounds__(KM_WAVES * 64) void km_assign_kernel(const uint16_t
           for (int i = 0; i < 16; ++i) acc[tt][i] = 0.f;
 #pragma unroll
         for (int kk = 0; kk < 8; ++kk) {
-          const uint4 a = *reinterpret_cast<const uint4*>(&sh_c[buf][half * 32 + r][kk * 16 + hh * 8]);
+          const uint4 a = *reinterpret_cast<const uint4*>(&sh_c[buf][half * 32 + r][((kk * 2 + hh) ^ (r & 15)) * 8]);
 #pragma unroll
           for (int tt = 0; tt < KM_TT; ++tt)
             acc[tt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ri_as_bf16x8(a), ri_as_bf16x8(b[tt][kk]), acc[tt], 0, 0,
@@ -103,7 +121,7 @@ __global__ __launch_bounds__(KM_WAVES * 64) void km_assign_kernel(const uint16_t
         }
         // argmax epilogue: the lane's 16 scores are in ascending row order, so the first score
         // equal to their maximum is the lowest row; the index search only runs when some lane
-        // of the wave improves on its best (rare once a few tiles have gone by)
+        // of the wave improves on its best (about half of the sub-tiles of a full-size pass)
 #pragma unroll
         for (int tt = 0; tt < KM_TT; ++tt) {
           float m = acc[tt][0];
@@ -122,7 +140,7 @@ __global__ __launch_bounds__(KM_WAVES * 64) void km_assign_kernel(const uint16_t
         }
       }
     }
-    if (nxt < nc) tile_store(buf ^ 1);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
   }
 #pragma unroll
