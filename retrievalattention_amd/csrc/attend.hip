@@ -615,6 +615,7 @@ extern "C" int ri_weighted_flash_decoding(const void* q, const void* k, const vo
                                           int S, int64_t kv_stride, float scale, void* workspace,
                                           size_t workspace_bytes, ri_stream_t stream) {
   if (!q || !k || !v || !out || !workspace) return RI_ERR_ARG;
+  if (ri_any_misaligned16(q, k, v, weight, prev_out, out, workspace)) return RI_ERR_ARG;
   if (BG <= 0 || BG > RI_MAX_GROUPS || gs <= 0 || gs > 16 || S < 0 || kv_stride < S) return RI_ERR_ARG;
   if ((prev_out == nullptr) != (prev_lse == nullptr)) return RI_ERR_ARG;
   if (workspace_bytes < attn_workspace_bytes(BG, gs)) return RI_ERR_WORKSPACE;
@@ -650,6 +651,7 @@ extern "C" int ri_wave_attention(const void* q, const void* steady_k, const void
                                  void* out, int32_t* valid_lengths, int BG, int gs, int nc, int es,
                                  float scale, void* workspace, size_t workspace_bytes, ri_stream_t stream) {
   if (!q || !steady_k || !steady_v || !store_k || !store_v || !meta || !out || !workspace) return RI_ERR_ARG;
+  if (ri_any_misaligned16(q, steady_k, steady_v, store_k, store_v, value_sum, out, workspace)) return RI_ERR_ARG;
   if (!row_src && (!ret_tok_off || !ret_start || np <= 0 || np > 1023)) return RI_ERR_ARG;
   if (BG <= 0 || BG > RI_MAX_GROUPS || gs <= 0 || gs > 16 || static_len < 0 || static_len > steady_stride ||
       es < 0 || nc <= 0)
@@ -699,6 +701,7 @@ extern "C" int ri_buffer_attention(const void* q, const void* buf_k, const void*
                                    void* out, int BG, int gs, int nc, int es, float scale, void* workspace,
                                    size_t workspace_bytes, ri_stream_t stream) {
   if (!q || !buf_k || !buf_v || !cache_seqlens || !out || !workspace) return RI_ERR_ARG;
+  if (ri_any_misaligned16(q, buf_k, buf_v, value_sum, out, workspace)) return RI_ERR_ARG;
   if (BG <= 0 || BG > RI_MAX_GROUPS || gs <= 0 || gs > 16 || max_len <= 0 || max_len > buf_stride || es < 0 ||
       nc <= 0)
     return RI_ERR_ARG;

@@ -98,6 +98,7 @@ extern "C" int ri_gather_copy_vectors(const void* src_keys, void* dst_keys, cons
                                       const int64_t* idx, int groups, int data_length, int buffer_length,
                                       int index_size, int copy_start, int copy_num, ri_stream_t stream) {
   if (!src_keys || !dst_keys || !src_values || !dst_values || !src_meta || !dst_meta || !idx) return RI_ERR_ARG;
+  if (ri_any_misaligned16(src_keys, dst_keys, src_values, dst_values)) return RI_ERR_ARG;
   if (groups <= 0 || copy_num < 0 || copy_start < 0 || copy_start + copy_num > index_size ||
       copy_num > buffer_length)
     return RI_ERR_ARG;
@@ -121,6 +122,7 @@ extern "C" int ri_gather_copy_and_concat(const void* k1, const void* k2, const v
   if (!k1 || !k2 || !k3 || !kdst || !v1 || !v2 || !v3 || !vdst || !off2 || !sizes2 || !dst2 || !num2 ||
       !off3 || !sizes3 || !dst3 || !num3 || !valid_lengths)
     return RI_ERR_ARG;
+  if (ri_any_misaligned16(k1, k2, k3, kdst, v1, v2, v3, vdst)) return RI_ERR_ARG;
   if (groups <= 0 || copy_vectors1 < 0 || copy_vectors1 > data_length1 || copy_vectors1 > buffer_length ||
       offset_length <= 0)
     return RI_ERR_ARG;
@@ -140,6 +142,7 @@ extern "C" int ri_gather_copy_and_scatter(const void* ksrc, void* kcache, const 
                                           int data_length, int buffer_length, int offset_length,
                                           int s_copy_start, ri_stream_t stream) {
   if (!ksrc || !kcache || !vsrc || !vcache || !src_off || !sizes || !dst_block || !num) return RI_ERR_ARG;
+  if (ri_any_misaligned16(ksrc, kcache, vsrc, vcache)) return RI_ERR_ARG;
   if (groups <= 0 || offset_length <= 0 || s_copy_start < 0) return RI_ERR_ARG;
   int x = offset_length / 8 + 1;
   if (x > 32) x = 32;

@@ -499,6 +499,7 @@ static int km_check(int P, int N, int nc) {
 extern "C" int ri_kmeans_assign(const void* data, const void* centroids, int32_t* assign, int P, int N,
                                 int nc, int seg, int64_t head_rows, ri_stream_t stream) {
   if (!data || !centroids || !assign) return RI_ERR_ARG;
+  if (ri_any_misaligned16(data, centroids)) return RI_ERR_ARG;
   int rc = km_check(P, N, nc);
   if (rc) return rc;
   if (nc % 32 != 0 || seg <= 0 || P % seg != 0) return RI_ERR_ARG;
@@ -598,6 +599,7 @@ extern "C" int ri_kmeans_update(const void* data, const int32_t* counts, const i
                                 int64_t head_rows, int normalize, void* workspace, size_t workspace_bytes,
                                 ri_stream_t stream) {
   if (!data || !counts || !offsets || !members || !centroids || !workspace) return RI_ERR_ARG;
+  if (ri_any_misaligned16(data, centroids, workspace)) return RI_ERR_ARG;
   int rc = km_check(P, N, nc);
   if (rc) return rc;
   if (seg <= 0 || P % seg != 0) return RI_ERR_ARG;
@@ -609,6 +611,7 @@ extern "C" int ri_kmeans_value_sum(const void* values, const int32_t* counts, co
                                    const int32_t* members, void* value_sum, int P, int N, int nc, void* workspace,
                                    size_t workspace_bytes, ri_stream_t stream) {
   if (!values || !counts || !offsets || !members || !value_sum || !workspace) return RI_ERR_ARG;
+  if (ri_any_misaligned16(values, value_sum, workspace)) return RI_ERR_ARG;
   int rc = km_check(P, N, nc);
   if (rc) return rc;
   return km_reduce<false>(values, counts, offsets, members, value_sum, P, N, nc, 1, (int64_t)N, 0, workspace,
@@ -619,6 +622,7 @@ extern "C" int ri_permute_rows(const void* in, const int32_t* members, void* out
                                int64_t in_stride_rows, int64_t out_stride_rows, ri_stream_t stream) {
   if (!in || !members || !out || P <= 0 || N <= 0 || P > 65535 || in_stride_rows < N || out_stride_rows < N)
     return RI_ERR_ARG;
+  if (ri_any_misaligned16(in, out)) return RI_ERR_ARG;
   km_permute_kernel<<<dim3((N + 15) / 16, P), 256, 0, (hipStream_t)stream>>>(
       (const uint4*)in, members, (uint4*)out, N, in_stride_rows, out_stride_rows);
   RI_HIP_CHECK_LAUNCH();

@@ -49,6 +49,14 @@ __host__ __device__ __forceinline__ uint32_t ri_bf16_sort_key(uint16_t b) {
   return (b & 0x8000u) ? (uint32_t)(~b & 0xffffu) : (uint32_t)(b | 0x8000u);
 }
 
+// Rows of bf16 matrices are read and written 16 bytes at a time: their base pointers must be
+// 16-byte aligned (a null pointer counts as aligned: optional arguments are checked elsewhere).
+static inline bool ri_misaligned16(const void* p) { return ((uintptr_t)p & 15u) != 0; }
+template <typename... P>
+static inline bool ri_any_misaligned16(P... p) {
+  return (ri_misaligned16((const void*)p) || ...);
+}
+
 #define RI_HIP_CHECK_LAUNCH()                         \
   do {                                                \
     hipError_t e__ = hipGetLastError();               \

@@ -161,6 +161,7 @@ extern "C" int ri_batch_gemm_softmax(const void* A, const void* B, void* D, floa
                                      void* Softmax, int batch_count, int m, int n, int k, float alpha,
                                      float beta, ri_stream_t stream) {
   if (!A || !B || !D || !Norm || !Sum || !Softmax || beta != 0.f) return RI_ERR_ARG;
+  if (ri_any_misaligned16(A, B, D, Softmax)) return RI_ERR_ARG;
   int rc = check_score_shape(batch_count, m, n, k);
   if (rc) return rc;
   hipStream_t s = (hipStream_t)stream;

@@ -387,6 +387,7 @@ extern "C" int ri_score_select(const void* q, const void* centroids, const uint8
                                int es, int page, int max_pages, float scale, void* workspace,
                                size_t workspace_bytes, ri_stream_t stream) {
   if (!q || !centroids || !logits || !ret_ids || !workspace) return RI_ERR_ARG;
+  if (ri_any_misaligned16(q, centroids, logits, workspace)) return RI_ERR_ARG;
   if (BG <= 0 || gs <= 0 || gs > 16 || nc <= 0 || (nc % 8) != 0) return RI_ERR_ARG;
   if (np <= 0 || np > 1023 || es < 0 || np + es > nc || nc > 65536) return RI_ERR_ARG;
   if (es > 0 && !est_ids) return RI_ERR_ARG;
@@ -423,6 +424,7 @@ extern "C" int ri_score_select(const void* q, const void* centroids, const uint8
 extern "C" int ri_score_logits(const void* q, const void* centroids, float* logits, int BG, int gs, int nc,
                                float scale, void* workspace, size_t workspace_bytes, ri_stream_t stream) {
   if (!q || !centroids || !logits || !workspace) return RI_ERR_ARG;
+  if (ri_any_misaligned16(q, centroids, logits, workspace)) return RI_ERR_ARG;
   if (BG <= 0 || gs <= 0 || gs > 16 || nc <= 0 || (nc % 4) != 0) return RI_ERR_ARG;
   if (workspace_bytes < ri_score_select_workspace_bytes(BG, gs, nc)) return RI_ERR_WORKSPACE;
   const int ntiles = (nc + RI_SCORE_TILE - 1) / RI_SCORE_TILE;

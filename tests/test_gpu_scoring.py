@@ -157,3 +157,21 @@ def test_score_select_rejects_bad_shapes(dev):
     with pytest.raises(RuntimeError, match="invalid argument"):
         kernels.score_select(q.to(dev), cent.to(dev), None, None, None, logits, None, None, ret, None, None, None,
                              None, 80, 0, 8, 16, 1.0)   # nprobe > nc
+
+
+def test_misaligned_rows_are_rejected(dev):
+    """Rows are read 16 bytes at a time: a matrix that does not start on a 16-byte boundary is an
+    invalid argument (nothing is launched)."""
+    from retrievalattention_amd import kernels
+    q, cent = _mixture(1, 4, 64, 0)
+    flat = torch.empty(64 * 128 + 8, dtype=torch.bfloat16, device=dev)
+    shifted = flat[1:1 + 64 * 128].view(1, 64, 128)          # 2 bytes off
+    shifted.copy_(cent.to(dev))
+    logits = torch.empty(1, 4, 64, dtype=torch.float32, device=dev)
+    ret = torch.empty(1, 4, dtype=torch.int32, device=dev)
+    with pytest.raises(RuntimeError, match="invalid argument"):
+        kernels.score_select(q.to(dev), shifted, None, None, None, logits, None, None, ret, None, None, None,
+                             None, 4, 0, 8, 16, 1.0)
+    k = torch.empty(1 * 40 * 128 + 8, dtype=torch.bfloat16, device=dev)[1:1 + 40 * 128].view(1, 40, 1, 128)
+    with pytest.raises(RuntimeError, match="invalid argument"):
+        kernels.weighted_flash_decoding(q.view(1, 1, 4, 128).to(dev), k, k)
