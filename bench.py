@@ -44,7 +44,7 @@ def log(*a):
     print(*a, file=sys.stderr, flush=True)
 
 
-def build_cache(cfg, L, dev, residency="device", block_cache="device"):
+def build_cache(cfg, L, dev, residency="device", block_cache="device", estimate_next=False):
     from retrievalattention_amd import synth
     from retrievalattention_amd.cache_hub import retroinfer_cache
     B, Hkv, gs, N = cfg["B"], cfg["Hkv"], cfg["gs"], cfg["N"]
@@ -58,7 +58,7 @@ def build_cache(cfg, L, dev, residency="device", block_cache="device"):
         max_new_length=new, static_pattern_start=synth.STEADY_START, static_pattern_end=synth.STEADY_END, core=8,
         n_centroids=cfg["nc"], n_segment=cfg["S"], nprobe=nprobe, max_compute_cluster_num=nprobe + es,
         cache_unit_size=8, cache_cluster_num=3 * nprobe, num_gpus=1, model_size=0, kv_residency=residency,
-        block_cache=block_cache)
+        block_cache=block_cache, use_cluster_estimation=estimate_next)
     queries = []
     t0 = time.time()
     for l in range(L):
@@ -172,6 +172,52 @@ def cpu_baseline(cache, cfg, queries, nprobe, es, static_len, max_seconds=30.0):
     return times[len(times) // 2], len(times), ref
 
 
+def bench_estimate_next(args, cache, queries, outs, L, static_len):
+    """The reference's use_cluster_estimation mode over the device-resident store: layers 0 and 1 choose
+    their zones from their own query; every later layer's zones are chosen at the end of the layer before
+    it, from a predicted query.  The bench predicts perfectly (the next layer's true query), so
+    the outputs must agree with those of the plain step; one pass over the L layers is one decoded token."""
+    def step(l):
+        return cache._compute(queries[l], l, queries[l + 1] if l + 1 < L else None, static_len)
+
+    for l in range(L):
+        o = step(l)
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for l in range(L):
+            step(l)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graphs = []
+    for l in range(L):
+        gr = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(gr):
+            o = step(l)
+        graphs.append((gr, o))
+    torch.cuda.synchronize()
+    for l in range(L):
+        graphs[l][0].replay()
+    torch.cuda.synchronize()
+    # same zones as the plain step; the estimation zone's scores come from another accumulation order
+    for l in range(L):
+        d = (graphs[l][1].float() - outs[l].float()).abs()
+        if float(d.max()) > 2e-2 or float(d.mean()) > 2e-3:
+            sys.exit(f"next-layer estimation: layer {l} differs from the plain step (max-abs {float(d.max())})")
+    for i in range(args.warmup):
+        graphs[i % L][0].replay()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(args.steps):
+        graphs[i % L][0].replay()
+    torch.cuda.synchronize()
+    t = (time.perf_counter() - t0) / args.steps
+    return {"us_per_layer_step": t * 1e6, "layers_per_token": L,
+            "note": "zones of layer l+1 chosen at the end of layer l from the (here exact) "
+                    "predicted query; layers 0 and 1 select for themselves; outputs checked against the plain step"}
+
+
 def bench_host(args, cfg, cache, queries, L, nprobe, es, static_len):
     """Host-resident clustered K/V: the reference's operator sequence (score+select, id copy to the
     host, block-cache look-up on the worker pool, gather of misses over the host link and hits
@@ -240,6 +286,9 @@ def main():
                     help="with --residency host: block cache manager as a kernel (HIP graph replays) or the "
                          "reference's worker threads (eager launches)")
     ap.add_argument("--no-kmeans", action="store_true", help="skip the prefill clustering measurement")
+    ap.add_argument("--estimate-next", action="store_true",
+                    help="also measure the step with next-layer cluster estimation (zones of layer l+1 chosen "
+                         "at the end of layer l from a predicted query)")
     ap.add_argument("--copy-probe", action="store_true",
                     help="also run 8 device copies of 256 MiB (a known-size kernel to scale rocprofv3 byte counters by)")
     args = ap.parse_args()
@@ -260,7 +309,8 @@ def main():
             b.copy_(a)
         torch.cuda.synchronize()
         del a, b
-    cache, queries, nprobe, es = build_cache(cfg, L, dev, args.residency, args.block_cache)
+    est_next = args.residency == "device" and args.estimate_next and not args.no_graph and L >= 4
+    cache, queries, nprobe, es = build_cache(cfg, L, dev, args.residency, args.block_cache, est_next)
     static_len = cache.static_pattern_total  # 4 + 64 + the token being decoded (already counted)
     if args.residency == "host":
         return bench_host(args, cfg, cache, queries, L, nprobe, es, static_len)
@@ -412,6 +462,8 @@ def main():
     if t_attn_in_step:
         result["stages"]["score_select"]["us_in_step"] = t_select_in_step * 1e6
         result["stages"]["wave_attention"]["us_in_step"] = t_attn_in_step * 1e6
+    if est_next:
+        result["next_layer_estimation"] = bench_estimate_next(args, cache, queries, outs, L, static_len)
     if not args.no_kmeans:
         result["prefill_kmeans"] = bench_kmeans(cfg, dev)
     if not args.no_cpu_baseline:

@@ -43,7 +43,7 @@ enum {
 const char* ri_status_string(int status);
 int ri_last_hip_error(void);
 /* ABI version: bumped when a signature changes. */
-int ri_abi_version(void);   /* 2 */
+int ri_abi_version(void);   /* 3 */
 /* Launches an empty kernel on `stream`: lets a caller measure the per-dispatch overhead that
  * event timings of back-to-back launches include.  No counterpart in the reference. */
 int ri_null_launch(ri_stream_t stream);
@@ -140,6 +140,10 @@ int ri_weighted_flash_decoding(const void* q, const void* k, const void* v, cons
  *   row_src [BG, row_src_stride]: store row of every retrieved token; or NULL with ret_tok_off
  *   [BG, np+1] and ret_start [BG, np]: rank r's tokens are the store rows ret_start[r] + i
  *   meta, est_ids, logits: as written by ri_score_select (or meta by ri_lru_access_update)
+ *   est_centroids [BG, nc, 128] bf16: given instead of logits (exactly one of the two is NULL when
+ *   es > 0) when the zones were chosen from another query than q (next-layer cluster estimation,
+ *   cache_hub/retroinfer_cache.py:582-617): the estimation zone's scores are then computed inside
+ *   the launch from the centroid rows of est_ids
  *   value_sum [BG, nc, 128] bf16, cluster_size_bf16 [BG, nc] bf16 (estimation weights)
  *   es may be 0 (no estimation zone).  out [BG, gs, 128] bf16; valid_lengths [BG] int32 or
  *   NULL receives static_len + retrieved tokens (what gather_copy_and_concat reports).
@@ -150,7 +154,7 @@ int ri_wave_attention(const void* q, const void* steady_k, const void* steady_v,
                       const void* store_v, int64_t store_stride, const int32_t* row_src,
                       int row_src_stride, const int32_t* ret_tok_off, const int32_t* ret_start, int np,
                       const int32_t* meta, const int32_t* est_ids,
-                      const float* logits, const void* value_sum,
+                      const float* logits, const void* est_centroids, const void* value_sum,
                       const void* cluster_size_bf16, void* out, int32_t* valid_lengths,
                       int BG, int gs, int nc, int es, float scale, void* workspace,
                       size_t workspace_bytes, ri_stream_t stream);

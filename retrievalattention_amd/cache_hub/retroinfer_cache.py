@@ -4,7 +4,7 @@ attributes (cache_hub/retroinfer_cache.py of the reference), running on the gfx9
 Two residencies of the clustered K/V:
 
   "device"  every cluster's K/V stays in HBM in cluster-contiguous order.  A decode step is
-            two fused calls: score_select (scores, zones, row table) and wave_attention
+            two fused calls: score_select (scores, zones, rank tables) and wave_attention
             (steady zone + retrieved clusters read in place + estimation zone).  No host
             round trip, no execution buffer, no block cache.
   "host"    the reference's arrangement: clustered K/V in pinned host memory, an LRU block
@@ -615,24 +615,29 @@ class retroinfer_cache(KV_Cache):
                                   search_next):
         """Device residency with next-layer cluster estimation (reference: retroinfer_cache.py:565,
         582-595): from the third layer on the zones come from the query the previous layer
-        predicted; the estimation zone is scored with the true query, the retrieval zone is
-        attended exactly.  A device-resident store has no transfer to hide, so this mode exists for
-        behavioural parity, not speed: the next layer's zones are chosen after this layer's attention."""
+        predicted; the estimation zone is scored with the true query (inside the attention launch,
+        from the centroid rows), the retrieval zone is attended exactly.  A device-resident store has
+        no transfer to hide, so this mode exists for behavioural parity, not speed: the next layer's
+        zones are chosen after this layer's attention, on the same stream.  (Choosing them on a second
+        stream during the attention was measured slower, 66-72 us against 59 us per layer-step at the
+        benchmark shape: two branches inside a replayed graph cost more than the overlap gains.)"""
         BG, gs, D = self.batch_groups, self.group_size, self.head_dim
         es = self.es_cluster_num
         q = queries.view(BG, gs, D)
         if search_here:
             self._select(queries, layer_idx, buf, True, layout=buf)
-        elif es > 0:
-            kernels.score_logits(q, self.centroids[layer_idx], self.logits, self.RSQRT_DIM)
         ret_tok_off, ret_start, _, meta = self.layouts[buf]
         out = torch.empty((BG, gs, D), dtype=self.dtype, device=queries.device)
+        # zones from the layer's own query: its logits are at hand; zones from a predicted query: the
+        # estimation zone is scored with the true query inside the attention launch
+        own = search_here and es > 0
         kernels.wave_attention(
             q, self.steady_zone_keys[layer_idx], self.steady_zone_values[layer_idx], static_len,
             self.list_keys[layer_idx], self.list_values[layer_idx], None, meta,
-            self.est_ids[buf] if es > 0 else None, self.logits if es > 0 else None, self.value_sum[layer_idx],
+            self.est_ids[buf] if es > 0 else None, self.logits if own else None, self.value_sum[layer_idx],
             self.cluster_size[layer_idx], out, self.valid_lengths[buf], es, self.RSQRT_DIM,
-            ret_tok_off=ret_tok_off, ret_start=ret_start)
+            ret_tok_off=ret_tok_off, ret_start=ret_start,
+            est_centroids=self.centroids[layer_idx] if es > 0 and not own else None)
         if search_next:
             self._select(queries_next, layer_idx + 1, nbuf, True, layout=nbuf)
         return out.view(self.batch_size, 1, self.num_heads, D)

@@ -51,7 +51,8 @@ struct AttendParams {
   int weight_stride;
   // estimation rows
   const int32_t* est_ids;     // [BG, es]
-  const float* logits;        // [BG, gs, nc]
+  const float* logits;        // [BG, gs, nc] scores of the estimation rows, or null:
+  const uint16_t* est_cent;   // [BG, nc, 128] then the scores are computed here from the centroid rows
   const uint16_t* value_sum;  // [BG, nc, 128]
   const uint16_t* csize;      // [BG, nc] bf16
   int nc;
@@ -292,10 +293,13 @@ __global__ __launch_bounds__(256, GS_PAD == 16 ? 1 : 3) void attend_kernel(Atten
   float* wsh = sh_w[wave];
   const int lenB = P.lenB_ptr ? P.lenB_ptr[(size_t)g * P.lenB_ptr_stride] : P.lenB_const;
 
-  if (split < P.S_kv) {
+  // Estimation rows whose scores are not handed in are key/value rows of their own: key = centroid,
+  // value = value sum, weight = cluster size, located through the id list.
+  const bool est_split = split >= P.S_kv;
+  if (!est_split || P.est_cent) {
     // ---------------- key/value rows ----------------
     // rank tables (requested together with everything else the prologue loads: no dependent round trip)
-    const bool tab = P.ret_off != nullptr;
+    const bool tab = !est_split && P.ret_off != nullptr;
     // every global load of the prologue is requested before the first of them is consumed
     int t_off[4], t_st[4];
     if (tab) {
@@ -324,16 +328,22 @@ __global__ __launch_bounds__(256, GS_PAD == 16 ? 1 : 3) void attend_kernel(Atten
       }
     }
     // (the row count is consumed only now: the loads above went out together with its load)
-    const int total = P.lenA + lenB;
+    const int lenA = est_split ? 0 : P.lenA;
+    const int total = est_split ? P.es : P.lenA + lenB;
     int r0, r1;
-    wave_rows(total, P.S_kv * 4, split * 4 + wave, &r0, &r1);
+    if (est_split)
+      wave_rows(total, P.S_es * 4, (split - P.S_kv) * 4 + wave, &r0, &r1);
+    else
+      wave_rows(total, P.S_kv * 4, split * 4 + wave, &r0, &r1);
     const uint16_t* qrow = &sh_q[n % GS_PAD][h * 8];
     const uint16_t* kA = P.kA + (size_t)g * P.strideA * RI_DIM;
     const uint16_t* vA = P.vA + (size_t)g * P.strideA * RI_DIM;
-    const uint16_t* kB = P.kB + (size_t)g * P.strideB * RI_DIM;
-    const uint16_t* vB = P.vB + (size_t)g * P.strideB * RI_DIM;
-    const int32_t* rs = P.row_src ? P.row_src + (size_t)g * P.rs_stride : nullptr;
-    const uint16_t* wB = P.weightB ? P.weightB + (size_t)g * P.weight_stride : nullptr;
+    const uint16_t* kB = est_split ? P.est_cent + (size_t)g * P.nc * RI_DIM : P.kB + (size_t)g * P.strideB * RI_DIM;
+    const uint16_t* vB = est_split ? P.value_sum + (size_t)g * P.nc * RI_DIM : P.vB + (size_t)g * P.strideB * RI_DIM;
+    const int32_t* rs = est_split ? P.est_ids + (size_t)g * P.es
+                                  : (P.row_src ? P.row_src + (size_t)g * P.rs_stride : nullptr);
+    const uint16_t* wB = (!est_split && P.weightB) ? P.weightB + (size_t)g * P.weight_stride : nullptr;
+    const uint16_t* wsrc = est_split ? P.csize + (size_t)g * P.nc : nullptr;  // weight by source row
     const int r_first = ri_head_reg<GS_PAD>(h);
     bool q_ready = false;
     if (tab) {  // the tables are searched while the rows are located
@@ -349,10 +359,10 @@ __global__ __launch_bounds__(256, GS_PAD == 16 ? 1 : 3) void attend_kernel(Atten
         int d = -1;
         float w = 1.f;
         if (row < s1) {
-          if (row < P.lenA) {
+          if (row < lenA) {
             d = row | ATT_FLAG_A;
           } else {
-            const int rb = row - P.lenA;
+            const int rb = row - lenA;
             if (tab) {
               // the last rank whose first row is <= rb (ranks of empty clusters share a first row
               // with the next rank, which is the one found)
@@ -366,6 +376,7 @@ __global__ __launch_bounds__(256, GS_PAD == 16 ? 1 : 3) void attend_kernel(Atten
               d = rs ? rs[rb] : rb;
             }
             if (wB) w = ri_bf16_to_f32(wB[rb]);
+            if (wsrc) w = ri_bf16_to_f32(wsrc[d]);
           }
         }
         dsc[i] = d;
@@ -647,16 +658,18 @@ extern "C" int ri_wave_attention(const void* q, const void* steady_k, const void
                                  const void* store_v, int64_t store_stride, const int32_t* row_src,
                                  int row_src_stride, const int32_t* ret_tok_off, const int32_t* ret_start, int np,
                                  const int32_t* meta, const int32_t* est_ids,
-                                 const float* logits, const void* value_sum, const void* cluster_size_bf16,
-                                 void* out, int32_t* valid_lengths, int BG, int gs, int nc, int es,
-                                 float scale, void* workspace, size_t workspace_bytes, ri_stream_t stream) {
+                                 const float* logits, const void* est_centroids, const void* value_sum,
+                                 const void* cluster_size_bf16, void* out, int32_t* valid_lengths, int BG, int gs,
+                                 int nc, int es, float scale, void* workspace, size_t workspace_bytes,
+                                 ri_stream_t stream) {
   if (!q || !steady_k || !steady_v || !store_k || !store_v || !meta || !out || !workspace) return RI_ERR_ARG;
-  if (ri_any_misaligned16(q, steady_k, steady_v, store_k, store_v, value_sum, out, workspace)) return RI_ERR_ARG;
+  if (ri_any_misaligned16(q, steady_k, steady_v, store_k, store_v, value_sum, est_centroids, out, workspace))
+    return RI_ERR_ARG;
   if (!row_src && (!ret_tok_off || !ret_start || np <= 0 || np > 1023)) return RI_ERR_ARG;
   if (BG <= 0 || BG > RI_MAX_GROUPS || gs <= 0 || gs > 16 || static_len < 0 || static_len > steady_stride ||
       es < 0 || nc <= 0)
     return RI_ERR_ARG;
-  if (es > 0 && (!est_ids || !logits || !value_sum || !cluster_size_bf16)) return RI_ERR_ARG;
+  if (es > 0 && (!est_ids || (!logits == !est_centroids) || !value_sum || !cluster_size_bf16)) return RI_ERR_ARG;
   if (workspace_bytes < attn_workspace_bytes(BG, gs)) return RI_ERR_WORKSPACE;
   const int gp = gs_pad_of(gs);
   AttendParams P = {};
@@ -679,6 +692,7 @@ extern "C" int ri_wave_attention(const void* q, const void* steady_k, const void
   P.lenB_ptr_stride = 4;
   P.est_ids = est_ids;
   P.logits = logits;
+  P.est_cent = (const uint16_t*)est_centroids;
   P.value_sum = (const uint16_t*)value_sum;
   P.csize = (const uint16_t*)cluster_size_bf16;
   P.nc = nc;
@@ -690,7 +704,9 @@ extern "C" int ri_wave_attention(const void* q, const void* steady_k, const void
   // the retrieved-token count is only known on the device: size the split for the row table
   // capacity scaled by the usual fill (a quarter) or for 16 tokens per rank, the estimation zone by
   // its exact size
-  plan_splits(static_len + (row_src ? row_src_stride / 4 : np * 16), es, BG, &P.S_kv, &P.S_es);
+  // (estimation rows scored here read a centroid row and a value-sum row: they weigh like key/value rows)
+  plan_splits(static_len + (row_src ? row_src_stride / 4 : np * 16), est_centroids ? 2 * es : es, BG, &P.S_kv,
+              &P.S_es);
   carve_workspace(P, workspace, BG, gp);
   return launch_attend(P, BG, gs, (hipStream_t)stream);
 }

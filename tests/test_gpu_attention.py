@@ -159,8 +159,17 @@ def test_wave_attention(dev, BG, gs, nc, nprobe, es, static_len, seed):
     kernels.wave_attention(qd, steady_k.to(dev), steady_v.to(dev), static_len, store_k.to(dev), store_v.to(dev),
                            None, meta, est if es else None, logits if es else None, vsum.to(dev),
                            size_bf.to(dev), out_t, vl, es, scale, ret_tok_off=off, ret_start=rst)
+    # and with the estimation zone scored inside the launch from the centroid rows (no logits handed in)
+    out_c = torch.empty_like(out)
+    if es:
+        kernels.wave_attention(qd, steady_k.to(dev), steady_v.to(dev), static_len, store_k.to(dev), store_v.to(dev),
+                               None, meta, est, None, vsum.to(dev), size_bf.to(dev), out_c, vl, es, scale,
+                               ret_tok_off=off, ret_start=rst, est_centroids=cent.to(dev))
+    else:
+        out_c.copy_(out_t)
     torch.cuda.synchronize()
-    # (the two modes may split the rows differently: equal up to rounding, both checked against the oracle)
+    # (the modes may split the rows differently: equal up to rounding, all checked against the oracle)
+    assert float((out_c.float() - out.float()).abs().max()) <= 4e-3
     assert float((out_t.float() - out.float()).abs().max()) <= 2e-3
     assert torch.equal(rst.cpu().long(), torch.gather(start.long(), 1, ret.cpu().long()))
     ret_c, est_c, lg = ret.cpu().long(), est.cpu()[:, :es].long(), logits.cpu()
@@ -181,3 +190,4 @@ def test_wave_attention(dev, BG, gs, nc, nprobe, es, static_len, seed):
         ref[b] = attention.weighted_flash_decoding(q[b:b + 1], kk, vv, None, po, pl)[0][0]
     _close(out.cpu(), ref)
     _close(out_t.cpu(), ref)
+    _close(out_c.cpu(), ref)
