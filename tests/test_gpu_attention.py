@@ -116,6 +116,10 @@ def test_closed_form_estimation_exact_for_singletons_and_identical_keys(dev):
     (2, 4, 8192, 147, 1900, 69, 1),
     (3, 7, 3840, 69, 890, 200, 2),
     (2, 8, 2048, 36, 0, 68, 3),      # no estimation zone
+    (2, 16, 1024, 20, 100, 69, 4),   # 16 query heads per group
+    (1, 1, 2048, 1000, 500, 10, 5),  # one head, close to the largest probe list (1023)
+    (2, 5, 512, 33, 77, 1, 6),       # odd group size, one steady token
+    (1, 3, 256, 1, 255, 0, 7),       # one probe, no steady zone, zones cover every cluster
 ])
 def test_wave_attention(dev, BG, gs, nc, nprobe, es, static_len, seed):
     """score_select + wave_attention against the oracle's composition of steps 4-8 of
