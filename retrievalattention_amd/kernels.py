@@ -330,21 +330,22 @@ def kmeans_assign(data, centroids, assign, P, N, nc, seg, head_rows):
           "kmeans_assign")
 
 
-def kmeans_build_lists(assign, counts, offsets, members, P, N, nc):
+def kmeans_build_lists(assign, counts, offsets, members, P, N, nc, slot=0):
+    """`slot` names the scratch area: calls that may run concurrently (different streams) use different slots."""
     nb = lib().ri_kmeans_workspace_bytes(P, N, nc)
-    ws = _workspace(nb, assign.device, "kmeans")
+    ws = _workspace(nb, assign.device, f"kmeans{slot}")
     check(lib().ri_kmeans_build_lists(_p(assign), _p(counts), _p(offsets), _p(members), P, N, nc, _p(ws),
                                       ws.numel(), _stream()), "kmeans_build_lists")
 
 
-def kmeans_update(data, counts, offsets, members, centroids, P, N, nc, seg, head_rows, normalize):
-    ws = _workspace(lib().ri_kmeans_reduce_workspace_bytes(P, N, nc), data.device, "kmeans_reduce")
+def kmeans_update(data, counts, offsets, members, centroids, P, N, nc, seg, head_rows, normalize, slot=0):
+    ws = _workspace(lib().ri_kmeans_reduce_workspace_bytes(P, N, nc), data.device, f"kmeans_reduce{slot}")
     check(lib().ri_kmeans_update(_p(data), _p(counts), _p(offsets), _p(members), _p(centroids), P, N, nc, seg,
                                  head_rows, int(bool(normalize)), _p(ws), ws.numel(), _stream()), "kmeans_update")
 
 
-def kmeans_value_sum(values, counts, offsets, members, value_sum, P, N, nc):
-    ws = _workspace(lib().ri_kmeans_reduce_workspace_bytes(P, N, nc), values.device, "kmeans_reduce")
+def kmeans_value_sum(values, counts, offsets, members, value_sum, P, N, nc, slot=0):
+    ws = _workspace(lib().ri_kmeans_reduce_workspace_bytes(P, N, nc), values.device, f"kmeans_reduce{slot}")
     check(lib().ri_kmeans_value_sum(_p(values), _p(counts), _p(offsets), _p(members), _p(value_sum), P, N, nc,
                                     _p(ws), ws.numel(), _stream()), "kmeans_value_sum")
 
