@@ -16,7 +16,10 @@ tests/golden/make_known_answers.py without this package.  How each function is p
                                   against torch.topk value-for-value and against brute force
   copies.*                        the loop oracles of library/retroinfer/test/test_gather_copy.py
                                   (:110-127, :190-194, :233-237), bit-exact
-  wavebuf.LruModel                brute-force list model + invariants (hit <=> resident, capacity,
+  wavebuf.LruModel                the reference's own BufferManager, compiled from its source by
+                                  oracle/build_ref.py into oracle/_ref/ (tests/test_wavebuf_ref.py:
+                                  same hit/miss/update lists step by step, block id values aside);
+                                  a hand-followed trace; invariants (hit <=> resident, capacity,
                                   unique block ids, least-recently-touched eviction)
   wavebuf.DeviceLruModel          the policy of the device-side block cache manager, which is this
                                   build's own (the reference manages the cache on CPU threads):

@@ -8,10 +8,13 @@ import torch
 from oracle.wavebuf import LruModel
 
 
-def _wb(B, H, nprobe, nc, final_nc, buffer_size, capacity, threads=3, list_len=4096, in_len=4096):
-    from retrievalattention_amd import kernels
-    pool = kernels.ThreadPool(threads)
-    wb = kernels.WaveBufferCPU(B, H, 128, nprobe, 8, nc, final_nc, buffer_size, capacity, threads, pool.get())
+def _wb(B, H, nprobe, nc, final_nc, buffer_size, capacity, threads=3, list_len=4096, in_len=4096, mod=None):
+    """A wave buffer with its index and K/V tensors; `mod` = module providing ThreadPool and WaveBufferCPU
+    (the library's by default)."""
+    if mod is None:
+        from retrievalattention_amd import kernels as mod
+    pool = mod.ThreadPool(threads)
+    wb = mod.WaveBufferCPU(B, H, 128, nprobe, 8, nc, final_nc, buffer_size, capacity, threads, pool.get())
     BG = B * H
     z = lambda *s: torch.zeros(s, dtype=torch.int32)
     idx = dict(hit_ids=z(BG, buffer_size), hit_sizes=z(BG, buffer_size), hit_cum=z(BG, buffer_size), hit_n=z(BG),
