@@ -207,8 +207,13 @@ __global__ __launch_bounds__(256) void km_sort_hist_kernel(const int32_t* __rest
   for (int b = lane; b < bins; b += 64) chunk_hist[((size_t)p * bins + b) * nchunks + chunk] = h[b];
 }
 
-// in-place exclusive prefix sum over the n = bins * nchunks entries of each problem
-__global__ __launch_bounds__(1024) void km_sort_scan_kernel(int32_t* __restrict__ chunk_hist, int n) {
+// in-place exclusive prefix sum over the n = bins * nchunks entries of each problem.
+// When the digit of this pass is the whole cluster id (offsets != nullptr), the scanned entry of
+// (digit c, chunk 0) is where list c starts: the CSR offsets and the counts are written here.
+__global__ __launch_bounds__(1024) void km_sort_scan_kernel(int32_t* __restrict__ chunk_hist, int n,
+                                                            int32_t* __restrict__ offsets,
+                                                            int32_t* __restrict__ counts, int nchunks, int nc,
+                                                            int N) {
   __shared__ int32_t sh_w[16];
   __shared__ int32_t sh_carry;
   int32_t* a = chunk_hist + (size_t)blockIdx.x * n;
@@ -247,6 +252,17 @@ __global__ __launch_bounds__(1024) void km_sort_scan_kernel(int32_t* __restrict_
     __syncthreads();
     if (threadIdx.x == 0) sh_carry += tot;
     __syncthreads();
+  }
+  if (!offsets) return;
+  // (the barrier above made the scanned table visible to the whole workgroup)
+  int32_t* off = offsets + (size_t)blockIdx.x * (nc + 1);
+  for (int c = threadIdx.x; c <= nc; c += 1024) {
+    const int32_t lo = (c < nc) ? a[(size_t)c * nchunks] : N;
+    off[c] = lo;
+    if (c < nc) {
+      const int32_t hi = (c + 1 < nc) ? a[(size_t)(c + 1) * nchunks] : N;
+      counts[(size_t)blockIdx.x * nc + c] = hi - lo;
+    }
   }
 }
 
@@ -538,7 +554,10 @@ extern "C" int ri_kmeans_build_lists(const int32_t* assign, int32_t* counts, int
   // pass over the low digit (the only one when the ids fit 9 bits)
   km_sort_hist_kernel<<<cgrid, 256, 0, s>>>(assign, chunk_hist, N, nchunks, 0, lo_bits);
   RI_HIP_CHECK_LAUNCH();
-  km_sort_scan_kernel<<<P, 1024, 0, s>>>(chunk_hist, (1 << lo_bits) * nchunks);
+  // one pass and no cluster id beyond nc: the scan itself yields offsets and counts
+  const bool direct = hi_bits == 0;
+  km_sort_scan_kernel<<<P, 1024, 0, s>>>(chunk_hist, (1 << lo_bits) * nchunks, direct ? offsets : nullptr,
+                                         direct ? counts : nullptr, nchunks, nc, N);
   RI_HIP_CHECK_LAUNCH();
   km_sort_scatter_kernel<<<cgrid, 256, 0, s>>>(assign, nullptr, chunk_hist, hi_bits ? tmp_key : nullptr,
                                                hi_bits ? tmp_tok : members, N, nchunks, 0, lo_bits);
@@ -546,16 +565,18 @@ extern "C" int ri_kmeans_build_lists(const int32_t* assign, int32_t* counts, int
   if (hi_bits) {
     km_sort_hist_kernel<<<cgrid, 256, 0, s>>>(tmp_key, chunk_hist, N, nchunks, lo_bits, hi_bits);
     RI_HIP_CHECK_LAUNCH();
-    km_sort_scan_kernel<<<P, 1024, 0, s>>>(chunk_hist, (1 << hi_bits) * nchunks);
+    km_sort_scan_kernel<<<P, 1024, 0, s>>>(chunk_hist, (1 << hi_bits) * nchunks, nullptr, nullptr, nchunks, nc, N);
     RI_HIP_CHECK_LAUNCH();
     km_sort_scatter_kernel<<<cgrid, 256, 0, s>>>(tmp_key, tmp_tok, chunk_hist, nullptr, members, N, nchunks,
                                                  lo_bits, hi_bits);
     RI_HIP_CHECK_LAUNCH();
   }
-  km_bounds_kernel<<<dim3((N + 255) / 256, P), 256, 0, s>>>(assign, members, offsets, N, nc);
-  RI_HIP_CHECK_LAUNCH();
-  km_counts_kernel<<<dim3((nc + 255) / 256, P), 256, 0, s>>>(offsets, counts, nc);
-  RI_HIP_CHECK_LAUNCH();
+  if (!direct) {
+    km_bounds_kernel<<<dim3((N + 255) / 256, P), 256, 0, s>>>(assign, members, offsets, N, nc);
+    RI_HIP_CHECK_LAUNCH();
+    km_counts_kernel<<<dim3((nc + 255) / 256, P), 256, 0, s>>>(offsets, counts, nc);
+    RI_HIP_CHECK_LAUNCH();
+  }
   return RI_OK;
 }
 
