@@ -43,7 +43,7 @@ enum {
 const char* ri_status_string(int status);
 int ri_last_hip_error(void);
 /* ABI version: bumped when a signature changes. */
-int ri_abi_version(void);   /* 3 */
+int ri_abi_version(void);   /* 4 */
 /* Launches an empty kernel on `stream`: lets a caller measure the per-dispatch overhead that
  * event timings of back-to-back launches include.  No counterpart in the reference. */
 int ri_null_launch(ri_stream_t stream);
@@ -135,7 +135,10 @@ int ri_weighted_flash_decoding(const void* q, const void* k, const void* v, cons
  * gather_copy_and_concat → weighted_flash_decoding, cache_hub/retroinfer_cache.py:598-674)
  * when every cluster's K/V already sits in device memory, reading K/V in place through
  * the row table instead of staging them in an execution buffer.
- *   steady_k/v [BG, steady_stride, 128]: first static_len rows attended
+ *   steady_k/v [BG, steady_stride, 128]: first static_len rows attended; with static_len_dev (one
+ *   int32 in device memory, or NULL) the count is read there when the kernel runs (clamped to
+ *   [0, steady_stride]) and static_len only sizes the split: a captured launch then stays valid while
+ *   the steady zone grows token by token
  *   store_k/v  [BG, store_stride, 128]: cluster-contiguous K/V
  *   row_src [BG, row_src_stride]: store row of every retrieved token; or NULL with ret_tok_off
  *   [BG, np+1] and ret_start [BG, np]: rank r's tokens are the store rows ret_start[r] + i
@@ -150,7 +153,8 @@ int ri_weighted_flash_decoding(const void* q, const void* k, const void* v, cons
  *   workspace: same rules as ri_weighted_flash_decoding (zeroed once by the caller). */
 size_t ri_wave_attention_workspace_bytes(int BG, int gs);
 int ri_wave_attention(const void* q, const void* steady_k, const void* steady_v,
-                      int64_t steady_stride, int static_len, const void* store_k,
+                      int64_t steady_stride, int static_len, const int32_t* static_len_dev,
+                      const void* store_k,
                       const void* store_v, int64_t store_stride, const int32_t* row_src,
                       int row_src_stride, const int32_t* ret_tok_off, const int32_t* ret_start, int np,
                       const int32_t* meta, const int32_t* est_ids,

@@ -38,7 +38,7 @@ class retroinfer_cache(KV_Cache):
                  head_dim, dtype, layer_mapping, max_new_length, static_pattern_start, static_pattern_end, core,
                  n_centroids, n_segment, nprobe, max_compute_cluster_num, cache_unit_size, cache_cluster_num,
                  num_gpus, model_size, use_cluster_estimation=False, kv_residency="auto",
-                 block_cache="device"):
+                 block_cache="device", device_positions=False):
         super().__init__(layer_num, batch_size, max_length, num_key_value_heads, num_heads, head_dim, dtype,
                          layer_mapping, num_gpus, model_size)
         if head_dim != 128 or dtype != torch.bfloat16:
@@ -115,6 +115,19 @@ class retroinfer_cache(KV_Cache):
         else:
             self._init_wave_buffer()
         self.allocate_computation_buffer()
+
+        # device_positions: the steady zone's length also lives in device memory, the new token's K/V is
+        # written at that position by an indexed copy and the attention reads the length when it runs,
+        # so a captured decode step (decode_update_kv_cache + compute of every layer) can be replayed
+        # token after token; the host counters are then advanced by token_replayed()
+        self.device_positions = bool(device_positions)
+        if self.device_positions:
+            if self.kv_residency != "device" or use_cluster_estimation or len(set(self.layer_mapping.values())) != 1:
+                raise ValueError("device_positions needs a device-resident store on one device, without "
+                                 "next-layer estimation")
+            d0 = self.layer_mapping[str(0)]
+            self.steady_len_dev = torch.tensor([self.static_pattern_total + 1], dtype=torch.int32, device=d0)
+            self.steady_pos_dev = torch.tensor([self.static_pattern_total], dtype=torch.int64, device=d0)
 
         self.copystream = torch.cuda.Stream()
         self.mainevents, self.copyevents = {}, {}
@@ -382,14 +395,43 @@ class retroinfer_cache(KV_Cache):
         self.logits = torch.zeros((BG, self.group_size, self.n_centroids), dtype=torch.float32,
                                   device=self.layer_mapping[str(0)])
         self.static_pattern_total = sps + spe
+        if self.device_positions:
+            self.steady_len_dev.fill_(self.static_pattern_total + 1)
+            self.steady_pos_dev.fill_(self.static_pattern_total)
+
+    def fold_due(self):
+        """True when the next token has to fold the generated tokens into the index first (every
+        THRESHOLD_LENGTH tokens).  A loop that replays captured steps calls prepare_token() then,
+        outside any capture, and captures its steps again: the fold re-allocates the score buffer."""
+        return self.static_pattern_total == self.static_pattern_start + self.static_pattern_end + THRESHOLD_LENGTH
+
+    def prepare_token(self):
+        if self.fold_due():
+            self._update_kv_cache()
+
+    def token_replayed(self):
+        """Host-side bookkeeping for one token decoded by replaying captured steps (device_positions):
+        the replay advanced the device-side position, this advances the host counters."""
+        self.context += 1
+        self.static_pattern_total += 1
 
     def decode_update_kv_cache(self, key_states, value_states, layer_idx):
         """Appends the new token's K/V to the steady zone (reference: retroinfer_cache.py:527-546)."""
-        if self.static_pattern_total == self.static_pattern_start + self.static_pattern_end + THRESHOLD_LENGTH:
-            self._update_kv_cache()
+        last = layer_idx == self.layer_num - 1
+        if self.device_positions:
+            capturing = torch.cuda.is_current_stream_capturing()
+            if not capturing:
+                self.prepare_token()
+            self.steady_zone_keys[layer_idx].index_copy_(2, self.steady_pos_dev, key_states.transpose(1, 2))
+            self.steady_zone_values[layer_idx].index_copy_(2, self.steady_pos_dev, value_states.transpose(1, 2))
+            # (the device-side position moves on after the last layer's attention, in compute())
+            if last and not capturing:
+                self.token_replayed()
+            return None, None
+        self.prepare_token()
         self.steady_zone_keys[layer_idx][:, :, self.static_pattern_total] = key_states[:, 0]
         self.steady_zone_values[layer_idx][:, :, self.static_pattern_total] = value_states[:, 0]
-        if layer_idx == self.layer_num - 1:
+        if last:
             self.context += 1
             self.static_pattern_total += 1
         return None, None
@@ -425,7 +467,11 @@ class retroinfer_cache(KV_Cache):
         queries [batch, 1, heads, dim] on the device; returns the same shape."""
         last = layer_idx == self.layer_num - 1
         static_len = self.static_pattern_total if last else self.static_pattern_total + 1
-        return self._compute(queries, layer_idx, queries_next, static_len)
+        out = self._compute(queries, layer_idx, queries_next, static_len)
+        if last and self.device_positions:   # the token is done: its row now belongs to the steady zone
+            self.steady_len_dev.add_(1)
+            self.steady_pos_dev.add_(1)
+        return out
 
     def _compute(self, queries, layer_idx, queries_next, static_len):
         """compute() for a given number of steady-zone tokens."""
@@ -451,7 +497,8 @@ class retroinfer_cache(KV_Cache):
             static_len, self.list_keys[layer_idx], self.list_values[layer_idx], None, self.meta,
             self.est_ids[buf] if es > 0 else None, self.logits if es > 0 else None, self.value_sum[layer_idx],
             self.cluster_size[layer_idx], out, self.valid_lengths[buf], es, self.RSQRT_DIM,
-            ret_tok_off=self.ret_tok_off, ret_start=self.ret_start)
+            ret_tok_off=self.ret_tok_off, ret_start=self.ret_start,
+            static_len_dev=self.steady_len_dev if self.device_positions else None)
         return out.view(self.batch_size, 1, self.num_heads, D)
 
     def block_cache_stats(self, layer_idx):

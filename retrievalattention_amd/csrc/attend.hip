@@ -32,6 +32,7 @@ struct AttendParams {
   const uint16_t* vA;
   int64_t strideA;
   int lenA;
+  const int32_t* lenA_ptr;  // when given: lenA is read here at launch time (clamped to [0, strideA])
   // region B: rows [0, lenB(g)) at kB/vB + (g*strideB + src(row))*128,
   // src(row) = row_src ? row_src[g*rs_stride + row] : row
   const uint16_t* kB;
@@ -193,7 +194,7 @@ __device__ __forceinline__ float2 ri_ld_partial(const float* p) {
 }
 
 template <int GS_PAD>
-__device__ __forceinline__ void combine_group(const AttendParams& P, int g, int S, int lenB) {
+__device__ __forceinline__ void combine_group(const AttendParams& P, int g, int S, int lenA, int lenB) {
   const int gs = P.gs;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   for (int j = wave; j < gs; j += 4) {
@@ -248,7 +249,7 @@ __device__ __forceinline__ void combine_group(const AttendParams& P, int g, int 
     *reinterpret_cast<uint32_t*>(P.out + ((size_t)g * gs + j) * RI_DIM + 2 * lane) = o;
     if (lane == 0 && P.lse_out) P.lse_out[(size_t)g * gs + j] = M + __logf(L);
   }
-  if (threadIdx.x == 0 && P.valid_lengths) P.valid_lengths[g] = P.lenA + lenB;
+  if (threadIdx.x == 0 && P.valid_lengths) P.valid_lengths[g] = lenA + lenB;
 }
 
 #define ATT_DESC_MAX 128  // rows of one wave whose descriptors are staged in LDS at a time
@@ -292,6 +293,7 @@ __global__ __launch_bounds__(256, GS_PAD == 16 ? 1 : 3) void attend_kernel(Atten
   int* dsc = sh_desc[wave];
   float* wsh = sh_w[wave];
   const int lenB = P.lenB_ptr ? P.lenB_ptr[(size_t)g * P.lenB_ptr_stride] : P.lenB_const;
+  const int lenA_all = P.lenA_ptr ? min(max(P.lenA_ptr[0], 0), (int)P.strideA) : P.lenA;
 
   // Estimation rows whose scores are not handed in are key/value rows of their own: key = centroid,
   // value = value sum, weight = cluster size, located through the id list.
@@ -328,8 +330,8 @@ __global__ __launch_bounds__(256, GS_PAD == 16 ? 1 : 3) void attend_kernel(Atten
       }
     }
     // (the row count is consumed only now: the loads above went out together with its load)
-    const int lenA = est_split ? 0 : P.lenA;
-    const int total = est_split ? P.es : P.lenA + lenB;
+    const int lenA = est_split ? 0 : lenA_all;
+    const int total = est_split ? P.es : lenA_all + lenB;
     int r0, r1;
     if (est_split)
       wave_rows(total, P.S_es * 4, (split - P.S_kv) * 4 + wave, &r0, &r1);
@@ -552,7 +554,7 @@ __global__ __launch_bounds__(256, GS_PAD == 16 ? 1 : 3) void attend_kernel(Atten
     sh_last = (__hip_atomic_fetch_add(&P.counters[g], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == S - 1);
   __syncthreads();
   if (!sh_last) return;
-  combine_group<GS_PAD>(P, g, S, lenB);
+  combine_group<GS_PAD>(P, g, S, lenA_all, lenB);
   if (threadIdx.x == 0) P.counters[g] = 0;  // ready for the next launch
 }
 
@@ -654,7 +656,8 @@ extern "C" int ri_weighted_flash_decoding(const void* q, const void* k, const vo
 }
 
 extern "C" int ri_wave_attention(const void* q, const void* steady_k, const void* steady_v,
-                                 int64_t steady_stride, int static_len, const void* store_k,
+                                 int64_t steady_stride, int static_len, const int32_t* static_len_dev,
+                                 const void* store_k,
                                  const void* store_v, int64_t store_stride, const int32_t* row_src,
                                  int row_src_stride, const int32_t* ret_tok_off, const int32_t* ret_start, int np,
                                  const int32_t* meta, const int32_t* est_ids,
@@ -678,6 +681,7 @@ extern "C" int ri_wave_attention(const void* q, const void* steady_k, const void
   P.vA = (const uint16_t*)steady_v;
   P.strideA = steady_stride;
   P.lenA = static_len;
+  P.lenA_ptr = static_len_dev;
   P.kB = (const uint16_t*)store_k;
   P.vB = (const uint16_t*)store_v;
   P.strideB = store_stride;

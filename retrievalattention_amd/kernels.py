@@ -259,17 +259,20 @@ def score_logits(q, centroids, logits, scale, slot=0):
 
 def wave_attention(q, steady_k, steady_v, static_len, store_k, store_v, row_src, meta, est_ids, logits,
                    value_sum, cluster_size_bf16, out, valid_lengths, es, scale, slot=0, ret_tok_off=None,
-                   ret_start=None, est_centroids=None):
+                   ret_start=None, est_centroids=None, static_len_dev=None):
     """Attention over steady zone + retrieved clusters (read in place) + estimation zone.
     The retrieved rows come from a row table (row_src) or, with row_src None, from the rank tables
     ret_tok_off [BG, np+1] and ret_start [BG, np].  The estimation zone's scores are read from `logits`
     or, with logits None, computed in the launch from the rows of `est_centroids` [BG, nc, 128].
+    With static_len_dev (int32 tensor of one element on the device) the number of steady rows is read
+    from it when the kernel runs; static_len then only sizes the split.
     `slot`: scratch area, one per concurrent call."""
     BG, gs, D = q.shape
     nc = value_sum.shape[1]
     nb = lib().ri_wave_attention_workspace_bytes(BG, gs)
     ws = _workspace(nb, q.device, f"attn{slot}")
-    check(lib().ri_wave_attention(_p(q), _p(steady_k), _p(steady_v), steady_k.shape[-2], static_len, _p(store_k),
+    check(lib().ri_wave_attention(_p(q), _p(steady_k), _p(steady_v), steady_k.shape[-2], static_len,
+                                  _p(static_len_dev), _p(store_k),
                                   _p(store_v), store_k.shape[-2], _p(row_src),
                                   0 if row_src is None else row_src.shape[1], _p(ret_tok_off), _p(ret_start),
                                   0 if ret_start is None else ret_start.shape[1], _p(meta), _p(est_ids), _p(logits),

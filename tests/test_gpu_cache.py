@@ -19,7 +19,7 @@ def _close(got, ref):
 
 
 def _make_cache(dev, residency, layers, B, Hkv, gs, ctx, n_centroids, n_segment, nprobe, es, new=8,
-                cache_cluster_num=None, use_cluster_estimation=False):
+                cache_cluster_num=None, use_cluster_estimation=False, device_positions=False):
     from retrievalattention_amd.cache_hub import retroinfer_cache
     # "host-cpu": host-resident store with the reference's worker-thread block cache manager;
     # "host": the same store with the device-side manager
@@ -32,7 +32,7 @@ def _make_cache(dev, residency, layers, B, Hkv, gs, ctx, n_centroids, n_segment,
         n_segment=n_segment, nprobe=nprobe, max_compute_cluster_num=nprobe + es, cache_unit_size=8,
         cache_cluster_num=cache_cluster_num if cache_cluster_num is not None else 3 * nprobe, num_gpus=1,
         model_size=8, use_cluster_estimation=use_cluster_estimation, kv_residency=residency,
-        block_cache=block_cache)
+        block_cache=block_cache, device_positions=device_positions)
 
 
 def _prefill(cache, K, V, layers, B):
@@ -300,3 +300,71 @@ def test_index_growth_after_1024_generated_tokens(dev, residency):
     _close(out.cpu().view(BG, gs, 128), ref)
     cI = cache.cI[0].cpu()
     check_zone_sets(aux["dist"], cI[:, :nprobe], cI[:, nprobe:], aux["ret"], aux["est"], nprobe, es, band=2.0)
+
+
+def test_captured_steps_replay_token_after_token(dev):
+    """device_positions: the steady zone's length lives on the device, so one captured decode step per
+    layer (append the token's K/V, attend) is replayed for token after token while the zone grows.
+    Every replayed token must match a twin cache that is stepped eagerly with the reference's calls."""
+    layers, B, Hkv, gs, ctx = 2, 2, 2, 4, 2048 + 68
+    nc, nprobe, es, tokens = 128, 8, 40, 6
+    K, V = _gen(layers, B, Hkv, gs, ctx, 128, dev, 31)
+    eager = _make_cache(dev, "device", layers, B, Hkv, gs, ctx, nc, 1, nprobe, es, new=64)
+    replay = _make_cache(dev, "device", layers, B, Hkv, gs, ctx, nc, 1, nprobe, es, new=64, device_positions=True)
+    _prefill(eager, K, V, layers, B)
+    _prefill(replay, K, V, layers, B)
+    g = torch.Generator().manual_seed(32)
+    draw = lambda: ([torch.randn(B, 1, Hkv * gs, 128, generator=g).to(torch.bfloat16).to(dev) for _ in range(layers)],
+                    [torch.randn(B, 1, Hkv, 128, generator=g).to(torch.bfloat16).to(dev) for _ in range(layers)],
+                    [torch.randn(B, 1, Hkv, 128, generator=g).to(torch.bfloat16).to(dev) for _ in range(layers)])
+    q_in = [torch.empty(B, 1, Hkv * gs, 128, dtype=torch.bfloat16, device=dev) for _ in range(layers)]
+    k_in = [torch.empty(B, 1, Hkv, 128, dtype=torch.bfloat16, device=dev) for _ in range(layers)]
+    v_in = [torch.empty(B, 1, Hkv, 128, dtype=torch.bfloat16, device=dev) for _ in range(layers)]
+
+    def step(cache, l, q, k, v):
+        cache.decode_update_kv_cache(k, v, l)
+        return cache.compute(q, l)
+
+    def load(qs, ks, vs):
+        for l in range(layers):
+            q_in[l].copy_(qs[l]); k_in[l].copy_(ks[l]); v_in[l].copy_(vs[l])
+
+    # first token eagerly on both (also the warm-up that capture needs), on a side stream
+    qs, ks, vs = draw()
+    load(qs, ks, vs)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        first = [step(replay, l, q_in[l], k_in[l], v_in[l]) for l in range(layers)]
+    torch.cuda.current_stream().wait_stream(side)
+    ref = [step(eager, l, qs[l], ks[l], vs[l]) for l in range(layers)]
+    torch.cuda.synchronize()
+    for l in range(layers):
+        assert torch.equal(first[l], ref[l])
+    assert replay.static_pattern_total == eager.static_pattern_total == 69
+    # capture one step per layer
+    graphs = []
+    for l in range(layers):
+        gr = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(gr):
+            o = step(replay, l, q_in[l], k_in[l], v_in[l])
+        graphs.append((gr, o))
+    assert replay.static_pattern_total == 69          # capturing moved nothing on the host
+    for t in range(tokens):
+        qs, ks, vs = draw()
+        load(qs, ks, vs)
+        assert not replay.fold_due()
+        for l in range(layers):
+            graphs[l][0].replay()
+        replay.token_replayed()
+        ref = [step(eager, l, qs[l], ks[l], vs[l]) for l in range(layers)]
+        torch.cuda.synchronize()
+        for l in range(layers):
+            d = (graphs[l][1].float() - ref[l].float()).abs()
+            assert float(d.max()) <= 2e-3, (t, l, float(d.max()))
+        assert replay.static_pattern_total == eager.static_pattern_total == 70 + t
+        assert int(replay.steady_len_dev) == replay.static_pattern_total + 1
+        for l in range(layers):   # the replays appended the same rows as the eager calls
+            n = eager.static_pattern_total
+            assert torch.equal(replay.steady_zone_keys[l][:, :, :n], eager.steady_zone_keys[l][:, :, :n])
+    assert int(replay.valid_lengths[(layers - 1) % 2].min()) > 69 + tokens - 1   # the grown zone was attended
