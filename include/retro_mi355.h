@@ -69,7 +69,7 @@ int ri_batch_gemm_softmax(const void* A, const void* B, void* D, float* Norm, fl
  *   q          [BG, gs, 128] bf16
  *   centroids  [BG, nc, 128] bf16
  *   mask       [BG, nc] uint8 (1 = empty cluster, scored as finfo(bf16).min) or NULL
- *   cluster_size_i32 [BG, nc] int32 token count per cluster, or NULL (then no row table)
+ *   cluster_size_i32 [BG, nc] int32 token count per cluster, or NULL (then no token layout)
  *   cluster_start    [BG, nc] int32 first row of the cluster in the cluster-contiguous
  *                    K/V store, or NULL
  * Outputs
@@ -133,8 +133,8 @@ int ri_weighted_flash_decoding(const void* q, const void* k, const void* v, cons
 /* Fused wave-index attention over a device-resident cluster store: replaces steps 4-8 of
  * retroinfer_cache.compute (gather_copy_vectors → weighted_flash_decoding →
  * gather_copy_and_concat → weighted_flash_decoding, cache_hub/retroinfer_cache.py:598-674)
- * when every cluster's K/V already sits in device memory, reading K/V in place through
- * the row table instead of staging them in an execution buffer.
+ * when every cluster's K/V already sits in device memory, reading K/V in place (located through
+ * the rank tables or a row table) instead of staging them in an execution buffer.
  *   steady_k/v [BG, steady_stride, 128]: first static_len rows attended; with static_len_dev (one
  *   int32 in device memory, or NULL) the count is read there when the kernel runs (clamped to
  *   [0, steady_stride]) and static_len only sizes the split: a captured launch then stays valid while

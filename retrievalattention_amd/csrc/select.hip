@@ -1,6 +1,6 @@
 // Cluster selection for the decode step (gfx950): from the fp32 logits of the scoring pass to
 // the retrieval zone (top nprobe clusters in rank order), the estimation zone (next es) and
-// the row table of the retrieved tokens.  Follows cache_hub/retroinfer_cache.py:572-575
+// the layout of the retrieved tokens (rank tables, optionally a row table).  Follows cache_hub/retroinfer_cache.py:572-575
 // (sum over the query group of the bf16 softmax, empty-cluster mask, top-k) and the buffer
 // cut-off of library/retroinfer/retroinfer_kernels/src/wave_buffer_cpu.cpp:207-216.
 //
@@ -11,7 +11,7 @@
 //                  per distinct key (scores lie in [0, 16], so ~16.8k bins cover every key), zone
 //                  membership with ties resolved by ascending id, rank order of the retrieval
 //                  zone straight from the histogram prefix, and the token layout (page
-//                  cut-off, row table).
+//                  cut-off; token prefix and first store row per rank, a row per token on request).
 #include "ri_common.h"
 
 #define SEL_THREADS 1024
