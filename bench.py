@@ -25,7 +25,7 @@ HBM_PEAK = 8.0e12  # bytes/s, MI355X
 # HBM bytes per attend_kernel launch from rocprofv3 counter runs of this script (FETCH_SIZE and
 # WRITE_SIZE, each scaled by what the counter reads for the known-size copy of --copy-probe);
 # the summaries are kept under profiles/.
-MEASURED_TRAFFIC = {"c2": int((31708.9 * 2.000 + 1201.1 * 1.000) * 1024)}
+MEASURED_TRAFFIC = {"c2": int((31708.0 * 2.000 + 1201.0 * 1.000) * 1024)}
 
 CONFIGS = {
     # name: batch, kv heads, group size, clustered tokens, mixture centres, centroids, segments, outliers, layers
