@@ -140,7 +140,16 @@ def bench_kmeans(cfg, dev, iters=10, reps=3):
     t_as = time_region(lambda: kernels.kmeans_assign(K, r.centroids, assign, Hkv, N, nc, 1, N), reps)
     flops = 2.0 * 128 * Hkv * N * ((iters - 1) * nc / S + nc)
     flops_as = 2.0 * 128 * Hkv * N * nc
-    return {"ms_per_sequence": t * 1e3, "tokens": N, "kv_heads": Hkv, "centroids": nc, "segments": S,
+    # the same clustering without segments (every iteration scores all centroids), from a seeded
+    # random choice of initial tokens
+    g = torch.Generator(device=dev).manual_seed(0)
+    init = torch.sort(torch.randperm(N, generator=g, device=dev)[:nc]).values
+    segment_k_means_csr(K, V, nc, iters, 1, init_indices=init)
+    t_un = time_region(lambda: segment_k_means_csr(K, V, nc, iters, 1, init_indices=init), reps)
+    flops_un = 2.0 * 128 * Hkv * N * iters * nc
+    unseg = {"ms_per_sequence": t_un * 1e3, "algorithmic_flops": flops_un, "achieved": flops_un / t_un / 1e12,
+             "frac": flops_un / t_un / MFMA_BF16_PEAK, "init": "seeded random tokens"}
+    return {"unsegmented": unseg, "ms_per_sequence": t * 1e3, "tokens": N, "kv_heads": Hkv, "centroids": nc, "segments": S,
             "iterations": iters, "algorithmic_flops": flops, "bound": "mfma", "achieved": flops / t / 1e12,
             "peak": MFMA_BF16_PEAK / 1e12, "unit": "TFLOP/s", "frac": flops / t / MFMA_BF16_PEAK,
             "global_assign": {"us": t_as * 1e6, "achieved": flops_as / t_as / 1e12,
