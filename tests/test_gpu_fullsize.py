@@ -18,6 +18,7 @@ MAX_ABS, MEAN_ABS = 2e-2, 2e-3
 
 SHAPES = {
     # batch, kv heads, group size, clustered tokens, centroids, segments, outlier channels, seed, residency
+    "c1": dict(B=1, Hkv=8, gs=4, N=8192, nc=512, S=1, outliers=False, seed=0, residency="device"),
     "c2": dict(B=4, Hkv=8, gs=4, N=131072, nc=8192, S=16, outliers=True, seed=0, residency="device"),
     "c4": dict(B=16, Hkv=4, gs=7, N=61440, nc=3840, S=8, outliers=False, seed=1, residency="host"),
     "c5": dict(B=8, Hkv=8, gs=8, N=262144, nc=16384, S=32, outliers=True, seed=0, residency="device"),
@@ -83,7 +84,7 @@ def _step(cache, q, dev, seed):
     return out
 
 
-@pytest.mark.parametrize("name", ["c2", "c5", "c4"])
+@pytest.mark.parametrize("name", ["c1", "c2", "c5", "c4"])
 def test_benchmark_shape_decode(dev, name):
     cfg = SHAPES[name]
     cache, q, nprobe, es = _build(dev, cfg)
