@@ -57,7 +57,8 @@ def build_cache(cfg, L, dev, residency="device", block_cache="device", estimate_
         num_heads=Hkv * gs, head_dim=128, dtype=torch.bfloat16, layer_mapping={str(l): "cuda:0" for l in range(L)},
         max_new_length=new, static_pattern_start=synth.STEADY_START, static_pattern_end=synth.STEADY_END, core=8,
         n_centroids=cfg["nc"], n_segment=cfg["S"], nprobe=nprobe, max_compute_cluster_num=nprobe + es,
-        cache_unit_size=8, cache_cluster_num=3 * nprobe, num_gpus=1, model_size=0, kv_residency=residency,
+        cache_unit_size=8, cache_cluster_num=max(int(cfg["nc"] * 0.05), nprobe), num_gpus=1, model_size=0,
+        kv_residency=residency,
         block_cache=block_cache, use_cluster_estimation=estimate_next)
     queries = []
     t0 = time.time()
