@@ -44,14 +44,14 @@ def log(*a):
     print(*a, file=sys.stderr, flush=True)
 
 
-def build_cache(cfg, L, dev, residency="device", block_cache="device", estimate_next=False):
+def build_cache(cfg, L, dev, residency="device", block_cache="device", estimate_next=False, new=2,
+                device_positions=False):
     from retrievalattention_amd import synth
     from retrievalattention_amd.cache_hub import retroinfer_cache
     B, Hkv, gs, N = cfg["B"], cfg["Hkv"], cfg["gs"], cfg["N"]
     nprobe = max(1, int(cfg["nc"] * 0.018))
     es = int(cfg["nc"] * 0.232)
     ctx = N + synth.STEADY_START + synth.STEADY_END
-    new = 2
     cache = retroinfer_cache(
         valid_start=[0] * B, layer_num=L, batch_size=B, max_length=ctx + new, num_key_value_heads=Hkv,
         num_heads=Hkv * gs, head_dim=128, dtype=torch.bfloat16, layer_mapping={str(l): "cuda:0" for l in range(L)},
@@ -59,7 +59,7 @@ def build_cache(cfg, L, dev, residency="device", block_cache="device", estimate_
         n_centroids=cfg["nc"], n_segment=cfg["S"], nprobe=nprobe, max_compute_cluster_num=nprobe + es,
         cache_unit_size=8, cache_cluster_num=max(int(cfg["nc"] * 0.05), nprobe), num_gpus=1, model_size=0,
         kv_residency=residency,
-        block_cache=block_cache, use_cluster_estimation=estimate_next)
+        block_cache=block_cache, use_cluster_estimation=estimate_next, device_positions=device_positions)
     queries = []
     t0 = time.time()
     for l in range(L):
@@ -228,6 +228,56 @@ def bench_estimate_next(args, cache, queries, outs, L, static_len):
                     "predicted query; layers 0 and 1 select for themselves; outputs checked against the plain step"}
 
 
+def bench_end_to_end(args, cfg, dev):
+    """A whole decoded token of a Llama-shaped model (random weights, the config's attention shape)
+    around the wave-index cache built from the synthetic K/V: every layer's norm, QKV projection,
+    rotary embedding, cache append, wave-index attention, output projection and MLP, captured once as
+    one HIP graph and replayed token after token (the steady zone grows by one row per token)."""
+    from retrievalattention_amd.model_hub import LlamaModel, LlamaShape
+    L, B, tokens = cfg["L"], cfg["B"], args.steps
+    heads = cfg["Hkv"] * cfg["gs"]
+    shape = LlamaShape(hidden_size=heads * 128, intermediate_size=cfg.get("ffn", 14336), num_layers=L, num_heads=heads,
+                       num_key_value_heads=cfg["Hkv"], head_dim=128, vocab_size=128256)
+    cache, queries, nprobe, es = build_cache(cfg, L, dev, new=tokens + args.warmup + 8, device_positions=True)
+    del queries
+    ctx = cache.context
+    model = LlamaModel(shape, ctx + tokens + args.warmup + 16, device=dev, seed=0)
+    model.kv_cache, model.attention_type = cache, "RetroInfer"
+    model.position.fill_(ctx)
+    tok = torch.zeros(B, 1, dtype=torch.int64, device=dev)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        logits = model.decode_forward(tok)          # first token eagerly (warm-up for the capture)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        logits = model.decode_forward(tok)
+    def one():
+        graph.replay()
+        cache.token_replayed()
+        tok.copy_(logits.argmax(-1))
+    for _ in range(args.warmup):
+        one()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(tokens):
+        one()
+    torch.cuda.synchronize()
+    t = (time.perf_counter() - t0) / tokens
+    weights = sum(w.numel() * 2 for l in model.layers for w in (l.wqkv, l.wo, l.gate_up_proj, l.down_proj)) + model.lm_head.numel() * 2
+    print(json.dumps({
+        "metric": "decode tokens/s end to end (random-weight model of the config's shape around the wave-index cache)",
+        "value": B / t, "unit": "tokens/s", "n_gpus": 1, "steps": tokens, "warmup": args.warmup, "ms_per_step": t * 1e3,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": f"{args.config}: {cfg['desc']}; {L} layers, hidden {shape.hidden_size}, MLP "
+                               f"{shape.intermediate_size}, vocabulary {shape.vocab_size}; one HIP graph per token",
+                   "batch": B, "context_tokens": ctx, "weight_bytes": weights,
+                   "weights_at_hbm_peak_ms": weights / HBM_PEAK * 1e3},
+        "roofline": None, "cpu_baseline": None}))
+
+
 def bench_host(args, cfg, cache, queries, L, nprobe, es, static_len):
     """Host-resident clustered K/V: the reference's operator sequence (score+select, id copy to the
     host, block-cache look-up on the worker pool, gather of misses over the host link and hits
@@ -335,6 +385,9 @@ def main():
     ap.add_argument("--estimate-next", action="store_true",
                     help="also measure the step with next-layer cluster estimation (zones of layer l+1 chosen "
                          "at the end of layer l from a predicted query)")
+    ap.add_argument("--end-to-end", action="store_true",
+                    help="a whole decoded token of a random-weight model of the config's shape (all layers, one "
+                         "HIP graph per token) instead of the attention-only layer-step")
     ap.add_argument("--copy-probe", action="store_true",
                     help="also run 8 device copies of 256 MiB (a known-size kernel to scale rocprofv3 byte counters by)")
     args = ap.parse_args()
@@ -355,6 +408,8 @@ def main():
             b.copy_(a)
         torch.cuda.synchronize()
         del a, b
+    if args.end_to_end:
+        return bench_end_to_end(args, cfg, dev)
     est_next = args.residency == "device" and args.estimate_next and not args.no_graph and L >= 4
     cache, queries, nprobe, es = build_cache(cfg, L, dev, args.residency, args.block_cache, est_next)
     static_len = cache.static_pattern_total  # 4 + 64 + the token being decoded (already counted)
