@@ -25,7 +25,7 @@ HBM_PEAK = 8.0e12  # bytes/s, MI355X
 # HBM bytes per attend_kernel launch from rocprofv3 counter runs of this script (FETCH_SIZE and
 # WRITE_SIZE, each scaled by what the counter reads for the known-size copy of --copy-probe);
 # the summaries are kept under profiles/.
-MEASURED_TRAFFIC = {"c2": int((31708.0 * 2.000 + 1201.0 * 1.000) * 1024)}
+MEASURED_TRAFFIC = {"c2": int((31709.9 * 2.000 + 1201.1 * 1.000) * 1024)}
 
 CONFIGS = {
     # name: batch, kv heads, group size, clustered tokens, mixture centres, centroids, segments, outliers, layers
@@ -200,29 +200,25 @@ def bench_estimate_next(args, cache, queries, outs, L, static_len):
             step(l)
     torch.cuda.current_stream().wait_stream(side)
     torch.cuda.synchronize()
-    graphs = []
-    for l in range(L):
-        gr = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(gr):
-            o = step(l)
-        graphs.append((gr, o))
-    torch.cuda.synchronize()
-    for l in range(L):
-        graphs[l][0].replay()
+    cycle = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(cycle):
+        cyc_outs = [step(l) for l in range(L)]
+    cycle.replay()
     torch.cuda.synchronize()
     # same zones as the plain step; the estimation zone's scores come from another accumulation order
     for l in range(L):
-        d = (graphs[l][1].float() - outs[l].float()).abs()
+        d = (cyc_outs[l].float() - outs[l].float()).abs()
         if float(d.max()) > 2e-2 or float(d.mean()) > 2e-3:
             sys.exit(f"next-layer estimation: layer {l} differs from the plain step (max-abs {float(d.max())})")
-    for i in range(args.warmup):
-        graphs[i % L][0].replay()
+    n_cyc = max(1, args.steps // L)
+    for _ in range(max(1, args.warmup // L)):
+        cycle.replay()
     torch.cuda.synchronize()
     t0 = time.perf_counter()
-    for i in range(args.steps):
-        graphs[i % L][0].replay()
+    for _ in range(n_cyc):
+        cycle.replay()
     torch.cuda.synchronize()
-    t = (time.perf_counter() - t0) / args.steps
+    t = (time.perf_counter() - t0) / (n_cyc * L)
     return {"us_per_layer_step": t * 1e6, "layers_per_token": L,
             "note": "zones of layer l+1 chosen at the end of layer l from the (here exact) "
                     "predicted query; layers 0 and 1 select for themselves; outputs checked against the plain step"}
@@ -296,24 +292,36 @@ def bench_host(args, cfg, cache, queries, L, nprobe, es, static_len):
     torch.cuda.synchronize()
     t_cold = (time.perf_counter() - t0) / L
     use_graph = cache.block_cache == "device" and not args.no_graph
-    if use_graph:   # the device-side manager has no host round trip: the whole step replays as a HIP graph
-        graphs = []
-        for l in range(L):
-            gr = torch.cuda.CUDAGraph()
-            with torch.cuda.graph(gr):
+    if use_graph:
+        # the device-side manager has no host round trip: the steps replay as HIP graphs.  A graph
+        # launch has a fixed cost of its own, so one graph holds a cycle of the layers, and the warm
+        # measurement (same queries every time) one graph of several cycles
+        cycle = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(cycle):
+            for l in range(L):
                 step(l)
-            graphs.append(gr)
-        run = lambda i: graphs[i % L].replay()
+        reps = max(1, 32 // L)
+        multi = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(multi):
+            for _ in range(reps):
+                for l in range(L):
+                    step(l)
+        run_cycle = cycle.replay
+        run_many, many = multi.replay, reps * L
     else:
-        run = lambda i: step(i % L)
-    for i in range(args.warmup):
-        run(i)
+        def run_cycle():
+            for l in range(L):
+                step(l)
+        run_many, many = run_cycle, L
+    for _ in range(max(1, args.warmup // many)):
+        run_many()
     torch.cuda.synchronize()
+    n_warm = max(1, args.steps // many)
     t0 = time.perf_counter()
-    for i in range(args.steps):
-        run(i)
+    for _ in range(n_warm):
+        run_many()
     torch.cuda.synchronize()
-    t_warm = (time.perf_counter() - t0) / args.steps
+    t_warm = (time.perf_counter() - t0) / (n_warm * many)
     stats = [cache.block_cache_stats(l) for l in range(L)]
     hit, miss = sum(s_[0] for s_ in stats), sum(s_[1] for s_ in stats)
     # drifting queries: each step's query is the layer's query plus noise drawn from a small pool, so
@@ -325,27 +333,29 @@ def bench_host(args, cfg, cache, queries, L, nprobe, es, static_len):
         pool = [[(b.float() + sigma * b.float().std() * torch.randn(b.shape, generator=g, device=b.device))
                  .to(b.dtype) for _ in range(8)] for b in base]
 
-        def drift_run(i):
-            l = i % L
-            queries[l].copy_(pool[l][(i // L) % 8])
-            run(i)
+        def drift_cycle(c):
+            for l in range(L):
+                queries[l].copy_(pool[l][c % 8])
+            run_cycle()
 
-        for i in range(args.warmup):
-            drift_run(i)
+        n_cyc = max(1, args.steps // L)
+        for c in range(max(1, args.warmup // L)):
+            drift_cycle(c)
         torch.cuda.synchronize()
         t0 = time.perf_counter()
-        for i in range(args.steps):
-            drift_run(i)
+        for c in range(n_cyc):
+            drift_cycle(c)
         torch.cuda.synchronize()
-        t_d = (time.perf_counter() - t0) / args.steps
-        # hit and miss blocks of 8 more (untimed) look-ups per layer
+        t_d = (time.perf_counter() - t0) / (n_cyc * L)
+        # hit and miss blocks of 8 more (untimed) cycles
         dh = dm = 0
-        for i in range(args.steps, args.steps + 8 * L):
-            drift_run(i)
+        for c in range(n_cyc, n_cyc + 8):
+            drift_cycle(c)
             torch.cuda.synchronize()
-            h_, m_ = cache.block_cache_stats(i % L)
-            dh += h_
-            dm += m_
+            for l in range(L):
+                h_, m_ = cache.block_cache_stats(l)
+                dh += h_
+                dm += m_
         per_step_miss = dm / (8 * L)
         drift[f"noise_{sigma}"] = {"us_per_layer_step": t_d * 1e6, "hit_blocks_sampled": dh, "miss_blocks_sampled": dm,
                                    "hit_fraction": dh / max(dh + dm, 1),
@@ -360,7 +370,7 @@ def bench_host(args, cfg, cache, queries, L, nprobe, es, static_len):
         "config": {"workload": f"{args.config}: {cfg['desc']}; clustered K/V in pinned host memory, block cache of "
                                f"{cache.cache_size if hasattr(cache, 'cache_size') else '?'} blocks per group, "
                                f"block cache manager on the {cache.block_cache}, nprobe {nprobe}, estimation zone {es}, {L} layers, "
-                               f"{'HIP graph replay' if use_graph else 'eager launches'}, warm = same "
+                               f"{'HIP graph replay (a cycle of the layers per graph)' if use_graph else 'eager launches'}, warm = same "
                                f"queries repeated", "batch": B, "context_tokens": cfg["N"],
                    "layers_for_tokens_per_s": cfg["L"], "warm_hit_blocks": hit, "warm_miss_blocks": miss},
         "drifting_queries": drift, "roofline": None, "cpu_baseline": None}))
@@ -447,6 +457,31 @@ def main():
             if not torch.equal(graphs[l][1], outs[l]):
                 sys.exit(f"graph replay of layer {l} differs from the eager result")
 
+    # one graph for a whole cycle of the L layers (what a decoded token replays): a graph launch has a
+    # fixed cost of its own, which a per-layer graph would pay L times per token
+    # (a config with few layers repeats its cycle inside the graph, up to 32 steps per graph)
+    cycle, CL = None, L * max(1, 32 // L)
+    if graphs is not None:
+        cycle = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(cycle):
+            cycle_outs = [step(i % L) for i in range(CL)]
+        cycle.replay()
+        torch.cuda.synchronize()
+        for i in range(CL):
+            if not torch.equal(cycle_outs[i], outs[i % L]):
+                sys.exit(f"cycle graph: step {i} differs from the eager result")
+
+    def run_steps(i0, n):
+        """Steps i0 .. i0+n-1 of the layer cycle: whole graphs of CL steps, the rest per layer."""
+        i = i0
+        while i < i0 + n:
+            if cycle is not None and i % CL == 0 and i + CL <= i0 + n:
+                cycle.replay()
+                i += CL
+            else:
+                run(i)
+                i += 1
+
     def run(i):
         l = i % L
         if graphs is not None:
@@ -454,12 +489,10 @@ def main():
         else:
             step(l)
 
-    for i in range(args.warmup):
-        run(i)
+    run_steps(0, max(args.warmup, CL))
     torch.cuda.synchronize()
     t0 = time.perf_counter()
-    for i in range(args.steps):
-        run(i)
+    run_steps(0, args.steps)
     torch.cuda.synchronize()
     t_step = (time.perf_counter() - t0) / args.steps
 
@@ -468,29 +501,28 @@ def main():
     # launch stream; the difference is attend_kernel plus the gap in front of it
     t_attn_in_step = None
     if graphs is not None:
-        sel_graphs = []
-        for l in range(L):
-            gr = torch.cuda.CUDAGraph()
-            with torch.cuda.graph(gr):
-                cache._select(queries[l], l, l % 2, True)
-            sel_graphs.append(gr)
+        sel_cycle = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(sel_cycle):
+            for i in range(CL):
+                cache._select(queries[i % L], i % L, i % 2, True)
         torch.cuda.synchronize()
         e0, e1, e2 = (torch.cuda.Event(enable_timing=True) for _ in range(3))
         best = [float("inf"), float("inf")]
+        n_cyc = max(1, args.steps // CL)
         for _ in range(3):
-            for i in range(args.warmup):
-                run(i)
+            for _ in range(2):
+                cycle.replay()
             e0.record()
-            for i in range(args.steps):
-                graphs[i % L][0].replay()
+            for _ in range(n_cyc):
+                cycle.replay()
             e1.record()
-            for i in range(args.steps):
-                sel_graphs[i % L].replay()
+            for _ in range(n_cyc):
+                sel_cycle.replay()
             e2.record()
             torch.cuda.synchronize()
             best = [min(best[0], e0.elapsed_time(e1)), min(best[1], e1.elapsed_time(e2))]
-        t_attn_in_step = (best[0] - best[1]) * 1e-3 / args.steps
-        t_select_in_step = best[1] * 1e-3 / args.steps
+        t_attn_in_step = (best[0] - best[1]) * 1e-3 / (n_cyc * CL)
+        t_select_in_step = best[1] * 1e-3 / (n_cyc * CL)
 
     # per-kernel pass: the same layer cycle launched eagerly, one event pair around each entry point's
     # launches on the launch stream (cold caches as in the timed region: every step is another layer)
@@ -537,7 +569,7 @@ def main():
         "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
         "config": {"workload": f"{args.config}: {cfg['desc']}; nprobe {nprobe}, estimation zone {es}, "
                                f"steady zone {static_len}, {L} layers with independent seeds, "
-                               f"{'HIP graph replay' if graphs is not None else 'eager launches'}",
+                               f"{'HIP graph replay (32 layer-steps per graph)' if graphs is not None else 'eager launches'}",
                    "batch": B, "context_tokens": cfg["N"], "layers_for_tokens_per_s": Lmodel,
                    "retrieved_tokens_per_group": t_ret / BG},
         "step_roofline": {"bound": "hbm", "algorithmic_bytes": total_bytes, "achieved": total_bytes / t_step / 1e9,
@@ -559,7 +591,7 @@ def main():
                           "frac": attn_bytes / t_dom / HBM_PEAK, "traffic": MEASURED_TRAFFIC.get(args.config),
                           "launch_us": t_dom * 1e6, "eager_event_us": t_attn * 1e6, "null_launch_us": t_null * 1e6,
                           "algorithmic_bytes": attn_bytes,
-                          "launches_timed": args.steps if t_attn_in_step else n_k}
+                          "launches_timed": max(1, args.steps // CL) * CL if t_attn_in_step else n_k}
     if t_attn_in_step:
         result["stages"]["score_select"]["us_in_step"] = t_select_in_step * 1e6
         result["stages"]["wave_attention"]["us_in_step"] = t_attn_in_step * 1e6
