@@ -471,13 +471,25 @@ def main():
             if not torch.equal(cycle_outs[i], outs[i % L]):
                 sys.exit(f"cycle graph: step {i} differs from the eager result")
 
+    # the timed region is exactly args.steps layer-steps: whole graphs of CL steps, then one graph that
+    # holds the remaining steps % CL steps
+    tail, n_tail = None, args.steps % CL
+    if graphs is not None and n_tail:
+        tail = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(tail):
+            for i in range(n_tail):
+                step(i % L)
+
     def run_steps(i0, n):
-        """Steps i0 .. i0+n-1 of the layer cycle: whole graphs of CL steps, the rest per layer."""
+        """Steps i0 .. i0+n-1 of the layer cycle."""
         i = i0
         while i < i0 + n:
             if cycle is not None and i % CL == 0 and i + CL <= i0 + n:
                 cycle.replay()
                 i += CL
+            elif tail is not None and i % CL == 0 and i + n_tail == i0 + n:
+                tail.replay()
+                i += n_tail
             else:
                 run(i)
                 i += 1
