@@ -24,6 +24,8 @@ def _make_cache(dev, residency, layers, B, Hkv, gs, ctx, n_centroids, n_segment,
     # "host-cpu": host-resident store with the reference's worker-thread block cache manager;
     # "host": the same store with the device-side manager
     block_cache = "host" if residency == "host-cpu" else "device"
+    if residency == "device-pos":       # device-resident store with the steady length kept on the device
+        residency, device_positions = "device", True
     residency = "host" if residency == "host-cpu" else residency
     return retroinfer_cache(
         valid_start=[0] * B, layer_num=layers, batch_size=B, max_length=ctx + new, num_key_value_heads=Hkv,
@@ -251,7 +253,7 @@ def test_next_layer_cluster_estimation(dev, residency):
 
 
 
-@pytest.mark.parametrize("residency", ["device", "host", "host-cpu"])
+@pytest.mark.parametrize("residency", ["device", "host", "host-cpu", "device-pos"])
 def test_index_growth_after_1024_generated_tokens(dev, residency):
     """Decode-time index update (reference: retroinfer_cache.py:462-546): once the steady zone holds
     1024 tokens beyond its 4 + 64, they are clustered into 64 new centroids and appended to the index
@@ -269,9 +271,14 @@ def test_index_growth_after_1024_generated_tokens(dev, residency):
     q = torch.randn(B, 1, Hkv * gs, 128, generator=g).to(torch.bfloat16).to(dev)
     for t in range(1030):
         cache.decode_update_kv_cache(gk[:, t:t + 1].to(dev), gv[:, t:t + 1].to(dev), 0)
-        if t in (0, 700):          # keep the block cache busy before the index grows
+        # keep the block cache busy before the index grows; with the steady length on the device
+        # every token's attention runs (it is what moves the device-side position on)
+        if t in (0, 700) or residency == "device-pos":
             cache.compute(q, 0)
     torch.cuda.synchronize()
+    if residency == "device-pos":
+        assert int(cache.steady_len_dev) == cache.static_pattern_total + 1
+        assert int(cache.steady_pos_dev) == cache.static_pattern_total
     assert cache.n_centroids == nc + 64 and cache.centroids[0].shape[1] == nc + 64
     assert cache.static_pattern_total == 4 + 64 + (1030 - 1024)   # the fold happened on the 1025th call
     lk, lv = cache.list_keys[0].view(BG, -1, 128), cache.list_values[0].view(BG, -1, 128)
