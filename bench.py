@@ -134,7 +134,11 @@ def bench_kmeans(cfg, dev, iters=10, reps=3):
         ks.append(k.to(torch.bfloat16)); vs.append(v.to(torch.bfloat16))
     K, V = torch.stack(ks).contiguous(), torch.stack(vs).contiguous()
     K = (K - K.mean(dim=1, keepdim=True)).contiguous()          # keys are centred before clustering
-    r = segment_k_means_csr(K, V, nc, iters, S)                  # warm-up
+    r = segment_k_means_csr(K, V, nc, iters, S, reuse_graph=False)   # warm-up; its result is kept below
+    # the library replays a clustering as one captured graph from the third call with keys at the same
+    # address on (as every layer and sequence of a prefill after the first two does): two untimed calls
+    for _ in range(2):
+        segment_k_means_csr(K, V, nc, iters, S)
     t = time_region(lambda: segment_k_means_csr(K, V, nc, iters, S), reps)
     # the global assignment alone: the one launch that holds most of the FLOPs
     assign = torch.empty((Hkv, N), dtype=torch.int32, device=dev)
@@ -145,7 +149,8 @@ def bench_kmeans(cfg, dev, iters=10, reps=3):
     # random choice of initial tokens
     g = torch.Generator(device=dev).manual_seed(0)
     init = torch.sort(torch.randperm(N, generator=g, device=dev)[:nc]).values
-    segment_k_means_csr(K, V, nc, iters, 1, init_indices=init)
+    for _ in range(2):
+        segment_k_means_csr(K, V, nc, iters, 1, init_indices=init)
     t_un = time_region(lambda: segment_k_means_csr(K, V, nc, iters, 1, init_indices=init), reps)
     flops_un = 2.0 * 128 * Hkv * N * iters * nc
     unseg = {"ms_per_sequence": t_un * 1e3, "algorithmic_flops": flops_un, "achieved": flops_un / t_un / 1e12,

@@ -110,6 +110,7 @@ class retroinfer_cache(KV_Cache):
         self.cluster_start = [zeros((BG, n_centroids), torch.int32, dev(l)) for l in L]
         self.cluster_size_i32 = [zeros((BG, n_centroids), torch.int32, dev(l)) for l in L]
         self.store_rows = [[0] * BG for _ in L]  # rows of the store in use, per group
+        self._centred_keys = {}                  # (device, tokens) -> buffer of centred keys for the clustering
         if self.kv_residency == "device":
             self._init_device_store()
         else:
@@ -248,6 +249,7 @@ class retroinfer_cache(KV_Cache):
                 self.stage_keys = self.stage_values = None
         self.clusters_cpu = self.cluster_size_cpu = None
         self.temp_keys = self.temp_values = None
+        self._centred_keys.clear()
 
     # ------------------------------------------------------------------ prefill
     def prefill_update_kv_cache(self, query_states, key_states, value_states, layer_idx, batch_idx):
@@ -287,8 +289,16 @@ class retroinfer_cache(KV_Cache):
             zone[layer_idx][batch_idx, :, sps:spt] = src[0, seq_len - spe:seq_len].transpose(0, 1)
 
         mean_key = torch.mean(self.temp_keys, dim=1, keepdim=True)
-        km = segment_k_means_csr(self.temp_keys - mean_key, self.temp_values, self.n_centroids,
-                                 num_segments=self.n_segment)
+        # the centred keys go to a buffer that keeps its address from call to call: the clustering of
+        # every further layer and sequence of this length then replays one captured graph
+        ck = self._centred_keys.get((dkey, valid_length))
+        if ck is None:
+            if len(self._centred_keys) >= 2:
+                self._centred_keys.clear()
+            ck = torch.empty_like(self.temp_keys)
+            self._centred_keys[(dkey, valid_length)] = ck
+        torch.sub(self.temp_keys, mean_key, out=ck)
+        km = segment_k_means_csr(ck, self.temp_values, self.n_centroids, num_segments=self.n_segment)
         self.centroids[layer_idx][rows].copy_(km.centroids + mean_key)
         self.value_sum[layer_idx][rows].copy_(km.value_sum)
         self.centroids_mask[layer_idx][rows].copy_(km.counts == 0)
