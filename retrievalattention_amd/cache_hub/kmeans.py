@@ -67,14 +67,16 @@ _MAX_GRAPHS = 4
 
 
 def segment_k_means_csr(key, value, num_centroids, num_iters=10, num_segments=1, init_indices=None,
-                        reuse_graph=True):
+                        reuse_graph=False):
     """Runs the clustering and returns a KMeansResult (no dense cluster lists, no host copy).
     key/value [G, N, 128] bf16 contiguous device tensors.
 
-    reuse_graph: the second call with keys at the same address and the same shape and parameters
-    captures the launches into a HIP graph, and later such calls replay it.  Results of replayed
-    calls live in the graph's own memory: they are overwritten by the next replay for the same key
-    tensor, so a caller that keeps them across calls copies them (value sums are always fresh)."""
+    reuse_graph (off unless asked for): the second call with keys at the same address and the same
+    shape and parameters captures the launches into a HIP graph, and later such calls replay it.
+    Results of replayed calls live in the graph's own memory: THEY ARE OVERWRITTEN by the next replay
+    for the same key tensor, so only a caller that consumes or copies them before its next call may
+    turn this on (prefill_update_kv_cache does: it copies everything into the cache's tensors at once;
+    value sums are always fresh)."""
     G, N, D = key.shape
     if D != 128 or key.dtype != torch.bfloat16 or not key.is_contiguous():
         raise ValueError("segment_k_means: expected contiguous bf16 [G, N, 128] keys")

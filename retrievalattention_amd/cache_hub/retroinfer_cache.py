@@ -298,7 +298,8 @@ class retroinfer_cache(KV_Cache):
             ck = torch.empty_like(self.temp_keys)
             self._centred_keys[(dkey, valid_length)] = ck
         torch.sub(self.temp_keys, mean_key, out=ck)
-        km = segment_k_means_csr(ck, self.temp_values, self.n_centroids, num_segments=self.n_segment)
+        km = segment_k_means_csr(ck, self.temp_values, self.n_centroids, num_segments=self.n_segment,
+                                 reuse_graph=True)   # results are copied out below, before the next call
         self.centroids[layer_idx][rows].copy_(km.centroids + mean_key)
         self.value_sum[layer_idx][rows].copy_(km.value_sum)
         self.centroids_mask[layer_idx][rows].copy_(km.counts == 0)
@@ -377,23 +378,37 @@ class retroinfer_cache(KV_Cache):
             self.value_sum[ldx] = torch.cat((self.value_sum[ldx], km.value_sum), dim=1)
             self.centroids_mask[ldx] = torch.cat((self.centroids_mask[ldx], km.counts == 0), dim=1)
             self.cluster_size[ldx] = torch.cat((self.cluster_size[ldx], km.counts.to(self.dtype)), dim=1)
-            base = self.store_rows[ldx][0]
-            self.cluster_start[ldx] = torch.cat((self.cluster_start[ldx], km.offsets[:, :ncu] + base), dim=1)
+            # every group appends behind its own rows: sequences with different left padding hold
+            # different numbers of clustered tokens (reference: wave_buffer_cpu.cpp:658, per group)
+            bases = list(self.store_rows[ldx])
+            base_t = torch.tensor(bases, dtype=torch.int32, device=km.offsets.device)[:, None]
+            self.cluster_start[ldx] = torch.cat((self.cluster_start[ldx], km.offsets[:, :ncu] + base_t), dim=1)
             self.cluster_size_i32[ldx] = torch.cat((self.cluster_size_i32[ldx], km.counts), dim=1)
-            self.store_rows[ldx] = [base + THRESHOLD_LENGTH] * BG
+            self.store_rows[ldx] = [b + THRESHOLD_LENGTH for b in bases]
+            runs, g0 = [], 0          # runs of consecutive groups that share a base
+            for g1 in range(1, BG + 1):
+                if g1 == BG or bases[g1] != bases[g0]:
+                    runs.append((g0, g1, bases[g0]))
+                    g0 = g1
             if self.kv_residency == "device":
-                assert base + THRESHOLD_LENGTH <= self.list_stride, "cluster store is full"
-                lk = self.list_keys[ldx].view(BG, self.list_stride, D)[:, base:]
-                lv = self.list_values[ldx].view(BG, self.list_stride, D)[:, base:]
-                kernels.permute_rows(uk, km.members, lk, BG, THRESHOLD_LENGTH, THRESHOLD_LENGTH, self.list_stride)
-                kernels.permute_rows(uv, km.members, lv, BG, THRESHOLD_LENGTH, THRESHOLD_LENGTH, self.list_stride)
+                assert max(bases) + THRESHOLD_LENGTH <= self.list_stride, "cluster store is full"
+                lk = self.list_keys[ldx].view(BG, self.list_stride, D)
+                lv = self.list_values[ldx].view(BG, self.list_stride, D)
+                for g0, g1, base in runs:
+                    kernels.permute_rows(uk[g0:g1], km.members[g0:g1], lk[g0:g1, base:], g1 - g0, THRESHOLD_LENGTH,
+                                         THRESHOLD_LENGTH, self.list_stride)
+                    kernels.permute_rows(uv[g0:g1], km.members[g0:g1], lv[g0:g1, base:], g1 - g0, THRESHOLD_LENGTH,
+                                         THRESHOLD_LENGTH, self.list_stride)
             elif self.block_cache == "device":
-                assert base + THRESHOLD_LENGTH <= self.list_stride, "cluster store is full"
+                assert max(bases) + THRESHOLD_LENGTH <= self.list_stride, "cluster store is full"
                 pk, pv = torch.empty_like(uk), torch.empty_like(uv)
                 kernels.permute_rows(uk, km.members, pk, BG, THRESHOLD_LENGTH, THRESHOLD_LENGTH, THRESHOLD_LENGTH)
                 kernels.permute_rows(uv, km.members, pv, BG, THRESHOLD_LENGTH, THRESHOLD_LENGTH, THRESHOLD_LENGTH)
-                self.list_keys[ldx].view(BG, self.list_stride, D)[:, base:base + THRESHOLD_LENGTH].copy_(pk)
-                self.list_values[ldx].view(BG, self.list_stride, D)[:, base:base + THRESHOLD_LENGTH].copy_(pv)
+                lk = self.list_keys[ldx].view(BG, self.list_stride, D)
+                lv = self.list_values[ldx].view(BG, self.list_stride, D)
+                for g0, g1, base in runs:
+                    lk[g0:g1, base:base + THRESHOLD_LENGTH].copy_(pk[g0:g1])
+                    lv[g0:g1, base:base + THRESHOLD_LENGTH].copy_(pv[g0:g1])
                 self.device_lru[ldx].set_sizes(self.cluster_size_i32[ldx])
             else:
                 self.copyevents[dkey].synchronize()

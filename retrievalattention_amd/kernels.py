@@ -32,14 +32,25 @@ def _need(t, dtype, name, cuda=True):
 
 
 _workspaces = {}
+_retired_workspaces = []   # superseded scratch tensors: captured HIP graphs may still hold their addresses
 
 
 def _workspace(nbytes, device, tag):
     """Per-(device, tag) scratch tensor, grown on demand and reused across calls.  It starts
-    zeroed: the attention kernels keep arrival counters in it that they leave at zero."""
+    zeroed: the attention kernels keep arrival counters in it that they leave at zero.
+    A scratch tensor that is outgrown is never freed: a HIP graph captured earlier replays with its
+    address, so handing the block back to the allocator would let that replay write into someone else's
+    memory.  Growing (or first use) during a capture is refused: the allocation would land in the graph's
+    private pool and its zero fill would become a memset node of the graph."""
     key = (str(device), tag)
     w = _workspaces.get(key)
     if w is None or w.numel() < nbytes:
+        if torch.cuda.is_current_stream_capturing():
+            raise RuntimeError(f"scratch area '{tag}' must grow to {nbytes} bytes during a stream capture: run the "
+                               "same call once before capturing")
+        if w is not None:
+            _retired_workspaces.append(w)
+            nbytes = max(nbytes, w.numel() * 3 // 2)
         w = torch.zeros(max(nbytes, 256), dtype=torch.uint8, device=device)
         _workspaces[key] = w
     return w

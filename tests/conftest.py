@@ -18,3 +18,14 @@ def dev():
     if not torch.cuda.is_available():
         pytest.skip("no GPU")
     return torch.device("cuda:0")
+
+
+def pytest_terminal_summary(terminalreporter):
+    """Boundary ties of the zone selections against the oracle's scores: how many accepted swaps lie
+    within one bf16 ulp of the boundary score and how many need the second ulp."""
+    from tests.parity import TIE_TALLY
+    if TIE_TALLY:
+        terminalreporter.write_line("zone boundary ties vs the oracle (label: checks, swaps <= 1 ulp, swaps in (1, 2] ulp)")
+        for k in sorted(TIE_TALLY):
+            c, a, b = TIE_TALLY[k]
+            terminalreporter.write_line(f"  {k}: {c}, {a}, {b}")

@@ -6,7 +6,6 @@ import pytest
 import torch
 
 from oracle import pipeline, scoring, attention
-from oracle import kmeans as okm
 from tests.parity import check_zone_sets
 
 pytestmark = pytest.mark.gpu
@@ -19,7 +18,7 @@ def _close(got, ref):
 
 
 def _make_cache(dev, residency, layers, B, Hkv, gs, ctx, n_centroids, n_segment, nprobe, es, new=8,
-                cache_cluster_num=None, use_cluster_estimation=False, device_positions=False):
+                cache_cluster_num=None, use_cluster_estimation=False, device_positions=False, valid_start=None):
     from retrievalattention_amd.cache_hub import retroinfer_cache
     # "host-cpu": host-resident store with the reference's worker-thread block cache manager;
     # "host": the same store with the device-side manager
@@ -28,7 +27,7 @@ def _make_cache(dev, residency, layers, B, Hkv, gs, ctx, n_centroids, n_segment,
         residency, device_positions = "device", True
     residency = "host" if residency == "host-cpu" else residency
     return retroinfer_cache(
-        valid_start=[0] * B, layer_num=layers, batch_size=B, max_length=ctx + new, num_key_value_heads=Hkv,
+        valid_start=valid_start or [0] * B, layer_num=layers, batch_size=B, max_length=ctx + new, num_key_value_heads=Hkv,
         num_heads=Hkv * gs, head_dim=128, dtype=torch.bfloat16, layer_mapping={str(l): "cuda:0" for l in range(layers)},
         max_new_length=new, static_pattern_start=4, static_pattern_end=64, core=4, n_centroids=n_centroids,
         n_segment=n_segment, nprobe=nprobe, max_compute_cluster_num=nprobe + es, cache_unit_size=8,
@@ -75,8 +74,6 @@ def test_decode_matches_oracle(dev, residency):
         for b in range(B):
             for h in range(Hkv):
                 keys = K[l][b][0, 4:ctx - 64, h].cpu(); vals = V[l][b][0, 4:ctx - 64, h].cpu()
-                mean = torch.mean(keys[None], dim=1, keepdim=True)
-                a, _, _ = okm.assign(keys - mean[0], (cache.centroids[l][b * Hkv + h].cpu() - mean[0]))
                 # use the sizes the cache reports; order inside a cluster = ascending token id
                 size = cache.cluster_size[l][b * Hkv + h].cpu().float().to(torch.int64)
                 if residency == "device":
@@ -261,14 +258,21 @@ def test_index_growth_after_1024_generated_tokens(dev, residency):
     the folded tokens, and decoding afterwards matches the oracle on the grown index."""
     layers, B, Hkv, gs, ctx = 1, 2, 2, 4, 2048 + 68
     nc, nprobe, es, new = 128, 8, 40, 1100
-    cache = _make_cache(dev, residency, layers, B, Hkv, gs, ctx, nc, 1, nprobe, es, new=new)
+    # the first sequence is left-padded: it holds fewer clustered tokens than the second, so the groups
+    # append their folded tokens at different store rows (reference: wave_buffer_cpu.cpp:658)
+    vstart = [64, 0]
+    cache = _make_cache(dev, residency, layers, B, Hkv, gs, ctx, nc, 1, nprobe, es, new=new, valid_start=vstart)
     K, V = _gen(layers, B, Hkv, gs, ctx, 128, dev, 21)
     _prefill(cache, K, V, layers, B)
-    BG, N = B * Hkv, ctx - 68
+    BG = B * Hkv
+    Ng = [ctx - 68 - vstart[gi // Hkv] for gi in range(BG)]     # clustered prompt tokens per group
     g = torch.Generator().manual_seed(22)
     gk = torch.randn(B, 1030, Hkv, 128, generator=g).to(torch.bfloat16)
     gv = torch.randn(B, 1030, Hkv, 128, generator=g).to(torch.bfloat16)
     q = torch.randn(B, 1, Hkv * gs, 128, generator=g).to(torch.bfloat16).to(dev)
+    lk, lv = cache.list_keys[0].view(BG, -1, 128), cache.list_values[0].view(BG, -1, 128)
+    before_k = [lk[gi, :Ng[gi]].cpu().clone() for gi in range(BG)]
+    before_v = [lv[gi, :Ng[gi]].cpu().clone() for gi in range(BG)]
     for t in range(1030):
         cache.decode_update_kv_cache(gk[:, t:t + 1].to(dev), gv[:, t:t + 1].to(dev), 0)
         # keep the block cache busy before the index grows; with the steady length on the device
@@ -282,20 +286,34 @@ def test_index_growth_after_1024_generated_tokens(dev, residency):
     assert cache.n_centroids == nc + 64 and cache.centroids[0].shape[1] == nc + 64
     assert cache.static_pattern_total == 4 + 64 + (1030 - 1024)   # the fold happened on the 1025th call
     lk, lv = cache.list_keys[0].view(BG, -1, 128), cache.list_values[0].view(BG, -1, 128)
+    size_i = cache.cluster_size_i32[0].cpu()
+    start_new = cache.cluster_start[0].cpu()[:, nc:]
     for b in range(B):
         for h in range(Hkv):
             gi = b * Hkv + h
+            N = Ng[gi]
             folded_k = torch.cat([K[0][b][0, ctx - 64:, h].cpu(), gk[b, :960, h]])      # prompt tail + first 960 generated
             folded_v = torch.cat([V[0][b][0, ctx - 64:, h].cpu(), gv[b, :960, h]])
+            # the prompt's clusters were not touched, the folded tokens sit right behind them
+            assert torch.equal(lk[gi, :N].cpu(), before_k[gi]) and torch.equal(lv[gi, :N].cpu(), before_v[gi])
             got_k, got_v = lk[gi, N:N + 1024].cpu(), lv[gi, N:N + 1024].cpu()
-            assert torch.equal(torch.sort(got_k.float().sum(1)).values, torch.sort(folded_k.float().sum(1)).values)
-            assert torch.equal(torch.sort(got_v.float().sum(1)).values, torch.sort(folded_v.float().sum(1)).values)
-    size_i = cache.cluster_size_i32[0].cpu()
-    assert bool((size_i[:, nc:].sum(1) == 1024).all()) and bool((size_i.sum(1) == N + 1024).all())
+            # cluster by cluster: rows [start, start + size) hold tokens of the folded set in ascending
+            # token order, and every folded token sits in exactly one cluster
+            fk = {bytes(r.view(torch.int16).numpy().tobytes()): i for i, r in enumerate(folded_k)}
+            seen = []
+            for c in range(64):
+                s0, n = int(start_new[gi, c]) - N, int(size_i[gi, nc + c])
+                ids = [fk[bytes(r.view(torch.int16).numpy().tobytes())] for r in got_k[s0:s0 + n]]
+                assert ids == sorted(ids), "tokens inside a cluster must be ascending"
+                assert torch.equal(got_v[s0:s0 + n], folded_v[ids])
+                seen += ids
+            assert sorted(seen) == list(range(1024))
+    assert bool((size_i[:, nc:].sum(1) == 1024).all())
+    assert size_i.sum(1).tolist() == [n + 1024 for n in Ng]
     out = cache.compute(q, 0)
     torch.cuda.synchronize()
-    sk = [lk[gi, :N + 1024].cpu() for gi in range(BG)]
-    sv = [lv[gi, :N + 1024].cpu() for gi in range(BG)]
+    sk = [lk[gi, :Ng[gi] + 1024].cpu() for gi in range(BG)]
+    sv = [lv[gi, :Ng[gi] + 1024].cpu() for gi in range(BG)]
     start = torch.cumsum(size_i.long(), 1) - size_i.long()
     assert torch.equal(start.int(), cache.cluster_start[0].cpu())
     static_len = cache.static_pattern_total

@@ -238,17 +238,35 @@ def test_segment_k_means_invariants_and_remainder_tokens():
             assert torch.equal(a1, a2)
 
 
-def test_prefill_index_centres_by_the_bf16_mean():
-    """retroinfer_cache.py:416-432: cluster (key - mean), store centroid + mean, mask = size == 0."""
-    g = torch.Generator().manual_seed(9)
-    keys = _r((2, 512, 128), g) + torch.tensor(3.0, dtype=torch.bfloat16)
-    vals = _r((2, 512, 128), g)
-    idx = pipeline.prefill_index(keys, vals, 32, 1, num_iters=3)
-    mean = torch.mean(keys, dim=1, keepdim=True)
-    cent, _, _, csize, _ = okm.segment_k_means(keys - mean, vals, 32, 3, 1)
-    assert torch.equal(idx["centroids"], cent + mean)
-    assert torch.equal(idx["mask"], csize == 0) and torch.equal(idx["size_bf16"], csize.to(torch.bfloat16))
-    assert float(idx["centroids"].float().mean()) > 2.0     # the mean was added back
+def test_prefill_index_hand_worked_case():
+    """retroinfer_cache.py:416-432 on a case small enough to follow by hand (every number is exact in bf16).
+    Eight tokens whose keys are 3 in every dimension except dimension 0, which holds 4 4 6 6 2 2 0 0:
+    the mean is 3 everywhere, the centred keys are (1 1 3 3 -1 -1 -3 -3) e0.  Four centroids start at
+    tokens 1 3 5 7 = (1, 3, -1, -3) e0.  First pass: every positive token scores highest on 3 e0 (cluster
+    1), every negative one on -3 e0 (cluster 3); their normalised means are e0 and -e0, clusters 0 and 2
+    are empty and keep e0 and -e0.  From then on clusters 0/1 tie and so do 2/3: the smaller id wins, so
+    the positive tokens sit in cluster 0 and the negative ones in cluster 2, while 1 and 3 stay empty at
+    e0 and -e0.  The last pass does not normalise: cluster 0 ends at 2 e0, cluster 2 at -2 e0.  With the
+    mean added back dimension 0 of the four centroids reads 5 4 1 2 and every other dimension 3."""
+    D = 128
+    keys = torch.full((1, 8, D), 3.0)
+    keys[0, :, 0] = torch.tensor([4.0, 4.0, 6.0, 6.0, 2.0, 2.0, 0.0, 0.0])
+    vals = torch.arange(1.0, 9.0)[None, :, None].expand(1, 8, D).contiguous()
+    idx = pipeline.prefill_index(keys.to(torch.bfloat16), vals.to(torch.bfloat16), 4, 1, num_iters=10)
+    want = torch.full((1, 4, D), 3.0)
+    want[0, :, 0] = torch.tensor([5.0, 4.0, 1.0, 2.0])
+    assert torch.equal(idx["centroids"].float(), want)
+    assert idx["size"].tolist() == [[4, 0, 4, 0]]
+    assert idx["mask"].tolist() == [[False, True, False, True]]
+    assert idx["size_bf16"].dtype == torch.bfloat16 and idx["size_bf16"].tolist() == [[4.0, 0.0, 4.0, 0.0]]
+    assert idx["assign"].tolist() == [[0, 0, 0, 0, 2, 2, 2, 2]]
+    vs = torch.zeros(1, 4, D)
+    vs[0, 0], vs[0, 2] = 10.0, 26.0            # 1+2+3+4 and 5+6+7+8
+    assert torch.equal(idx["value_sum"].float(), vs)
+    assert idx["lists"][0, 0, :4].tolist() == [0, 1, 2, 3] and idx["lists"][0, 2, :4].tolist() == [4, 5, 6, 7]
+    # the cluster-contiguous store of this index: cluster 0's tokens, then cluster 2's
+    sk, sv, start = pipeline.cluster_store(keys[0], vals[0], idx["lists"][0].numpy(), idx["size"][0])
+    assert start.tolist() == [0, 4, 4, 8] and torch.equal(sk, keys[0]) and torch.equal(sv, vals[0])
 
 
 # ---------------------------------------------------------------- LRU model
