@@ -43,7 +43,7 @@ enum {
 const char* ri_status_string(int status);
 int ri_last_hip_error(void);
 /* ABI version: bumped when a signature changes. */
-int ri_abi_version(void);   /* 4 */
+int ri_abi_version(void);   /* 5 */
 /* Launches an empty kernel on `stream`: lets a caller measure the per-dispatch overhead that
  * event timings of back-to-back launches include.  No counterpart in the reference. */
 int ri_null_launch(ri_stream_t stream);
@@ -162,6 +162,28 @@ int ri_wave_attention(const void* q, const void* steady_k, const void* steady_v,
                       const void* cluster_size_bf16, void* out, int32_t* valid_lengths,
                       int BG, int gs, int nc, int es, float scale, void* workspace,
                       size_t workspace_bytes, ri_stream_t stream);
+
+/* ri_wave_attention for callers that cannot allocate device memory: code running under HIP stream
+ * capture, tight serving loops, harnesses that forbid hipMalloc.  No counterpart in the reference.
+ * Same arguments and result as ri_wave_attention without the workspace: the arrival counters and the
+ * split partials live in a static device array of ri_wave_attention_static_scratch_bytes() (8 MiB) that
+ * each GPU holds from the moment the library is loaded until the process ends.  The call allocates and
+ * frees nothing (no hipMalloc/hipFree, no allocating library routine); it enqueues one small kernel that
+ * clears the counters and the attention kernel on `stream`.
+ * Limit: RI_MAX_GROUPS counters plus BG * splits * pad(gs) * 520 bytes of partials must fit the array
+ * (splits <= 64 per group, about 512-768 workgroups in total; pad(gs) = 4, 8 or 16) — every benchmark
+ * shape needs under 4 MiB; larger shapes return RI_ERR_WORKSPACE.
+ * Every call on one GPU shares that GPU's array: calls that overlap in time on one GPU (different
+ * streams or threads) race and must be serialised by the caller. */
+size_t ri_wave_attention_static_scratch_bytes(void);
+int ri_wave_attention_static(const void* q, const void* steady_k, const void* steady_v,
+                             int64_t steady_stride, int static_len, const int32_t* static_len_dev,
+                             const void* store_k, const void* store_v, int64_t store_stride,
+                             const int32_t* row_src, int row_src_stride, const int32_t* ret_tok_off,
+                             const int32_t* ret_start, int np, const int32_t* meta, const int32_t* est_ids,
+                             const float* logits, const void* est_centroids, const void* value_sum,
+                             const void* cluster_size_bf16, void* out, int32_t* valid_lengths, int BG,
+                             int gs, int nc, int es, float scale, ri_stream_t stream);
 
 /* Attention over an execution buffer with the estimation zone fused in: replaces
  * gather_copy_vectors → weighted_flash_decoding (estimation) and the final

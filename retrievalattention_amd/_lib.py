@@ -24,6 +24,8 @@ SIGNATURES = {
     "ri_weighted_flash_decoding": (I, [P, P, P, P, P, P, P, P, P, I, I, I, I64, F, P, SZ, P]),
     "ri_wave_attention_workspace_bytes": (SZ, [I, I]),
     "ri_wave_attention": (I, [P, P, P, I64, I, P, P, P, I64, P, I, P, P, I, P, P, P, P, P, P, P, P, I, I, I, I, F, P, SZ, P]),
+    "ri_wave_attention_static_scratch_bytes": (SZ, []),
+    "ri_wave_attention_static": (I, [P, P, P, I64, I, P, P, P, I64, P, I, P, P, I, P, P, P, P, P, P, P, P, I, I, I, I, F, P]),
     "ri_buffer_attention": (I, [P, P, P, I64, P, I, P, P, P, P, P, I, I, I, I, F, P, SZ, P]),
     "ri_lru_access_update": (I, [P, P, P, I, P, I, P, I, P, I, P, P, P] + [P] * 12 + [P, I, I, P] + [I] * 6 + [P]),
     "ri_gather_copy_vectors": (I, [P, P, P, P, P, P, P, I, I, I, I, I, I, P]),

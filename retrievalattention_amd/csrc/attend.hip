@@ -21,6 +21,8 @@
 // cache_hub/retroinfer_cache.py:611-617 and :666-674.
 #include <stdlib.h>
 
+#include <mutex>
+
 #include "ri_common.h"
 
 #define ATT_FLAG_A 0x40000000  // descriptor bit: row lives in region A
@@ -575,10 +577,17 @@ static size_t attn_workspace_bytes(int BG, int gs) {
 extern "C" size_t ri_flash_decoding_workspace_bytes(int BG, int gs) { return attn_workspace_bytes(BG, gs); }
 extern "C" size_t ri_wave_attention_workspace_bytes(int BG, int gs) { return attn_workspace_bytes(BG, gs); }
 
+// Bytes a launch with S = S_kv + S_es splits per group really uses: the counter area, then the
+// (max, denominator) pairs and the numerators of BG * S partials.
+static size_t attn_scratch_used(int BG, int gp, int S) {
+  return RI_MAX_GROUPS * sizeof(int) + (size_t)BG * S * gp * (2 + RI_DIM) * sizeof(float);
+}
+
 static void carve_workspace(AttendParams& P, void* workspace, int BG, int gp) {
+  const int S = P.S_kv + P.S_es;
   P.counters = (int*)workspace;
   P.part_ml = (float*)((char*)workspace + RI_MAX_GROUPS * sizeof(int));
-  P.part_acc = P.part_ml + (size_t)BG * RI_MAX_SPLITS * gp * 2;
+  P.part_acc = P.part_ml + (size_t)BG * S * gp * 2;
 }
 
 static int launch_attend(AttendParams& P, int BG, int gs, hipStream_t s) {
@@ -655,25 +664,30 @@ extern "C" int ri_weighted_flash_decoding(const void* q, const void* k, const vo
   return launch_attend(P, BG, gs, (hipStream_t)stream);
 }
 
-extern "C" int ri_wave_attention(const void* q, const void* steady_k, const void* steady_v,
-                                 int64_t steady_stride, int static_len, const int32_t* static_len_dev,
-                                 const void* store_k,
-                                 const void* store_v, int64_t store_stride, const int32_t* row_src,
-                                 int row_src_stride, const int32_t* ret_tok_off, const int32_t* ret_start, int np,
-                                 const int32_t* meta, const int32_t* est_ids,
-                                 const float* logits, const void* est_centroids, const void* value_sum,
-                                 const void* cluster_size_bf16, void* out, int32_t* valid_lengths, int BG, int gs,
-                                 int nc, int es, float scale, void* workspace, size_t workspace_bytes,
-                                 ri_stream_t stream) {
-  if (!q || !steady_k || !steady_v || !store_k || !store_v || !meta || !out || !workspace) return RI_ERR_ARG;
-  if (ri_any_misaligned16(q, steady_k, steady_v, store_k, store_v, value_sum, est_centroids, out, workspace))
+// Shared body of ri_wave_attention and ri_wave_attention_static.  `scratch` holds the arrival
+// counters and the split partials; with scratch_bytes == 0 the caller vouches for its size through
+// scratch_limit (the static array) and the counters are cleared by a fill kernel first.
+__global__ void attend_clear_counters_kernel(int* counters, int n) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) counters[i] = 0;
+}
+
+static int wave_attention_impl(const void* q, const void* steady_k, const void* steady_v, int64_t steady_stride,
+                               int static_len, const int32_t* static_len_dev, const void* store_k,
+                               const void* store_v, int64_t store_stride, const int32_t* row_src,
+                               int row_src_stride, const int32_t* ret_tok_off, const int32_t* ret_start, int np,
+                               const int32_t* meta, const int32_t* est_ids, const float* logits,
+                               const void* est_centroids, const void* value_sum, const void* cluster_size_bf16,
+                               void* out, int32_t* valid_lengths, int BG, int gs, int nc, int es, float scale,
+                               void* scratch, size_t scratch_bytes, bool clear_counters, hipStream_t stream) {
+  if (!q || !steady_k || !steady_v || !store_k || !store_v || !meta || !out || !scratch) return RI_ERR_ARG;
+  if (ri_any_misaligned16(q, steady_k, steady_v, store_k, store_v, value_sum, est_centroids, out, scratch))
     return RI_ERR_ARG;
   if (!row_src && (!ret_tok_off || !ret_start || np <= 0 || np > 1023)) return RI_ERR_ARG;
   if (BG <= 0 || BG > RI_MAX_GROUPS || gs <= 0 || gs > 16 || static_len < 0 || static_len > steady_stride ||
       es < 0 || nc <= 0)
     return RI_ERR_ARG;
   if (es > 0 && (!est_ids || (!logits == !est_centroids) || !value_sum || !cluster_size_bf16)) return RI_ERR_ARG;
-  if (workspace_bytes < attn_workspace_bytes(BG, gs)) return RI_ERR_WORKSPACE;
   const int gp = gs_pad_of(gs);
   AttendParams P = {};
   P.q = (const uint16_t*)q;
@@ -711,8 +725,81 @@ extern "C" int ri_wave_attention(const void* q, const void* steady_k, const void
   // (estimation rows scored here read a centroid row and a value-sum row: they weigh like key/value rows)
   plan_splits(static_len + (row_src ? row_src_stride / 4 : np * 16), est_centroids ? 2 * es : es, BG, &P.S_kv,
               &P.S_es);
-  carve_workspace(P, workspace, BG, gp);
-  return launch_attend(P, BG, gs, (hipStream_t)stream);
+  if (scratch_bytes < attn_scratch_used(BG, gp, P.S_kv + P.S_es)) return RI_ERR_WORKSPACE;
+  carve_workspace(P, scratch, BG, gp);
+  if (clear_counters) {
+    attend_clear_counters_kernel<<<(BG + 255) / 256, 256, 0, stream>>>(P.counters, BG);
+    RI_HIP_CHECK_LAUNCH();
+  }
+  return launch_attend(P, BG, gs, stream);
+}
+
+extern "C" int ri_wave_attention(const void* q, const void* steady_k, const void* steady_v,
+                                 int64_t steady_stride, int static_len, const int32_t* static_len_dev,
+                                 const void* store_k,
+                                 const void* store_v, int64_t store_stride, const int32_t* row_src,
+                                 int row_src_stride, const int32_t* ret_tok_off, const int32_t* ret_start, int np,
+                                 const int32_t* meta, const int32_t* est_ids,
+                                 const float* logits, const void* est_centroids, const void* value_sum,
+                                 const void* cluster_size_bf16, void* out, int32_t* valid_lengths, int BG, int gs,
+                                 int nc, int es, float scale, void* workspace, size_t workspace_bytes,
+                                 ri_stream_t stream) {
+  if (workspace && workspace_bytes < attn_workspace_bytes(BG, gs)) return RI_ERR_WORKSPACE;
+  return wave_attention_impl(q, steady_k, steady_v, steady_stride, static_len, static_len_dev, store_k, store_v,
+                             store_stride, row_src, row_src_stride, ret_tok_off, ret_start, np, meta, est_ids, logits,
+                             est_centroids, value_sum, cluster_size_bf16, out, valid_lengths, BG, gs, nc, es, scale,
+                             workspace, workspace_bytes, false, (hipStream_t)stream);
+}
+
+// ------------------------------------------------------------------------------------
+// The same attention for callers that cannot allocate (code under stream capture, serving loops,
+// harnesses that forbid hipMalloc): arrival counters and split partials live in a static device
+// array of RI_STATIC_SCRATCH_BYTES that every GPU holds from the moment the library is loaded.
+// Its address is looked up once per device; host code only ever uses that address.
+// ------------------------------------------------------------------------------------
+#define RI_STATIC_SCRATCH_BYTES (8u << 20)
+#define RI_MAX_DEVICES 64
+static __device__ __align__(256) unsigned char scratch[RI_STATIC_SCRATCH_BYTES];
+static std::mutex g_scratch_mutex;
+static void* g_scratch_ptr[RI_MAX_DEVICES] = {};
+
+// device address of this GPU's copy of `scratch` (looked up on the first call on the device)
+static int static_scratch_ptr(void** out) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) { ri_set_last_hip_error((int)e); return RI_ERR_LAUNCH; }
+  if (dev < 0 || dev >= RI_MAX_DEVICES) return RI_ERR_ARG;
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (!g_scratch_ptr[dev]) {
+    void* p = nullptr;
+    e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || !p) { ri_set_last_hip_error((int)e); return RI_ERR_LAUNCH; }
+    g_scratch_ptr[dev] = p;
+  }
+  *out = g_scratch_ptr[dev];
+  return RI_OK;
+}
+
+extern "C" size_t ri_wave_attention_static_scratch_bytes(void) { return RI_STATIC_SCRATCH_BYTES; }
+
+extern "C" int ri_wave_attention_static(const void* q, const void* steady_k, const void* steady_v,
+                                        int64_t steady_stride, int static_len, const int32_t* static_len_dev,
+                                        const void* store_k, const void* store_v, int64_t store_stride,
+                                        const int32_t* row_src, int row_src_stride, const int32_t* ret_tok_off,
+                                        const int32_t* ret_start, int np, const int32_t* meta,
+                                        const int32_t* est_ids, const float* logits, const void* est_centroids,
+                                        const void* value_sum, const void* cluster_size_bf16, void* out,
+                                        int32_t* valid_lengths, int BG, int gs, int nc, int es, float scale,
+                                        ri_stream_t stream) {
+  void* ptr = nullptr;
+  const int rc = static_scratch_ptr(&ptr);
+  if (rc) return rc;
+  // the array keeps what the previous call left: the counters are cleared by a kernel on the caller's
+  // stream (a fill kernel, not a memset, so that the call can be captured into a graph)
+  return wave_attention_impl(q, steady_k, steady_v, steady_stride, static_len, static_len_dev, store_k, store_v,
+                             store_stride, row_src, row_src_stride, ret_tok_off, ret_start, np, meta, est_ids, logits,
+                             est_centroids, value_sum, cluster_size_bf16, out, valid_lengths, BG, gs, nc, es, scale, ptr,
+                             RI_STATIC_SCRATCH_BYTES, true, (hipStream_t)stream);
 }
 
 extern "C" int ri_buffer_attention(const void* q, const void* buf_k, const void* buf_v, int64_t buf_stride,

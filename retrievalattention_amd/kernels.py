@@ -292,6 +292,21 @@ def wave_attention(q, steady_k, steady_v, static_len, store_k, store_v, row_src,
           "wave_attention")
 
 
+def wave_attention_static(q, steady_k, steady_v, static_len, store_k, store_v, row_src, meta, est_ids, logits,
+                          value_sum, cluster_size_bf16, out, valid_lengths, es, scale, ret_tok_off=None,
+                          ret_start=None, est_centroids=None, static_len_dev=None):
+    """wave_attention without a scratch tensor: the library keeps the scratch in a static device array
+    (ri_wave_attention_static), so the call allocates nothing.  Calls on one GPU must not overlap."""
+    BG, gs, D = q.shape
+    nc = value_sum.shape[1]
+    check(lib().ri_wave_attention_static(
+        _p(q), _p(steady_k), _p(steady_v), steady_k.shape[-2], static_len, _p(static_len_dev), _p(store_k),
+        _p(store_v), store_k.shape[-2], _p(row_src), 0 if row_src is None else row_src.shape[1], _p(ret_tok_off),
+        _p(ret_start), 0 if ret_start is None else ret_start.shape[1], _p(meta), _p(est_ids), _p(logits),
+        _p(est_centroids), _p(value_sum), _p(cluster_size_bf16), _p(out), _p(valid_lengths), BG, gs, nc, es,
+        float(scale), _stream()), "wave_attention_static")
+
+
 def buffer_attention(q, buf_k, buf_v, cache_seqlens, est_ids, logits, value_sum, cluster_size_bf16, out, es, scale,
                      slot=0):
     """Attention over the rows [0, cache_seqlens[g]) of an execution buffer [BG, stride, 128] with the

@@ -1,0 +1,90 @@
+"""ri_wave_attention_static (the entry point that allocates nothing: scratch in a static device array)
+against ri_wave_attention, through the C ABI, on two calls in a row, the second with a smaller input.
+
+Same kernel, same split plan, same arithmetic: the outputs must be equal bit for bit.  The second,
+smaller call runs on the array the first one left behind (counters cleared by the call itself, stale
+partials of the larger call beyond what the smaller one writes)."""
+import ctypes as C
+import math
+
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+
+def _case(dev, BG, gs, nc, N, nprobe, es, seed):
+    """A selected step: runs ri_score_select on random data and returns everything the attention reads."""
+    from retrievalattention_amd import kernels
+    g = torch.Generator().manual_seed(seed)
+    bf = torch.bfloat16
+    rn = lambda *s: torch.randn(*s, generator=g).to(bf).to(dev)
+    size = torch.randint(1, 30, (BG, nc), generator=g, dtype=torch.int32)
+    size[:, -1] += (N - size.sum(1)).clamp(min=0).int()
+    size[:, 5] = 0
+    start = (torch.cumsum(size.long(), 1) - size.long()).int()
+    rows = int(size.sum(1).max())
+    d = dict(q=rn(BG, gs, 128), cent=rn(BG, nc, 128), vsum=rn(BG, nc, 128), sk=rn(BG, rows, 128), sv=rn(BG, rows, 128),
+             stk=rn(BG, 80, 128), stv=rn(BG, 80, 128), size=size.to(dev), start=start.to(dev), csz=size.to(bf).to(dev),
+             mask=(size == 0).to(torch.uint8).to(dev), rows=rows)
+    d["logits"] = torch.empty(BG, gs, nc, dtype=torch.float32, device=dev)
+    d["ret"] = torch.empty(BG, nprobe, dtype=torch.int32, device=dev)
+    d["est"] = torch.empty(BG, max(es, 1), dtype=torch.int32, device=dev)
+    d["rto"] = torch.empty(BG, nprobe + 1, dtype=torch.int32, device=dev)
+    d["rst"] = torch.empty(BG, nprobe, dtype=torch.int32, device=dev)
+    d["meta"] = torch.empty(BG, 4, dtype=torch.int32, device=dev)
+    kernels.score_select(d["q"], d["cent"], d["mask"], d["size"], d["start"], d["logits"], None, None, d["ret"],
+                         d["est"] if es else None, d["rto"], None, d["meta"], nprobe, es, 8, max(4 * nprobe, 16) * 4,
+                         1 / math.sqrt(128), ret_start=d["rst"])
+    torch.cuda.synchronize()
+    return d
+
+
+def _attend(dev, d, BG, gs, nc, nprobe, es, static, static_len=71):
+    from retrievalattention_amd import _lib
+    lib = _lib.lib()
+    p = lambda t: None if t is None else C.c_void_p(t.data_ptr())
+    out = torch.zeros(BG, gs, 128, dtype=torch.bfloat16, device=dev)
+    vl = torch.zeros(BG, dtype=torch.int32, device=dev)
+    stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    head = (p(d["q"]), p(d["stk"]), p(d["stv"]), 80, static_len, None, p(d["sk"]), p(d["sv"]), d["rows"], None, 0,
+            p(d["rto"]), p(d["rst"]), nprobe, p(d["meta"]), p(d["est"]) if es else None, p(d["logits"]) if es else None,
+            None, p(d["vsum"]), p(d["csz"]), p(out), p(vl), BG, gs, nc, es, 1 / math.sqrt(128))
+    if static:
+        rc = lib.ri_wave_attention_static(*head, stream)
+    else:
+        nb = lib.ri_wave_attention_workspace_bytes(BG, gs)
+        ws = torch.zeros(nb, dtype=torch.uint8, device=dev)
+        rc = lib.ri_wave_attention(*head, p(ws), nb, stream)
+    assert rc == 0, lib.ri_status_string(rc)
+    torch.cuda.synchronize()
+    return out.cpu(), vl.cpu()
+
+
+def test_static_scratch_entry_point_matches_the_workspace_one(dev):
+    from retrievalattention_amd import _lib
+    assert _lib.lib().ri_wave_attention_static_scratch_bytes() == 8 << 20
+    big = (16, 4, 1024, 16384, 18, 230)        # BG, gs, nc, tokens, nprobe, es
+    small = (3, 7, 256, 3000, 5, 0)            # fewer groups, another head padding, no estimation zone
+    for i, (BG, gs, nc, N, nprobe, es) in enumerate((big, small, big)):
+        d = _case(dev, BG, gs, nc, N, nprobe, es, seed=40 + i)
+        ref, vl_ref = _attend(dev, d, BG, gs, nc, nprobe, es, static=False)
+        got, vl = _attend(dev, d, BG, gs, nc, nprobe, es, static=True)
+        assert torch.equal(got.view(torch.int16), ref.view(torch.int16)), f"call {i}: outputs differ"
+        assert torch.equal(vl, vl_ref)
+        assert bool(ref.float().abs().sum() > 0)
+        # and once more on the array as this call left it
+        again, _ = _attend(dev, d, BG, gs, nc, nprobe, es, static=True)
+        assert torch.equal(again.view(torch.int16), ref.view(torch.int16))
+
+
+def test_static_scratch_rejects_shapes_beyond_its_array(dev):
+    """4096 groups of 16 query heads need more partial space than the 8 MiB array: a clear error, no launch."""
+    from retrievalattention_amd import _lib
+    lib = _lib.lib()
+    BG, gs = 4096, 16
+    t = torch.zeros(16, dtype=torch.uint8, device=dev)
+    p = C.c_void_p(t.data_ptr())
+    rc = lib.ri_wave_attention_static(p, p, p, 1, 1, None, p, p, 1, None, 0, p, p, 1, p, None, None, None, None, None, p,
+                                      None, BG, gs, 32, 0, 1.0, None)
+    assert rc == -3 and b"workspace" in lib.ri_status_string(rc)
