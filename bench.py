@@ -22,10 +22,36 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK = 8.0e12  # bytes/s, MI355X
 
-# HBM bytes per attend_kernel launch from rocprofv3 counter runs of this script (FETCH_SIZE and
-# WRITE_SIZE, each scaled by what the counter reads for the known-size copy of --copy-probe);
-# the summaries are kept under profiles/.
-MEASURED_TRAFFIC = {"c2": int((31709.9 * 2.000 + 1201.1 * 1.000) * 1024)}
+# HBM bytes per attend_kernel launch come from rocprofv3 counter runs of this script (FETCH_SIZE and
+# WRITE_SIZE, each scaled by what the counter reads for the known-size copy of --copy-probe): the figures
+# sit in a small data file next to the summary they were taken from, with a hash of the kernel source
+# they were measured on; a figure measured on another version of the kernel is not reported.
+TRAFFIC_FILE = os.path.join(ROOT, "profiles", "attend_kernel_traffic.json")
+ATTEND_SOURCES = [os.path.join(ROOT, "retrievalattention_amd", "csrc", f) for f in ("attend.hip", "attend_common.h")]
+
+
+def kernel_source_hash():
+    import hashlib
+    h = hashlib.sha256()
+    for f in ATTEND_SOURCES:
+        with open(f, "rb") as fh:
+            h.update(fh.read())
+    return h.hexdigest()[:16]
+
+
+def measured_traffic(config):
+    """(bytes per attend_kernel launch or None, where the figure comes from)."""
+    try:
+        with open(TRAFFIC_FILE) as fh:
+            rec = json.load(fh).get(config)
+    except (OSError, ValueError):
+        return None, f"{os.path.relpath(TRAFFIC_FILE, ROOT)} missing"
+    if not rec:
+        return None, f"no counter run recorded for {config}"
+    if rec.get("kernel_source_sha256_16") != kernel_source_hash():
+        return None, f"{rec['source']}: measured on another version of the kernel (stale, not reported)"
+    nbytes = int((rec["fetch_kib"] * rec["fetch_scale"] + rec["write_kib"] * rec["write_scale"]) * 1024)
+    return nbytes, rec["source"]
 
 CONFIGS = {
     # name: batch, kv heads, group size, clustered tokens, mixture centres, centroids, segments, outliers, layers
@@ -45,7 +71,7 @@ def log(*a):
 
 
 def build_cache(cfg, L, dev, residency="device", block_cache="device", estimate_next=False, new=2,
-                device_positions=False):
+                device_positions=False, overlap_miss_staging=True):
     from retrievalattention_amd import synth
     from retrievalattention_amd.cache_hub import retroinfer_cache
     B, Hkv, gs, N = cfg["B"], cfg["Hkv"], cfg["gs"], cfg["N"]
@@ -59,7 +85,8 @@ def build_cache(cfg, L, dev, residency="device", block_cache="device", estimate_
         n_centroids=cfg["nc"], n_segment=cfg["S"], nprobe=nprobe, max_compute_cluster_num=nprobe + es,
         cache_unit_size=8, cache_cluster_num=max(int(cfg["nc"] * 0.05), nprobe), num_gpus=1, model_size=0,
         kv_residency=residency,
-        block_cache=block_cache, use_cluster_estimation=estimate_next, device_positions=device_positions)
+        block_cache=block_cache, use_cluster_estimation=estimate_next, device_positions=device_positions,
+        overlap_miss_staging=overlap_miss_staging)
     queries = []
     t0 = time.time()
     for l in range(L):
@@ -106,6 +133,36 @@ def algorithmic_bytes(cache, cfg, nprobe, es, layer, static_len):
         "out": BG * gs * D * e,
     }
     return parts, t_ret
+
+
+def read_probe(dev, mib=64, nbuf=24):
+    """What a read-only kernel reaches: ri_probe_stream_read over `nbuf` buffers of `mib` MiB in turn
+    (1.5 GiB in all, far more than the 256 MB last-level cache holds), one launch per buffer inside a
+    HIP graph, for several workgroup counts and loads in flight; best of five replays each."""
+    from retrievalattention_amd import _lib
+    lib = _lib.lib()
+    nbytes = mib << 20
+    bufs = [torch.ones(nbytes, dtype=torch.uint8, device=dev) for _ in range(nbuf)]
+    sink = torch.zeros(16, dtype=torch.uint8, device=dev)
+    out = {}
+    for wgs in (256, 512, 1024, 2048, 4096):
+        for u in (4, 8, 16):
+            def launches():
+                st = torch.cuda.current_stream().cuda_stream
+                for b in bufs:
+                    _lib.check(lib.ri_probe_stream_read(b.data_ptr(), nbytes, wgs, u, sink.data_ptr(), st), "probe")
+            launches()
+            torch.cuda.synchronize()
+            g = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(g):
+                launches()
+            best = float("inf")
+            for _ in range(5):
+                best = min(best, time_region(g.replay, 2))
+            out[f"{wgs}x256_threads_{u}_loads"] = round(nbytes * nbuf / best / 1e9, 1)
+    top = max(out, key=out.get)
+    return {"unit": "GB/s", "bytes_per_launch": nbytes, "buffers_cycled": nbuf, "best": top, "best_GBps": out[top],
+            "frac_of_peak": out[top] * 1e9 / HBM_PEAK, "all": out}
 
 
 def time_region(fn, iters):
@@ -169,8 +226,8 @@ def cpu_baseline(cache, cfg, queries, nprobe, es, static_len, max_seconds=30.0):
     torch.set_num_threads(os.cpu_count() or 1)
     l = 0
     rows = cache.store_rows[l]
-    sk = [cache.list_keys[l].view(BG, -1, 128)[g, :rows[g]].cpu() for g in range(BG)]
-    sv = [cache.list_values[l].view(BG, -1, 128)[g, :rows[g]].cpu() for g in range(BG)]
+    sk = [cache.list_keys[l].view(BG, -1, 128)[g, :rows[g]].cpu().clone() for g in range(BG)]
+    sv = [cache.list_values[l].view(BG, -1, 128)[g, :rows[g]].cpu().clone() for g in range(BG)]
     args = (queries[l].view(BG, gs, 128).cpu(), cache.steady_zone_keys[l].view(BG, -1, 128).cpu(),
             cache.steady_zone_values[l].view(BG, -1, 128).cpu(), static_len, cache.centroids[l].cpu(),
             cache.value_sum[l].cpu(), cache.centroids_mask[l].cpu(), cache.cluster_size_i32[l].cpu(),
@@ -332,7 +389,7 @@ def bench_host(args, cfg, cache, queries, L, nprobe, es, static_len):
     # drifting queries: each step's query is the layer's query plus noise drawn from a small pool, so
     # part of every probe list is new and its blocks come over the host link
     drift = {}
-    for sigma in (0.5, 0.75, 1.0):
+    for sigma in [float(x) for x in args.drift.split(",") if x]:
         g = torch.Generator(device=queries[0].device).manual_seed(7)
         base = [q.clone() for q in queries]
         pool = [[(b.float() + sigma * b.float().std() * torch.randn(b.shape, generator=g, device=b.device))
@@ -367,6 +424,79 @@ def bench_host(args, cfg, cache, queries, L, nprobe, es, static_len):
                                    "host_link_GBps": per_step_miss * 8 * 128 * 2 * 2 / t_d / 1e9}
         for q, b in zip(queries, base):
             q.copy_(b)
+    # warm steady state, stage by stage: the same layer cycle launched eagerly with an event pair around
+    # each stage (every retrieved block hits: the stream of cache blocks, estimation rows and steady zone
+    # through attend_kernel is what moves the bytes)
+    BG, gs = cfg["B"] * cfg["Hkv"], cfg["gs"]
+    stage_us = None
+    if cache.block_cache == "device":
+        from retrievalattention_amd import kernels
+        names = ["score_select", "lru_access_update", "concat_gather (miss staging)", "attention", "admission scatter"]
+        n_k = max(L, min(args.steps, 128) // L * L)
+        ev = [[torch.cuda.Event(enable_timing=True) for _ in range(6)] for _ in range(n_k)]
+        D, rows, stage0 = 128, cache.cache_blocks * cache.page_size, cache.cache_size * cache.page_size
+        out_tmp = torch.empty((BG, gs, D), dtype=torch.bfloat16, device=queries[0].device)
+        for i in range(n_k):
+            l, e = i % L, ev[i]
+            q = queries[l].view(BG, gs, D)
+            ck, cv = cache.cache_keys[l].view(BG, rows, D), cache.cache_values[l].view(BG, rows, D)
+            e[0].record()
+            cache._select(queries[l], l, 0, False)
+            e[1].record()
+            cache._access_in_place(l, 0)
+            e[2].record()
+            cache._stage_misses(l, 0)
+            e[3].record()
+            kernels.wave_attention(q, cache.steady_zone_keys[l], cache.steady_zone_values[l], static_len, ck, cv,
+                                   cache.row_src, cache.meta, cache.est_ids[0] if es > 0 else None,
+                                   cache.logits if es > 0 else None, cache.value_sum[l], cache.cluster_size[l], out_tmp,
+                                   cache.valid_lengths[0], es, cache.RSQRT_DIM)
+            e[4].record()
+            kernels.gather_copy_and_scatter(
+                ck[:, stage0:], cache.cache_keys[l], cv[:, stage0:], cache.cache_values[l],
+                cache.update_buffer_indices[l], cache.update_unit_sizes[l], cache.update_cache_indices[l],
+                cache.update_num_units[l], BG, rows, cache.cache_stride, cache.buffer_size, 0)
+            e[5].record()
+            if i % 16 == 15:
+                torch.cuda.synchronize()
+        torch.cuda.synchronize()
+        stage_us = {nm: sum(e[k].elapsed_time(e[k + 1]) for e in ev) * 1e3 / n_k for k, nm in enumerate(names)}
+    parts, t_ret = algorithmic_bytes(cache, cfg, nprobe, es, (L - 1), static_len)
+    attn_bytes = parts["estimation"] + parts["kv"] + parts["out"]
+    total_bytes = sum(parts.values())
+    roofline = None
+    if stage_us is not None:
+        t_attn = stage_us["attention"] * 1e-6
+        roofline = {"bound": "hbm", "kernel": "attend_kernel (ri_wave_attention over the block cache, every block a hit)",
+                    "achieved": attn_bytes / t_attn / 1e9, "peak": HBM_PEAK / 1e9, "unit": "GB/s",
+                    "frac": attn_bytes / t_attn / HBM_PEAK, "traffic": None,
+                    "traffic_source": "no counter run recorded for the host-resident path",
+                    "launch_us": stage_us["attention"], "algorithmic_bytes": attn_bytes,
+                    "note": "event pair around one eager launch (includes its dispatch)"}
+    cpu = None
+    if not args.no_cpu_baseline:
+        t_cpu, n, ref = cpu_baseline(cache, cfg, queries, nprobe, es, static_len)
+        out0 = step(0)
+        torch.cuda.synchronize()
+        d = (out0.view(BG, gs, 128).cpu().float() - ref.float()).abs()
+        cpu = {"value": B / (cfg["L"] * t_cpu), "unit": "tokens/s", "us_per_layer_step": t_cpu * 1e6,
+               "cores": torch.get_num_threads(), "kind": "port",
+               "sample": f"median of {n} full-shape decode layer-steps of layer 0 (oracle/pipeline.py)",
+               "note": "the checker's restatement, not a tuned CPU implementation: float64 matrix products and a "
+                       "Python loop over the groups",
+               "max_abs_vs_gpu": float(d.max()), "mean_abs_vs_gpu": float(d.mean())}
+    link = max((v["host_link_GBps"] for v in drift.values()), default=0.0)
+    # what the link gives a plain copy: 256 MiB from pinned host memory to the device, best of 5
+    pin = torch.empty(256 << 20, dtype=torch.uint8, pin_memory=True)
+    dst = torch.empty(256 << 20, dtype=torch.uint8, device=queries[0].device)
+    t_copy = float("inf")
+    for _ in range(5):
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        dst.copy_(pin, non_blocking=True)
+        torch.cuda.synchronize()
+        t_copy = min(t_copy, time.perf_counter() - t0)
+    link_peak = pin.numel() / t_copy / 1e9
     print(json.dumps({
         "metric": "decode tokens/s at 128K ctx (attention only, B / (L * t_layer_step)); us/layer-step and % HBM roofline alongside",
         "value": B / (cfg["L"] * t_warm), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -374,11 +504,21 @@ def bench_host(args, cfg, cache, queries, L, nprobe, es, static_len):
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
         "config": {"workload": f"{args.config}: {cfg['desc']}; clustered K/V in pinned host memory, block cache of "
                                f"{cache.cache_size if hasattr(cache, 'cache_size') else '?'} blocks per group, "
-                               f"block cache manager on the {cache.block_cache}, nprobe {nprobe}, estimation zone {es}, {L} layers, "
+                               f"block cache manager on the {cache.block_cache}, miss staging "
+                               f"{'beside' if cache.overlap_miss_staging else 'before'} the attention, nprobe {nprobe}, "
+                               f"estimation zone {es}, {L} layers, "
                                f"{'HIP graph replay (a cycle of the layers per graph)' if use_graph else 'eager launches'}, warm = same "
                                f"queries repeated", "batch": B, "context_tokens": cfg["N"],
                    "layers_for_tokens_per_s": cfg["L"], "warm_hit_blocks": hit, "warm_miss_blocks": miss},
-        "drifting_queries": drift, "roofline": None, "cpu_baseline": None}))
+        "step_roofline": {"bound": "hbm", "algorithmic_bytes": total_bytes, "achieved": total_bytes / t_warm / 1e9,
+                          "peak": HBM_PEAK / 1e9, "unit": "GB/s", "frac": total_bytes / t_warm / HBM_PEAK},
+        "stages_us": stage_us,
+        "drifting_queries": drift,
+        "host_link": {"bound": "host link (pinned host memory read in place by concat_gather_kernel)",
+                      "achieved": link, "peak": link_peak, "unit": "GB/s", "frac": link / link_peak if link else None,
+                      "note": "achieved = missed K and V bytes per step over the whole step time, best drift level; "
+                              "peak = a 256 MiB copy from pinned host memory measured in this run"},
+        "roofline": roofline, "cpu_baseline": cpu}))
 
 
 def main():
@@ -396,6 +536,10 @@ def main():
     ap.add_argument("--block-cache", default="device", choices=["device", "host"],
                     help="with --residency host: block cache manager as a kernel (HIP graph replays) or the "
                          "reference's worker threads (eager launches)")
+    ap.add_argument("--overlap", action="store_true",
+                    help="with --residency host: attend the cached rows while the missed blocks are staged")
+    ap.add_argument("--drift", default="0.5,0.75,1.0",
+                    help="with --residency host: noise levels of the drifting-query measurements (empty: none)")
     ap.add_argument("--no-kmeans", action="store_true", help="skip the prefill clustering measurement")
     ap.add_argument("--estimate-next", action="store_true",
                     help="also measure the step with next-layer cluster estimation (zones of layer l+1 chosen "
@@ -403,6 +547,10 @@ def main():
     ap.add_argument("--end-to-end", action="store_true",
                     help="a whole decoded token of a random-weight model of the config's shape (all layers, one "
                          "HIP graph per token) instead of the attention-only layer-step")
+    ap.add_argument("--repeats", type=int, default=21,
+                    help="repetitions of the timed region of --steps layer-steps; the median is reported")
+    ap.add_argument("--read-probe", action="store_true",
+                    help="also measure what a read-only streaming kernel reaches on this part (ri_probe_stream_read)")
     ap.add_argument("--copy-probe", action="store_true",
                     help="also run 8 device copies of 256 MiB (a known-size kernel to scale rocprofv3 byte counters by)")
     args = ap.parse_args()
@@ -426,7 +574,8 @@ def main():
     if args.end_to_end:
         return bench_end_to_end(args, cfg, dev)
     est_next = args.residency == "device" and args.estimate_next and not args.no_graph and L >= 4
-    cache, queries, nprobe, es = build_cache(cfg, L, dev, args.residency, args.block_cache, est_next)
+    cache, queries, nprobe, es = build_cache(cfg, L, dev, args.residency, args.block_cache, est_next,
+                                             overlap_miss_staging=args.overlap)
     static_len = cache.static_pattern_total  # 4 + 64 + the token being decoded (already counted)
     if args.residency == "host":
         return bench_host(args, cfg, cache, queries, L, nprobe, es, static_len)
@@ -508,10 +657,16 @@ def main():
 
     run_steps(0, max(args.warmup, CL))
     torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    run_steps(0, args.steps)
-    torch.cuda.synchronize()
-    t_step = (time.perf_counter() - t0) / args.steps
+    # the timed region (exactly args.steps layer-steps between two synchronisations) is repeated and the
+    # median repetition reported: a short region is a single graph replay, one sample of which says little
+    reps_t = []
+    for _ in range(max(args.repeats, 1)):
+        t0 = time.perf_counter()
+        run_steps(0, args.steps)
+        torch.cuda.synchronize()
+        reps_t.append((time.perf_counter() - t0) / args.steps)
+    reps_t.sort()
+    t_step = reps_t[len(reps_t) // 2]
 
     # the dominant kernel's duration inside the replayed step: the same layer cycle without its launch
     # (score_kernel + dist_kernel + select_kernel only), both cycles timed by one event pair each on the
@@ -583,9 +738,12 @@ def main():
         "metric": "decode tokens/s at 128K ctx (attention only, B / (L * t_layer_step)); us/layer-step and % HBM roofline alongside",
         "value": tokens_per_s, "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": t_step * 1e3, "us_per_layer_step": t_step * 1e6, "higher_is_better": True,
+        "timed_region": {"repeats": len(reps_t), "statistic": "median", "min_us_per_layer_step": reps_t[0] * 1e6,
+                         "max_us_per_layer_step": reps_t[-1] * 1e6},
         "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
         "config": {"workload": f"{args.config}: {cfg['desc']}; nprobe {nprobe}, estimation zone {es}, "
-                               f"steady zone {static_len}, {L} layers with independent seeds, "
+                               f"steady zone {static_len}, {L} layers with independent seeds (seeded Gaussian-mixture "
+                               f"K/V drawn by torch's generator on the device), "
                                f"{'HIP graph replay (32 layer-steps per graph)' if graphs is not None else 'eager launches'}",
                    "batch": B, "context_tokens": cfg["N"], "layers_for_tokens_per_s": Lmodel,
                    "retrieved_tokens_per_group": t_ret / BG},
@@ -603,9 +761,10 @@ def main():
     # without it); an event pair around one eager launch also counts the dispatch of the launch
     # (eager_event_us; null_launch_us is what the same pair reads around an empty kernel).
     t_dom = t_attn_in_step if t_attn_in_step else t_attn
+    traffic, traffic_source = measured_traffic(args.config)
     result["roofline"] = {"bound": "hbm", "kernel": "attend_kernel (ri_wave_attention)",
                           "achieved": attn_bytes / t_dom / 1e9, "peak": HBM_PEAK / 1e9, "unit": "GB/s",
-                          "frac": attn_bytes / t_dom / HBM_PEAK, "traffic": MEASURED_TRAFFIC.get(args.config),
+                          "frac": attn_bytes / t_dom / HBM_PEAK, "traffic": traffic, "traffic_source": traffic_source,
                           "launch_us": t_dom * 1e6, "eager_event_us": t_attn * 1e6, "null_launch_us": t_null * 1e6,
                           "algorithmic_bytes": attn_bytes,
                           "launches_timed": max(1, args.steps // CL) * CL if t_attn_in_step else n_k}
@@ -614,6 +773,8 @@ def main():
         result["stages"]["wave_attention"]["us_in_step"] = t_attn_in_step * 1e6
     if est_next:
         result["next_layer_estimation"] = bench_estimate_next(args, cache, queries, outs, L, static_len)
+    if args.read_probe:
+        result["read_probe"] = read_probe(dev)
     if not args.no_kmeans:
         result["prefill_kmeans"] = bench_kmeans(cfg, dev)
     if not args.no_cpu_baseline:
@@ -622,6 +783,8 @@ def main():
         result["cpu_baseline"] = {"value": B / (Lmodel * t_cpu), "unit": "tokens/s", "us_per_layer_step": t_cpu * 1e6,
                                   "cores": torch.get_num_threads(), "kind": "port",
                                   "sample": f"median of {n} full-shape decode layer-steps of layer 0 (oracle/pipeline.py)",
+                                  "note": "the checker's restatement, not a tuned CPU implementation: float64 matrix "
+                                          "products and a Python loop over the groups",
                                   "max_abs_vs_gpu": float(d.max()), "mean_abs_vs_gpu": float(d.mean())}
     print(json.dumps(result))
 

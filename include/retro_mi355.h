@@ -47,6 +47,13 @@ int ri_abi_version(void);   /* 5 */
 /* Launches an empty kernel on `stream`: lets a caller measure the per-dispatch overhead that
  * event timings of back-to-back launches include.  No counterpart in the reference. */
 int ri_null_launch(ri_stream_t stream);
+/* Read-only streaming probe: `workgroups` workgroups of 256 threads read `bytes` bytes of `buf` once with
+ * `loads_in_flight` (4, 8 or 16) 16-byte loads outstanding per thread and reduce them; `sink` (4 bytes of
+ * device memory, or NULL) is written only if the reduction hits a magic value.  Lets a caller measure the
+ * read bandwidth a kernel can reach on the part, the ceiling of the streaming kernels.  No counterpart in
+ * the reference. */
+int ri_probe_stream_read(const void* buf, size_t bytes, int workgroups, int loads_in_flight, void* sink,
+                         ri_stream_t stream);
 
 /* ------------------------------------------------------------------------------------
  * (2) Centroid scoring
@@ -162,6 +169,25 @@ int ri_wave_attention(const void* q, const void* steady_k, const void* steady_v,
                       const void* cluster_size_bf16, void* out, int32_t* valid_lengths,
                       int BG, int gs, int nc, int es, float scale, void* workspace,
                       size_t workspace_bytes, ri_stream_t stream);
+
+/* One part of a wave attention over a row table (host-resident store, block cache managed on the device;
+ * cache_hub/retroinfer_cache.py:629-674, where the reference overlaps the transfer of missed blocks with
+ * other work on its copy stream): as ri_wave_attention with row_src, but of the table's rows only those
+ * whose source row lies in [src_row_lo, src_row_hi) are attended.  (prev_out [BG, gs, 128] bf16, prev_lse
+ * [BG, gs] fp32), both or neither, is an earlier part's result that is merged in (log-sum-exp rule);
+ * lse_out [BG, gs] fp32 or NULL receives this part's log-sum-exp.  static_len = 0 leaves the steady zone
+ * out, es = 0 the estimation zone.  Two calls over complementary windows, the second with the first's
+ * (out, lse_out) as its previous result, equal one ri_wave_attention up to the bf16 rounding of the
+ * intermediate output.  Workspace as for ri_wave_attention. */
+int ri_wave_attention_part(const void* q, const void* steady_k, const void* steady_v,
+                           int64_t steady_stride, int static_len, const int32_t* static_len_dev,
+                           const void* store_k, const void* store_v, int64_t store_stride,
+                           const int32_t* row_src, int row_src_stride, int src_row_lo, int src_row_hi,
+                           const int32_t* meta, const int32_t* est_ids, const float* logits,
+                           const void* value_sum, const void* cluster_size_bf16, const void* prev_out,
+                           const float* prev_lse, void* out, float* lse_out, int32_t* valid_lengths,
+                           int BG, int gs, int nc, int es, float scale, void* workspace,
+                           size_t workspace_bytes, ri_stream_t stream);
 
 /* ri_wave_attention for callers that cannot allocate device memory: code running under HIP stream
  * capture, tight serving loops, harnesses that forbid hipMalloc.  No counterpart in the reference.

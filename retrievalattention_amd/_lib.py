@@ -16,6 +16,7 @@ SIGNATURES = {
     "ri_last_hip_error": (I, []),
     "ri_abi_version": (I, []),
     "ri_null_launch": (I, [P]),
+    "ri_probe_stream_read": (I, [P, SZ, I, I, P, P]),
     "ri_batch_gemm_softmax": (I, [P, P, P, P, P, P, I, I, I, I, F, F, P]),
     "ri_score_select_workspace_bytes": (SZ, [I, I, I]),
     "ri_score_select": (I, [P] * 13 + [I, P, I, I, I, I, I, I, I, F, P, SZ, P]),
@@ -24,6 +25,7 @@ SIGNATURES = {
     "ri_weighted_flash_decoding": (I, [P, P, P, P, P, P, P, P, P, I, I, I, I64, F, P, SZ, P]),
     "ri_wave_attention_workspace_bytes": (SZ, [I, I]),
     "ri_wave_attention": (I, [P, P, P, I64, I, P, P, P, I64, P, I, P, P, I, P, P, P, P, P, P, P, P, I, I, I, I, F, P, SZ, P]),
+    "ri_wave_attention_part": (I, [P, P, P, I64, I, P, P, P, I64, P, I, I, I, P, P, P, P, P, P, P, P, P, P, I, I, I, I, F, P, SZ, P]),
     "ri_wave_attention_static_scratch_bytes": (SZ, []),
     "ri_wave_attention_static": (I, [P, P, P, I64, I, P, P, P, I64, P, I, P, P, I, P, P, P, P, P, P, P, P, I, I, I, I, F, P]),
     "ri_buffer_attention": (I, [P, P, P, I64, P, I, P, P, P, P, P, I, I, I, I, F, P, SZ, P]),

@@ -11,18 +11,21 @@
 //   * estimation rows ("EST" splits): the score of a cluster is the logit already computed
 //     by the scoring kernel, the "value" row is the cluster's value sum and the softmax
 //     denominator is weighted by the cluster size.
-// P·V runs on the vector ALU in fp32: lane (c, h) accumulates dims 8c..8c+7 over rows
-// h, h+4, h+8, h+12 of each chunk, for all heads.  Every workgroup writes a
-// (max, denominator, numerator) partial; the workgroup that finishes last for a group merges
-// the partials (and an optional previous result) with the log-sum-exp rule and writes the
+// P·V runs on the matrix cores too: the chunk's probabilities go to LDS as bf16 [head][row], the 16 x 128
+// value tile row-major, and eight MFMA 16x16x16 (B operands read with LDS transpose loads) add the chunk
+// to fp32 accumulators that hold, per lane, four heads of one dimension per 16-wide tile.  Every
+// workgroup writes a (max, denominator, numerator) partial; the workgroup that finishes last for a group
+// merges the partials (and an optional previous result) with the log-sum-exp rule and writes the
 // output, so the whole call is one launch.
 //
 // Semantics follow the weighted_flash_decoding call sites at
 // cache_hub/retroinfer_cache.py:611-617 and :666-674.
+#include <stdint.h>
 #include <stdlib.h>
 
 #include <mutex>
 
+#include "attend_common.h"
 #include "ri_common.h"
 
 #define ATT_FLAG_A 0x40000000  // descriptor bit: row lives in region A
@@ -42,6 +45,9 @@ struct AttendParams {
   int64_t strideB;
   const int32_t* row_src;
   int rs_stride;
+  // with a row table: only rows whose source row lies in [src_lo, src_hi) are attended, the others are
+  // skipped like padding rows (a second launch takes them, merging this one's result as its previous one)
+  int src_lo, src_hi;
   // or, without a row table: rank r of np clusters covers rows [ret_off[r], ret_off[r+1]) of region B,
   // stored contiguously from row ret_start[r] (ret_off has np + 1 entries, constant from the last kept rank on)
   const int32_t* ret_off;
@@ -76,105 +82,6 @@ struct AttendParams {
   int32_t* valid_lengths;    // [BG] or null: lenA + lenB(g)
 };
 
-// Softmax bookkeeping is spread over the four 16-lane groups of a wave: group h keeps
-// NH = GS_PAD/4 heads (the MFMA hands every group four heads; with GS_PAD = 4 all groups see the
-// same four, so each keeps one).  ri_head_reg(h) is the first accumulator register group h keeps,
-// ri_head_of(h, i) the head held in kept slot i.
-template <int GS_PAD>
-__device__ __forceinline__ int ri_head_reg(int h) {
-  return GS_PAD == 4 ? h : (GS_PAD == 8 ? (h >> 1) * 2 : 0);
-}
-template <int GS_PAD>
-__device__ __forceinline__ int ri_head_of(int h, int i) {
-  return (4 * h + ri_head_reg<GS_PAD>(h) + i) % GS_PAD;
-}
-
-typedef short bf16x4s_t __attribute__((ext_vector_type(4)));
-
-#define ATT_VT_STRIDE 144  // LDS row stride of the 16 x 128 value tile in bf16 elements (288 bytes)
-
-template <int GS_PAD>
-struct WaveState {
-  float m[GS_PAD / 4];
-  float l[GS_PAD / 4];
-  // P·V accumulators in MFMA 16x16 layout: acc[dt][i] of lane l = head 4*(l/16)+i, dim 16*dt + l%16
-  f32x4_t acc[8];
-};
-
-__device__ __forceinline__ uint16_t ri_to_bf16_hw(float x) {
-  const __bf16 b = (__bf16)x;
-  return __builtin_bit_cast(uint16_t, b);
-}
-
-// One chunk of 16 rows.
-//   sv[NH]  scores of the heads this lane keeps for row n = lane%16 (lane group h = lane/16)
-//   v[4]    value rows h, h+4, h+8, h+12 of the chunk, dims 8n..8n+7 (as loaded from memory)
-// Softmax bookkeeping in fp32 per lane; P goes to LDS as bf16 [head][row], the value tile to LDS
-// row-major; P·V = 8 MFMA 16x16x16 whose B operands come from LDS transpose reads
-// (ds_read_b64_tr_b16: lane l of a 16-lane group receives element l%4 of the 8-byte pieces
-// addressed by lanes l/4, l/4+4, l/4+8, l/4+12 — four consecutive rows of one column).
-template <int GS_PAD>
-__device__ __forceinline__ void chunk_update(WaveState<GS_PAD>& st, const float* sv, bool valid, float w,
-                                             const uint4 v[4], uint16_t* vt, uint16_t* pb, float* al_sh,
-                                             int lane) {
-  constexpr int NH = GS_PAD / 4;
-  const int n = lane & 15, h = lane >> 4;
-  // value tile -> LDS
-#pragma unroll
-  for (int i = 0; i < 4; ++i) *reinterpret_cast<uint4*>(vt + (h + 4 * i) * ATT_VT_STRIDE + 8 * n) = v[i];
-  float al[NH];
-  bool rescale = false;
-#pragma unroll
-  for (int i = 0; i < NH; ++i) {
-    const float s = valid ? sv[i] : -INFINITY;
-    float cm = s;
-    cm = fmaxf(cm, __shfl_xor(cm, 1));
-    cm = fmaxf(cm, __shfl_xor(cm, 2));
-    cm = fmaxf(cm, __shfl_xor(cm, 4));
-    cm = fmaxf(cm, __shfl_xor(cm, 8));
-    const float mn = fmaxf(st.m[i], cm);
-    float p;
-    if (mn == -INFINITY) {
-      al[i] = 1.f;
-      p = 0.f;
-    } else {
-      al[i] = __expf(st.m[i] - mn);  // exp(-inf) = 0 for the first chunk
-      p = valid ? __expf(s - mn) : 0.f;
-    }
-    rescale |= (al[i] != 1.f);
-    st.l[i] = st.l[i] * al[i] + w * p;
-    st.m[i] = mn;
-    pb[ri_head_of<GS_PAD>(h, i) * 16 + n] = ri_to_bf16_hw(p);
-  }
-  // the running maximum rarely moves after the first chunks: rescale only when some head's did
-  const bool any_rescale = __any(rescale);
-  if (any_rescale && n == 0) {
-#pragma unroll
-    for (int i = 0; i < NH; ++i) al_sh[ri_head_of<GS_PAD>(h, i)] = al[i];
-  }
-  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-  __builtin_amdgcn_wave_barrier();
-  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-  if (any_rescale) {
-    const float4 a4 = *reinterpret_cast<const float4*>(al_sh + 4 * h);
-#pragma unroll
-    for (int dt = 0; dt < 8; ++dt) {
-      st.acc[dt][0] *= a4.x; st.acc[dt][1] *= a4.y; st.acc[dt][2] *= a4.z; st.acc[dt][3] *= a4.w;
-    }
-  }
-  // A operand: P[head n][rows 4h..4h+3]
-  const bf16x4s_t pa = *reinterpret_cast<const bf16x4s_t*>(pb + n * 16 + 4 * h);
-  const uint16_t* vsrc = vt + (4 * h + (n >> 2)) * ATT_VT_STRIDE + 4 * (n & 3);
-#pragma unroll
-  for (int dt = 0; dt < 8; ++dt) {
-    const bf16x4s_t vb = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-        (bf16x4s_t __attribute__((address_space(3)))*)(vsrc + 16 * dt));
-    st.acc[dt] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(pa, vb, st.acc[dt], 0, 0, 0);
-  }
-  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-  __builtin_amdgcn_wave_barrier();  // the tile and P are rewritten by the next chunk
-}
-
 // rows of a wave: the group's `total` rows are cut into `nwaves` runs of a multiple of 16 rows
 __device__ __forceinline__ void wave_rows(int total, int nwaves, int wid, int* r0, int* r1) {
   int rpw = (total + nwaves - 1) / nwaves;
@@ -186,15 +93,6 @@ __device__ __forceinline__ void wave_rows(int total, int nwaves, int wid, int* r
 // Merges the S split partials of group g (and the optional previous result) and writes the
 // output: wave w of the calling workgroup takes heads w, w+4, ...; lanes first cover the splits
 // (statistics), then two dims each.
-// The partials were written by other workgroups of the same launch; they are read with
-// device-scope loads (which go past this compute unit's non-coherent cache lines) instead of
-// an acquire fence that would drop the whole cache.
-__device__ __forceinline__ float2 ri_ld_partial(const float* p) {
-  const uint64_t v = __hip_atomic_load(reinterpret_cast<const uint64_t*>(p), __ATOMIC_RELAXED,
-                                       __HIP_MEMORY_SCOPE_AGENT);
-  return make_float2(__uint_as_float((uint32_t)v), __uint_as_float((uint32_t)(v >> 32)));
-}
-
 template <int GS_PAD>
 __device__ __forceinline__ void combine_group(const AttendParams& P, int g, int S, int lenA, int lenB) {
   const int gs = P.gs;
@@ -378,6 +276,7 @@ __global__ __launch_bounds__(256, GS_PAD == 16 ? 1 : 3) void attend_kernel(Atten
               d = sh_rst[lo] + rb - sh_roff[lo];
             } else {
               d = rs ? rs[rb] : rb;
+              if (!est_split && P.row_src && (d < P.src_lo || d >= P.src_hi)) d = -1;
             }
             if (wB) w = ri_bf16_to_f32(wB[rb]);
             if (wsrc) w = ri_bf16_to_f32(wsrc[d]);
@@ -548,8 +447,22 @@ __global__ __launch_bounds__(256, GS_PAD == 16 ? 1 : 3) void attend_kernel(Atten
   }
 
   // ---------------- last workgroup of the group merges all splits ----------------
-  // The partial went out with device-coherent stores; once they have completed the arrival is
-  // announced.  The last workgroup to arrive reads every partial with device-coherent loads.
+  // Hand-off of the partials between workgroups of one launch, without fences:
+  //  * the partial was written above with agent-scope atomic stores: on gfx950 those are write-through
+  //    stores (sc1) that complete in the memory-side cache every compute unit shares, not in this
+  //    compute unit's L1 or this chiplet's L2;
+  //  * s_waitcnt(0) returns when all of this wave's stores have been acknowledged there, the barrier
+  //    makes that true for the whole workgroup, and only then does one thread announce the arrival with
+  //    an agent-scope atomic increment (performed at the same shared level);
+  //  * the workgroup that sees the count complete reads the partials with agent-scope atomic loads
+  //    (combine_group), which bypass the non-coherent cache levels.
+  // So every partial is globally visible before its arrival can be counted, and the reader cannot hit a
+  // stale line.  The C++ memory model would express this with a release increment and an acquire on the
+  // last arriver; at agent scope those compile to a write-back and an invalidate of the whole L2, which
+  // was measured at +15 us per launch (35.2 us instead of 20.0 us at the benchmark shape), while the
+  // data that must be ordered is only this workgroup's own 2 KB.  The asm statement keeps the compiler
+  // from moving the stores below the wait.
+  asm volatile("" ::: "memory");
   __builtin_amdgcn_s_waitcnt(0);
   __syncthreads();
   if (threadIdx.x == 0)
@@ -557,7 +470,9 @@ __global__ __launch_bounds__(256, GS_PAD == 16 ? 1 : 3) void attend_kernel(Atten
   __syncthreads();
   if (!sh_last) return;
   combine_group<GS_PAD>(P, g, S, lenA_all, lenB);
-  if (threadIdx.x == 0) P.counters[g] = 0;  // ready for the next launch
+  // ready for the next launch (every arrival of this launch has been counted; launches that share the
+  // workspace do not overlap)
+  if (threadIdx.x == 0) __hip_atomic_store(&P.counters[g], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 // ------------------------------------------------------------------------------------
@@ -679,8 +594,11 @@ static int wave_attention_impl(const void* q, const void* steady_k, const void* 
                                const int32_t* meta, const int32_t* est_ids, const float* logits,
                                const void* est_centroids, const void* value_sum, const void* cluster_size_bf16,
                                void* out, int32_t* valid_lengths, int BG, int gs, int nc, int es, float scale,
-                               void* scratch, size_t scratch_bytes, bool clear_counters, hipStream_t stream) {
+                               void* scratch, size_t scratch_bytes, bool clear_counters, hipStream_t stream,
+                               int src_lo = INT32_MIN, int src_hi = INT32_MAX, const void* prev_out = nullptr,
+                               const float* prev_lse = nullptr, float* lse_out = nullptr) {
   if (!q || !steady_k || !steady_v || !store_k || !store_v || !meta || !out || !scratch) return RI_ERR_ARG;
+  if ((prev_out == nullptr) != (prev_lse == nullptr) || ri_misaligned16(prev_out)) return RI_ERR_ARG;
   if (ri_any_misaligned16(q, steady_k, steady_v, store_k, store_v, value_sum, est_centroids, out, scratch))
     return RI_ERR_ARG;
   if (!row_src && (!ret_tok_off || !ret_start || np <= 0 || np > 1023)) return RI_ERR_ARG;
@@ -701,6 +619,11 @@ static int wave_attention_impl(const void* q, const void* steady_k, const void* 
   P.strideB = store_stride;
   P.row_src = row_src;
   P.rs_stride = row_src_stride;
+  P.src_lo = src_lo;
+  P.src_hi = src_hi;
+  P.prev_out = (const uint16_t*)prev_out;
+  P.prev_lse = prev_lse;
+  P.lse_out = lse_out;
   if (!row_src) {
     P.ret_off = ret_tok_off;
     P.ret_start = ret_start;
@@ -749,6 +672,29 @@ extern "C" int ri_wave_attention(const void* q, const void* steady_k, const void
                              store_stride, row_src, row_src_stride, ret_tok_off, ret_start, np, meta, est_ids, logits,
                              est_centroids, value_sum, cluster_size_bf16, out, valid_lengths, BG, gs, nc, es, scale,
                              workspace, workspace_bytes, false, (hipStream_t)stream);
+}
+
+// Part of a wave attention: the steady zone and estimation zone as asked for, and of the rows of the row
+// table only those whose source row lies in [src_row_lo, src_row_hi); an earlier part's result comes in
+// as (prev_out, prev_lse) and this part's log-sum-exp goes out, so that two launches over disjoint row
+// windows give the attention over all rows.  Used with a host-resident store: the rows already in the
+// block cache are attended while the missed blocks are still being staged, and the staged rows follow.
+extern "C" int ri_wave_attention_part(const void* q, const void* steady_k, const void* steady_v,
+                                      int64_t steady_stride, int static_len, const int32_t* static_len_dev,
+                                      const void* store_k, const void* store_v, int64_t store_stride,
+                                      const int32_t* row_src, int row_src_stride, int src_row_lo, int src_row_hi,
+                                      const int32_t* meta, const int32_t* est_ids, const float* logits,
+                                      const void* value_sum, const void* cluster_size_bf16, const void* prev_out,
+                                      const float* prev_lse, void* out, float* lse_out, int32_t* valid_lengths,
+                                      int BG, int gs, int nc, int es, float scale, void* workspace,
+                                      size_t workspace_bytes, ri_stream_t stream) {
+  if (!row_src || src_row_lo >= src_row_hi) return RI_ERR_ARG;
+  if (workspace && workspace_bytes < attn_workspace_bytes(BG, gs)) return RI_ERR_WORKSPACE;
+  return wave_attention_impl(q, steady_k, steady_v, steady_stride, static_len, static_len_dev, store_k, store_v,
+                             store_stride, row_src, row_src_stride, nullptr, nullptr, 0, meta, est_ids, logits, nullptr,
+                             value_sum, cluster_size_bf16, out, valid_lengths, BG, gs, nc, es, scale, workspace,
+                             workspace_bytes, false, (hipStream_t)stream, src_row_lo, src_row_hi, prev_out, prev_lse,
+                             lse_out);
 }
 
 // ------------------------------------------------------------------------------------

@@ -19,6 +19,43 @@ extern "C" int ri_null_launch(ri_stream_t stream) {
   return RI_OK;
 }
 
+// Read-only streaming probe: every thread keeps `U` 16-byte loads in flight and walks the buffer with a
+// grid stride, xor-reducing what it reads.  What a kernel that only reads can reach on this part is the
+// ceiling the scoring and attention kernels are measured against (a device copy also writes).
+template <int U>
+__global__ __launch_bounds__(256) void probe_read_kernel(const uint4* __restrict__ p, size_t n16, uint32_t* sink) {
+  uint32_t acc = 0;
+  const size_t stride = (size_t)gridDim.x * 256;
+  size_t i = blockIdx.x * (size_t)256 + threadIdx.x;
+  for (; i + (U - 1) * stride < n16; i += U * stride) {
+    uint4 v[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) v[u] = p[i + u * stride];
+#pragma unroll
+    for (int u = 0; u < U; ++u) acc ^= v[u].x ^ v[u].y ^ v[u].z ^ v[u].w;
+  }
+  for (; i < n16; i += stride) {
+    const uint4 v = p[i];
+    acc ^= v.x ^ v.y ^ v.z ^ v.w;
+  }
+  if (acc == 0x12345678u && sink) sink[0] = acc;   // keeps the loads alive; practically never true
+}
+
+extern "C" int ri_probe_stream_read(const void* buf, size_t bytes, int workgroups, int loads_in_flight, void* sink,
+                                    ri_stream_t stream) {
+  if (!buf || bytes < 16 || workgroups <= 0 || ri_misaligned16(buf)) return RI_ERR_ARG;
+  hipStream_t s = (hipStream_t)stream;
+  const size_t n16 = bytes / 16;
+  switch (loads_in_flight) {
+    case 4: probe_read_kernel<4><<<workgroups, 256, 0, s>>>((const uint4*)buf, n16, (uint32_t*)sink); break;
+    case 8: probe_read_kernel<8><<<workgroups, 256, 0, s>>>((const uint4*)buf, n16, (uint32_t*)sink); break;
+    case 16: probe_read_kernel<16><<<workgroups, 256, 0, s>>>((const uint4*)buf, n16, (uint32_t*)sink); break;
+    default: return RI_ERR_ARG;
+  }
+  RI_HIP_CHECK_LAUNCH();
+  return RI_OK;
+}
+
 extern "C" const char* ri_status_string(int status) {
   switch (status) {
     case RI_OK: return "ok";

@@ -292,6 +292,21 @@ def wave_attention(q, steady_k, steady_v, static_len, store_k, store_v, row_src,
           "wave_attention")
 
 
+def wave_attention_part(q, steady_k, steady_v, static_len, store_k, store_v, row_src, src_row_lo, src_row_hi, meta,
+                        est_ids, logits, value_sum, cluster_size_bf16, out, lse_out, es, scale, prev_out=None,
+                        prev_lse=None, valid_lengths=None, slot=0):
+    """wave_attention over the rows of the row table whose source row lies in [src_row_lo, src_row_hi), merging an
+    earlier part's (prev_out, prev_lse) and returning this part's log-sum-exp in lse_out [BG, gs] fp32."""
+    BG, gs, D = q.shape
+    nc = value_sum.shape[1]
+    ws = _workspace(lib().ri_wave_attention_workspace_bytes(BG, gs), q.device, f"attn{slot}")
+    check(lib().ri_wave_attention_part(
+        _p(q), _p(steady_k), _p(steady_v), steady_k.shape[-2], static_len, None, _p(store_k), _p(store_v),
+        store_k.shape[-2], _p(row_src), row_src.shape[1], int(src_row_lo), int(src_row_hi), _p(meta), _p(est_ids),
+        _p(logits), _p(value_sum), _p(cluster_size_bf16), _p(prev_out), _p(prev_lse), _p(out), _p(lse_out),
+        _p(valid_lengths), BG, gs, nc, es, float(scale), _p(ws), ws.numel(), _stream()), "wave_attention_part")
+
+
 def wave_attention_static(q, steady_k, steady_v, static_len, store_k, store_v, row_src, meta, est_ids, logits,
                           value_sum, cluster_size_bf16, out, valid_lengths, es, scale, ret_tok_off=None,
                           ret_start=None, est_centroids=None, static_len_dev=None):

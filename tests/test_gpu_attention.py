@@ -154,6 +154,22 @@ def test_wave_attention(dev, BG, gs, nc, nprobe, es, static_len, seed):
                            rows, meta, est if es else None, logits if es else None, vsum.to(dev),
                            size_bf.to(dev), out, vl, es, scale)
     torch.cuda.synchronize()
+    # the same in two parts over complementary windows of source rows (how a host-resident store attends the
+    # rows already in its block cache while the missed blocks are still being staged): steady zone,
+    # estimation zone and the lower rows first, then the upper rows with the first part merged in
+    mid = ntok // 2
+    p_out = torch.empty_like(out)
+    p_lse = torch.empty(BG, gs, dtype=torch.float32, device=dev)
+    out_p = torch.empty_like(out)
+    vl_p = torch.empty_like(vl)
+    kernels.wave_attention_part(qd, steady_k.to(dev), steady_v.to(dev), static_len, store_k.to(dev), store_v.to(dev),
+                                rows, 0, mid, meta, est if es else None, logits if es else None, vsum.to(dev),
+                                size_bf.to(dev), p_out, p_lse, es, scale, valid_lengths=vl_p)
+    kernels.wave_attention_part(qd, steady_k.to(dev), steady_v.to(dev), 0, store_k.to(dev), store_v.to(dev), rows,
+                                mid, ntok + 1, meta, None, None, vsum.to(dev), size_bf.to(dev), out_p, None, 0, scale,
+                                prev_out=p_out, prev_lse=p_lse)
+    torch.cuda.synchronize()
+    assert torch.equal(vl_p, vl)
     # the same through the rank tables (token prefix + first store row per rank) instead of the row table
     rst = torch.empty(BG, nprobe, dtype=torch.int32, device=dev)
     out_t = torch.empty_like(out)
@@ -195,3 +211,5 @@ def test_wave_attention(dev, BG, gs, nc, nprobe, es, static_len, seed):
     _close(out.cpu(), ref)
     _close(out_t.cpu(), ref)
     _close(out_c.cpu(), ref)
+    _close(out_p.cpu(), ref)
+    assert float((out_p.float() - out.float()).abs().max()) <= 1.6e-2   # the first part went through bf16

@@ -23,6 +23,8 @@ def _make_cache(dev, residency, layers, B, Hkv, gs, ctx, n_centroids, n_segment,
     # "host-cpu": host-resident store with the reference's worker-thread block cache manager;
     # "host": the same store with the device-side manager
     block_cache = "host" if residency == "host-cpu" else "device"
+    overlap = residency == "host-overlap"   # device-side manager, cached rows attended beside the miss staging
+    residency = "host" if overlap else residency
     if residency == "device-pos":       # device-resident store with the steady length kept on the device
         residency, device_positions = "device", True
     residency = "host" if residency == "host-cpu" else residency
@@ -33,7 +35,7 @@ def _make_cache(dev, residency, layers, B, Hkv, gs, ctx, n_centroids, n_segment,
         n_segment=n_segment, nprobe=nprobe, max_compute_cluster_num=nprobe + es, cache_unit_size=8,
         cache_cluster_num=cache_cluster_num if cache_cluster_num is not None else 3 * nprobe, num_gpus=1,
         model_size=8, use_cluster_estimation=use_cluster_estimation, kv_residency=residency,
-        block_cache=block_cache, device_positions=device_positions)
+        block_cache=block_cache, device_positions=device_positions, overlap_miss_staging=overlap)
 
 
 def _prefill(cache, K, V, layers, B):
@@ -55,7 +57,7 @@ def _gen(layers, B, Hkv, gs, ctx, nmix, dev, seed):
     return K, V
 
 
-@pytest.mark.parametrize("residency", ["device", "host", "host-cpu"])
+@pytest.mark.parametrize("residency", ["device", "host", "host-overlap", "host-cpu"])
 def test_decode_matches_oracle(dev, residency):
     """Prefill + three decode steps; every compute() is compared with the oracle's decode step
     run on the index the cache actually holds."""
@@ -139,7 +141,7 @@ def test_full_retrieval_equals_dense_attention(dev):
     _close(out.view(Hkv, gs, 128), ref)
 
 
-@pytest.mark.parametrize("host_kind", ["host", "host-cpu"])
+@pytest.mark.parametrize("host_kind", ["host", "host-overlap", "host-cpu"])
 def test_host_and_device_residency_agree_and_cache_warms(dev, host_kind):
     """Same inputs through both residencies: identical selections, outputs within tolerance;
     repeated queries turn misses into hits in the LRU block cache."""
@@ -166,7 +168,7 @@ def test_host_and_device_residency_agree_and_cache_warms(dev, host_kind):
         assert torch.equal(cd.valid_lengths[0].cpu(), ch.valid_lengths[0].cpu())
         hits.append(ch.block_cache_stats(0)[0])
     assert hits[0] == 0 and hits[1] > 0 and hits[2] >= hits[1]
-    if host_kind == "host":
+    if host_kind in ("host", "host-overlap"):
         # device-side manager: what sits in the block cache is what the store holds for those clusters
         lru, BG = ch.device_lru[0], B * Hkv
         size = ch.cluster_size_i32[0].cpu()
@@ -193,7 +195,7 @@ def test_host_and_device_residency_agree_and_cache_warms(dev, host_kind):
         assert checked > 0
 
 
-@pytest.mark.parametrize("residency", ["device", "host", "host-cpu"])
+@pytest.mark.parametrize("residency", ["device", "host", "host-overlap", "host-cpu"])
 def test_next_layer_cluster_estimation(dev, residency):
     """use_cluster_estimation (reference: retroinfer_cache.py:565, 582-595): layers 0 and 1 choose their
     zones from their own query; every later layer uses the zones the previous layer chose from a
