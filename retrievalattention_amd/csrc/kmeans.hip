@@ -313,6 +313,100 @@ __global__ __launch_bounds__(256) void km_sort_scatter_kernel(const int32_t* __r
   }
 }
 
+// The three launches above in one, for problems that fit one workgroup (at most KM_SMALL_MAX tokens,
+// cluster ids of at most 9 bits: a segment of the segmented iterations): sixteen waves take
+// consecutive chunks of the problem's tokens, count their digits into wave-private LDS rows, the
+// workgroup scans the [digit][wave] table in LDS, and every wave scatters its chunk as
+// km_sort_scatter_kernel does.  Same stable order, hence the same lists; the digit table never
+// leaves LDS.  Writes offsets and counts like the one-pass scan.
+#define KM_SMALL_WAVES 16
+#define KM_SMALL_MAX (KM_SMALL_WAVES * KM_SORT_CHUNK)
+
+__global__ __launch_bounds__(KM_SMALL_WAVES * 64) void km_sort_small_kernel(const int32_t* __restrict__ keys,
+                                                                           int32_t* __restrict__ offsets,
+                                                                           int32_t* __restrict__ counts,
+                                                                           int32_t* __restrict__ members, int N,
+                                                                           int nc, int bits) {
+  __shared__ int32_t sh[KM_SMALL_WAVES][KM_SORT_MAX_BINS];
+  __shared__ int32_t sh_w[KM_SMALL_WAVES];
+  const int p = blockIdx.x;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int bins = 1 << bits;
+  const int rounds = (N + KM_SMALL_WAVES * 64 - 1) / (KM_SMALL_WAVES * 64);   // 64-token rounds per wave
+  const int base = wave * rounds * 64;
+  int32_t* run = sh[wave];
+  for (int b = lane; b < bins; b += 64) run[b] = 0;
+  km_wave_lds_sync();
+  int32_t k[KM_SORT_ROUNDS];
+#pragma unroll
+  for (int r = 0; r < KM_SORT_ROUNDS; ++r) {
+    const int i = base + r * 64 + lane;
+    k[r] = (r < rounds && i < N) ? (keys[(size_t)p * N + i] & (bins - 1)) : -1;
+  }
+#pragma unroll
+  for (int r = 0; r < KM_SORT_ROUNDS; ++r)
+    if (k[r] >= 0) atomicAdd(&run[k[r]], 1);
+  __syncthreads();
+  // exclusive scan in (digit, wave) order: thread t owns digit t / 2, waves 8 (t % 2) .. + 7
+  {
+    const int t = threadIdx.x, bin = t >> 1, w0 = (t & 1) * 8;
+    int32_t v[8], tot = 0;
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      v[u] = (bin < bins) ? sh[w0 + u][bin] : 0;
+      tot += v[u];
+    }
+    int32_t inc = tot;
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+      const int32_t o = __shfl_up(inc, d);
+      if (lane >= d) inc += o;
+    }
+    if (lane == 63) sh_w[wave] = inc;
+    const int32_t pair = tot + __shfl_down(tot, 1);   // even t: the digit's count over all waves
+    __syncthreads();
+    int32_t ex = inc - tot;
+#pragma unroll
+    for (int w = 0; w < KM_SMALL_WAVES; ++w)
+      if (w < wave) ex += sh_w[w];
+    if ((t & 1) == 0 && bin < nc) {
+      offsets[(size_t)p * (nc + 1) + bin] = ex;
+      counts[(size_t)p * nc + bin] = pair;
+    }
+    if (t == 0) offsets[(size_t)p * (nc + 1) + nc] = N;
+    if (bin < bins) {
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        sh[w0 + u][bin] = ex;
+        ex += v[u];
+      }
+    }
+  }
+  __syncthreads();
+  const uint64_t below = (1ull << lane) - 1ull;
+#pragma unroll
+  for (int r = 0; r < KM_SORT_ROUNDS; ++r) {
+    if (r < rounds) {   // uniform
+      const bool valid = k[r] >= 0;
+      const int bin = valid ? k[r] : 0;
+      uint64_t peers = __ballot(valid);  // lanes of this round with the same digit
+      for (int b = 0; b < bits; ++b) {
+        const bool bit = (bin >> b) & 1;
+        const uint64_t m = __ballot(valid && bit);
+        peers &= bit ? m : ~m;
+      }
+      const int start = run[bin];
+      km_wave_lds_sync();  // every lane has read the running position before the leader advances it
+      if (valid) {
+        const int pos = start + __popcll(peers & below);
+        if (lane == 63 - __clzll((long long)peers)) run[bin] = start + __popcll(peers);
+        members[(size_t)p * N + pos] = base + r * 64 + lane;
+      }
+      km_wave_lds_sync();
+    }
+  }
+}
+
 // CSR offsets from the sorted members: position i starts every cluster in (key[i-1], key[i]]
 __global__ __launch_bounds__(256) void km_bounds_kernel(const int32_t* __restrict__ assign,
                                                         const int32_t* __restrict__ members,
@@ -341,9 +435,17 @@ __global__ __launch_bounds__(256) void km_counts_kernel(const int32_t* __restric
 // list-ordered reductions.  A list is summed in blocks of KM_BLK rows: inside a block one fp32
 // add per row in list order starting from +0, then the block sums are added in block order
 // starting from block 0's.  One wave per block, lane l owns dims 2l and 2l+1.  Lists of at
-// most KM_BLK rows (nearly all of them) finish in the first kernel; longer lists are split into
-// block items that run in parallel and are folded by a third kernel, so that a few huge
-// clusters (the first Lloyd iterations produce them) do not serialise the pass.
+// most KM_BLK rows (nearly all of them) are finished by their own wave.  A longer list (the first
+// Lloyd iterations produce a few huge ones) is split into its blocks, which other waves of the same
+// launch sum in parallel, and a second, small launch adds the block sums in order.
+//
+// Which wave sums which block needs no queue and no counter: block j of a long list that starts at
+// list offset o owns slot 2 * (o / KM_BLK) + j of its problem.  Two long lists never share a slot (a
+// list of more than KM_BLK rows ends at least as many whole blocks later as it has blocks beyond its
+// first), slots stay below km_item_cap(N), and the owner of a slot, if it has one, is the last
+// cluster whose offset is below KM_BLK * (slot / 2 + 1): every later list starts at or after the
+// owner's end, which is not.  A wave given a slot finds that cluster by a 64-way search of the
+// offsets and leaves when the cluster is short or has fewer blocks.
 // ------------------------------------------------------------------------------------
 #define KM_BLK 256
 
@@ -389,21 +491,60 @@ __device__ __forceinline__ void km_finish(float s0, float s1, int count, int nor
   *op = (uint32_t)ri_f32_to_bf16(s0) | ((uint32_t)ri_f32_to_bf16(s1) << 16);
 }
 
-// item slots of one problem: every list longer than KM_BLK takes ceil(s / KM_BLK) <= 2 s / KM_BLK
+// slots of one problem: the last list starts below N and a slot index is at most 2 (N / KM_BLK) + 1
 static inline int km_item_cap(int N) { return 2 * (N / KM_BLK) + 2; }
 
+// The long list that owns `slot`, found by the whole wave: returns its cluster (or -1), its length
+// in s, its list offset in o and the block of it that the slot stands for in j.
+// off[0 .. nc] ascending, off[0] = 0.
+__device__ __forceinline__ int km_slot_owner(const int32_t* __restrict__ off, int nc, int slot, int& s, int& o,
+                                             int& j) {
+  const int lane = threadIdx.x & 63;
+  const int limit = KM_BLK * (slot / 2 + 1);
+  // last index in [0, nc) whose offset is below limit: narrow [lo, lo + len) 64 ways per round
+  int lo = 0, len = nc;
+  while (len > 1) {
+    const int stride = (len + 63) / 64;
+    const int i = lo + lane * stride;
+    const bool below = (i < lo + len) && off[i] < limit;
+    const int k = __popcll(__ballot(below));   // probes are ascending: the first k are below (k >= 1)
+    const int nlo = lo + (k - 1) * stride;
+    len = min(stride, lo + len - nlo);
+    lo = nlo;
+  }
+  o = off[lo];
+  s = off[lo + 1] - o;
+  j = slot - 2 * (o / KM_BLK);
+  if (s <= KM_BLK || j < 0 || j >= (s + KM_BLK - 1) / KM_BLK) return -1;
+  return lo;
+}
+
+// grid (item workgroups + ceil(nc / 4), P), four waves each.  The first item_wgs workgroups take
+// one slot per wave (blocks of long lists, their fp32 sums go to partial[p][slot]); the others one
+// cluster per wave.
 template <bool MEAN>
 __global__ __launch_bounds__(256) void km_reduce_kernel(const uint16_t* __restrict__ rows,
                                                         const int32_t* __restrict__ counts,
                                                         const int32_t* __restrict__ offsets,
                                                         const int32_t* __restrict__ members,
-                                                        uint16_t* __restrict__ out, int32_t* __restrict__ item_count,
-                                                        int32_t* __restrict__ item_base,
-                                                        int32_t* __restrict__ items, int cap, int N, int nc, int seg,
+                                                        uint16_t* __restrict__ out, float2* __restrict__ partial,
+                                                        int item_wgs, int cap, int N, int nc, int seg,
                                                         int64_t head_rows, int normalize) {
   const int p = blockIdx.y;
-  const int c = blockIdx.x * 4 + (threadIdx.x >> 6);
   const int lane = threadIdx.x & 63;
+  const int32_t* off = offsets + (size_t)p * (nc + 1);
+  const uint32_t* rp = reinterpret_cast<const uint32_t*>(rows + km_row0(p, seg, head_rows, N) * RI_DIM) + lane;
+  if ((int)blockIdx.x < item_wgs) {
+    const int slot = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (slot >= cap) return;
+    int s, o, j;
+    if (km_slot_owner(off, nc, slot, s, o, j) < 0) return;
+    float s0 = 0.f, s1 = 0.f;
+    km_sum_rows(rp, members + (size_t)p * N + o, j * KM_BLK, min(s, (j + 1) * KM_BLK), s0, s1);
+    partial[((size_t)p * cap + slot) * 64 + lane] = make_float2(s0, s1);
+    return;
+  }
+  const int c = ((int)blockIdx.x - item_wgs) * 4 + (threadIdx.x >> 6);
   if (c >= nc) return;
   const int s = counts[(size_t)p * nc + c];
   uint32_t* op = reinterpret_cast<uint32_t*>(out + ((size_t)p * nc + c) * RI_DIM) + lane;
@@ -411,88 +552,47 @@ __global__ __launch_bounds__(256) void km_reduce_kernel(const uint16_t* __restri
     if (!MEAN) *op = 0u;  // empty cluster: zero value sum; the centroid is left untouched
     return;
   }
-  if (s > KM_BLK) {  // queue the blocks of a long list
-    const int nb = (s + KM_BLK - 1) / KM_BLK;
-    int base = 0;
-    if (lane == 0) {
-      base = atomicAdd(&item_count[p], nb);
-      item_base[(size_t)p * nc + c] = base;
-    }
-    base = __shfl(base, 0);
-    for (int j = lane; j < nb; j += 64) items[(size_t)p * cap + base + j] = c;
-    return;
-  }
-  const int32_t* mem = members + (size_t)p * N + offsets[(size_t)p * (nc + 1) + c];
-  const uint32_t* rp = reinterpret_cast<const uint32_t*>(rows + km_row0(p, seg, head_rows, N) * RI_DIM) + lane;
+  if (s > KM_BLK) return;  // summed by the slot waves, finished by km_reduce_fold_kernel
   float s0 = 0.f, s1 = 0.f;
-  km_sum_rows(rp, mem, 0, s, s0, s1);
+  km_sum_rows(rp, members + (size_t)p * N + off[c], 0, s, s0, s1);
   km_finish<MEAN>(s0, s1, s, normalize, op);
 }
 
-// one wave per queued block: its fp32 sum goes to partial[item]
-__global__ __launch_bounds__(256) void km_reduce_blocks_kernel(const uint16_t* __restrict__ rows,
-                                                               const int32_t* __restrict__ counts,
-                                                               const int32_t* __restrict__ offsets,
-                                                               const int32_t* __restrict__ members,
-                                                               const int32_t* __restrict__ item_count,
-                                                               const int32_t* __restrict__ item_base,
-                                                               const int32_t* __restrict__ items,
-                                                               float2* __restrict__ partial, int cap, int N, int nc,
-                                                               int seg, int64_t head_rows) {
-  const int p = blockIdx.y;
-  const int lane = threadIdx.x & 63;
-  const int n_items = item_count[p];
-  for (int it = blockIdx.x * 4 + (threadIdx.x >> 6); it < n_items; it += gridDim.x * 4) {
-    const int c = items[(size_t)p * cap + it];
-    const int j = it - item_base[(size_t)p * nc + c];
-    const int s = counts[(size_t)p * nc + c];
-    const int k0 = j * KM_BLK, k1 = min(s, k0 + KM_BLK);
-    const int32_t* mem = members + (size_t)p * N + offsets[(size_t)p * (nc + 1) + c];
-    const uint32_t* rp = reinterpret_cast<const uint32_t*>(rows + km_row0(p, seg, head_rows, N) * RI_DIM) + lane;
-    float s0 = 0.f, s1 = 0.f;
-    km_sum_rows(rp, mem, k0, k1, s0, s1);
-    partial[((size_t)p * cap + it) * 64 + lane] = make_float2(s0, s1);
-  }
-}
-
-// the wave of a long list's first item folds the block sums in block order and finishes
+// grid (item workgroups, P): the wave of a long list's first slot adds the block sums in block
+// order and finishes the cluster
 template <bool MEAN>
-__global__ __launch_bounds__(256) void km_reduce_fold_kernel(const int32_t* __restrict__ counts,
-                                                             const int32_t* __restrict__ item_count,
-                                                             const int32_t* __restrict__ item_base,
-                                                             const int32_t* __restrict__ items,
+__global__ __launch_bounds__(256) void km_reduce_fold_kernel(const int32_t* __restrict__ offsets,
                                                              const float2* __restrict__ partial,
                                                              uint16_t* __restrict__ out, int cap, int nc,
                                                              int normalize) {
   const int p = blockIdx.y;
   const int lane = threadIdx.x & 63;
-  const int n_items = item_count[p];
-  for (int it = blockIdx.x * 4 + (threadIdx.x >> 6); it < n_items; it += gridDim.x * 4) {
-    const int c = items[(size_t)p * cap + it];
-    if (it != item_base[(size_t)p * nc + c]) continue;
-    const int s = counts[(size_t)p * nc + c];
-    const int nb = (s + KM_BLK - 1) / KM_BLK;
-    const float2* pp = partial + ((size_t)p * cap + it) * 64 + lane;
-    float2 t = pp[0];
-    int j = 1;
-    for (; j + 4 <= nb; j += 4) {
-      float2 v[4];
+  const int slot = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (slot >= cap) return;
+  int s, o, j;
+  const int c = km_slot_owner(offsets + (size_t)p * (nc + 1), nc, slot, s, o, j);
+  if (c < 0 || j != 0) return;
+  const int nb = (s + KM_BLK - 1) / KM_BLK;
+  const float2* pp = partial + ((size_t)p * cap + slot) * 64 + lane;
+  float2 t = pp[0];
+  int b = 1;
+  for (; b + 4 <= nb; b += 4) {
+    float2 v[4];
 #pragma unroll
-      for (int u = 0; u < 4; ++u) v[u] = pp[(size_t)(j + u) * 64];
+    for (int u = 0; u < 4; ++u) v[u] = pp[(size_t)(b + u) * 64];
 #pragma unroll
-      for (int u = 0; u < 4; ++u) {
-        t.x += v[u].x;
-        t.y += v[u].y;
-      }
+    for (int u = 0; u < 4; ++u) {
+      t.x += v[u].x;
+      t.y += v[u].y;
     }
-    for (; j < nb; ++j) {
-      const float2 v = pp[(size_t)j * 64];
-      t.x += v.x;
-      t.y += v.y;
-    }
-    uint32_t* op = reinterpret_cast<uint32_t*>(out + ((size_t)p * nc + c) * RI_DIM) + lane;
-    km_finish<MEAN>(t.x, t.y, s, normalize, op);
   }
+  for (; b < nb; ++b) {
+    const float2 v = pp[(size_t)b * 64];
+    t.x += v.x;
+    t.y += v.y;
+  }
+  uint32_t* op = reinterpret_cast<uint32_t*>(out + ((size_t)p * nc + c) * RI_DIM) + lane;
+  km_finish<MEAN>(t.x, t.y, s, normalize, op);
 }
 
 // out[p, i, :] = in[p, members[p, i], :]; 16 lanes per row
@@ -516,20 +616,35 @@ static int km_check(int P, int N, int nc) {
   return RI_OK;
 }
 
-extern "C" int ri_kmeans_assign(const void* data, const void* centroids, int32_t* assign, int P, int N,
-                                int nc, int seg, int64_t head_rows, ri_stream_t stream) {
+static int km_sort_chunks(int N) { return (N + KM_SORT_CHUNK - 1) / KM_SORT_CHUNK; }
+
+// digit widths of the list sort: one pass when the cluster ids fit 9 bits, else two of about half each
+static void km_sort_bits(int nc, int& lo_bits, int& hi_bits) {
+  int total_bits = 1;
+  while ((1 << total_bits) < nc) ++total_bits;
+  lo_bits = total_bits <= 9 ? total_bits : (total_bits + 1) / 2;
+  hi_bits = total_bits - lo_bits;
+}
+
+static int km_assign_args(const void* data, const void* centroids, const int32_t* assign, int P, int N, int nc,
+                          int seg) {
   if (!data || !centroids || !assign) return RI_ERR_ARG;
   if (ri_any_misaligned16(data, centroids)) return RI_ERR_ARG;
   int rc = km_check(P, N, nc);
   if (rc) return rc;
   if (nc % 32 != 0 || seg <= 0 || P % seg != 0) return RI_ERR_ARG;
+  return RI_OK;
+}
+
+extern "C" int ri_kmeans_assign(const void* data, const void* centroids, int32_t* assign, int P, int N,
+                                int nc, int seg, int64_t head_rows, ri_stream_t stream) {
+  int rc = km_assign_args(data, centroids, assign, P, N, nc, seg);
+  if (rc) return rc;
   km_assign_kernel<<<dim3((N + KM_WG_TOKENS - 1) / KM_WG_TOKENS, P), KM_WAVES * 64, 0, (hipStream_t)stream>>>(
       (const uint16_t*)data, (const uint16_t*)centroids, assign, N, nc, seg, head_rows);
   RI_HIP_CHECK_LAUNCH();
   return RI_OK;
 }
-
-static int km_sort_chunks(int N) { return (N + KM_SORT_CHUNK - 1) / KM_SORT_CHUNK; }
 
 extern "C" size_t ri_kmeans_workspace_bytes(int P, int N, int nc) {
   if (P <= 0 || N <= 0 || nc <= 0) return 0;
@@ -537,23 +652,19 @@ extern "C" size_t ri_kmeans_workspace_bytes(int P, int N, int nc) {
   return ((size_t)P * KM_SORT_MAX_BINS * km_sort_chunks(N) + 2 * (size_t)P * N) * sizeof(int32_t);
 }
 
-extern "C" int ri_kmeans_build_lists(const int32_t* assign, int32_t* counts, int32_t* offsets,
-                                     int32_t* members, int P, int N, int nc, void* workspace,
-                                     size_t workspace_bytes, ri_stream_t stream) {
-  if (!assign || !counts || !offsets || !members || !workspace) return RI_ERR_ARG;
-  int rc = km_check(P, N, nc);
-  if (rc) return rc;
-  if (nc > (1 << 18)) return RI_ERR_ARG;  // two passes of at most 9 bits
-  if (workspace_bytes < ri_kmeans_workspace_bytes(P, N, nc)) return RI_ERR_WORKSPACE;
-  hipStream_t s = (hipStream_t)stream;
+static int km_build_lists(const int32_t* assign, int32_t* counts, int32_t* offsets, int32_t* members, int P, int N,
+                          int nc, void* workspace, hipStream_t s) {
   const int nchunks = km_sort_chunks(N);
   int32_t* chunk_hist = (int32_t*)workspace;
   int32_t* tmp_key = chunk_hist + (size_t)P * KM_SORT_MAX_BINS * nchunks;
   int32_t* tmp_tok = tmp_key + (size_t)P * N;
-  int total_bits = 1;
-  while ((1 << total_bits) < nc) ++total_bits;
-  const int lo_bits = total_bits <= 9 ? total_bits : (total_bits + 1) / 2;
-  const int hi_bits = total_bits - lo_bits;
+  int lo_bits, hi_bits;
+  km_sort_bits(nc, lo_bits, hi_bits);
+  if (hi_bits == 0 && N <= KM_SMALL_MAX) {
+    km_sort_small_kernel<<<P, KM_SMALL_WAVES * 64, 0, s>>>(assign, offsets, counts, members, N, nc, lo_bits);
+    RI_HIP_CHECK_LAUNCH();
+    return RI_OK;
+  }
   const dim3 cgrid((nchunks + 3) / 4, P);
   // pass over the low digit (the only one when the ids fit 9 bits)
   km_sort_hist_kernel<<<cgrid, 256, 0, s>>>(assign, chunk_hist, N, nchunks, 0, lo_bits);
@@ -584,12 +695,28 @@ extern "C" int ri_kmeans_build_lists(const int32_t* assign, int32_t* counts, int
   return RI_OK;
 }
 
+static int km_lists_args(const int32_t* assign, const int32_t* counts, const int32_t* offsets, const int32_t* members,
+                         int P, int N, int nc, const void* workspace, size_t workspace_bytes) {
+  if (!assign || !counts || !offsets || !members || !workspace) return RI_ERR_ARG;
+  int rc = km_check(P, N, nc);
+  if (rc) return rc;
+  if (nc > (1 << 18)) return RI_ERR_ARG;  // two passes of at most 9 bits
+  if (workspace_bytes < ri_kmeans_workspace_bytes(P, N, nc)) return RI_ERR_WORKSPACE;
+  return RI_OK;
+}
+
+extern "C" int ri_kmeans_build_lists(const int32_t* assign, int32_t* counts, int32_t* offsets,
+                                     int32_t* members, int P, int N, int nc, void* workspace,
+                                     size_t workspace_bytes, ri_stream_t stream) {
+  int rc = km_lists_args(assign, counts, offsets, members, P, N, nc, workspace, workspace_bytes);
+  if (rc) return rc;
+  return km_build_lists(assign, counts, offsets, members, P, N, nc, workspace, (hipStream_t)stream);
+}
+
 extern "C" size_t ri_kmeans_reduce_workspace_bytes(int P, int N, int nc) {
   if (P <= 0 || N <= 0 || nc <= 0) return 0;
-  const size_t cap = (size_t)km_item_cap(N);
-  // item_count [P] + item_base [P, nc] + items [P, cap] + partial [P, cap, 128] fp32
-  return ((size_t)P + (size_t)P * nc + (size_t)P * cap) * sizeof(int32_t) + (size_t)P * cap * RI_DIM * sizeof(float) +
-         256;
+  // partial [P, cap, 128] fp32
+  return (size_t)P * (size_t)km_item_cap(N) * RI_DIM * sizeof(float) + 256;
 }
 
 template <bool MEAN>
@@ -598,23 +725,14 @@ static int km_reduce(const void* rows, const int32_t* counts, const int32_t* off
                      size_t workspace_bytes, hipStream_t s) {
   if (workspace_bytes < ri_kmeans_reduce_workspace_bytes(P, N, nc)) return RI_ERR_WORKSPACE;
   const int cap = km_item_cap(N);
-  int32_t* item_count = (int32_t*)workspace;
-  int32_t* item_base = item_count + P;
-  int32_t* items = item_base + (size_t)P * nc;
-  uintptr_t pa = (uintptr_t)(items + (size_t)P * cap);
-  float2* partial = (float2*)((pa + 255) & ~(uintptr_t)255);
-  km_zero_kernel<<<1, 256, 0, s>>>(item_count, (size_t)P);
+  float2* partial = (float2*)(((uintptr_t)workspace + 255) & ~(uintptr_t)255);
+  const int item_wgs = (cap + 3) / 4;
+  if ((long long)item_wgs + (nc + 3) / 4 > 0x7fffffffLL) return RI_ERR_ARG;
+  km_reduce_kernel<MEAN><<<dim3(item_wgs + (nc + 3) / 4, P), 256, 0, s>>>(
+      (const uint16_t*)rows, counts, offsets, members, (uint16_t*)out, partial, item_wgs, cap, N, nc, seg, head_rows,
+      normalize);
   RI_HIP_CHECK_LAUNCH();
-  km_reduce_kernel<MEAN><<<dim3((nc + 3) / 4, P), 256, 0, s>>>((const uint16_t*)rows, counts, offsets, members,
-                                                               (uint16_t*)out, item_count, item_base, items, cap, N,
-                                                               nc, seg, head_rows, normalize);
-  RI_HIP_CHECK_LAUNCH();
-  const int gx = min((cap + 3) / 4, 1024);
-  km_reduce_blocks_kernel<<<dim3(gx, P), 256, 0, s>>>((const uint16_t*)rows, counts, offsets, members, item_count,
-                                                      item_base, items, partial, cap, N, nc, seg, head_rows);
-  RI_HIP_CHECK_LAUNCH();
-  km_reduce_fold_kernel<MEAN><<<dim3(gx, P), 256, 0, s>>>(counts, item_count, item_base, items, partial,
-                                                          (uint16_t*)out, cap, nc, normalize);
+  km_reduce_fold_kernel<MEAN><<<dim3(item_wgs, P), 256, 0, s>>>(offsets, partial, (uint16_t*)out, cap, nc, normalize);
   RI_HIP_CHECK_LAUNCH();
   return RI_OK;
 }

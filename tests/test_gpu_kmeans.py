@@ -152,6 +152,66 @@ def test_long_lists_blocked_sums(dev):
             assert torch.equal(vs[p].cpu(), okm.value_sum(vals[p], a, nc))
 
 
+def test_long_lists_back_to_back(dev):
+    """Long lists placed so that their blocks sit as close together as the layout allows (lengths
+    just above one, two and three blocks, at offsets just below and at block boundaries, with empty
+    and one-row clusters between and after them): every block is summed exactly once, in order."""
+    from retrievalattention_amd import kernels
+    sizes = [[255, 257, 0, 257, 1, 511, 0, 0, 512, 513, 255, 769, 3, 0, 300, 0],
+             [0, 0, 1025, 1, 257, 257, 257, 0, 2, 256, 256, 258, 254, 768, 0, 0],
+             [4000, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 257]]
+    P, nc = len(sizes), 32
+    N = max(sum(r) for r in sizes)
+    g = torch.Generator().manual_seed(21)
+    assign = torch.empty(P, N, dtype=torch.int32)
+    for p, row in enumerate(sizes):
+        row = row + [0] * (nc - len(row))
+        row[nc - 2] += N - sum(row)                      # the remainder goes to one late cluster
+        ids = torch.repeat_interleave(torch.arange(nc, dtype=torch.int32), torch.tensor(row))
+        assign[p] = ids[torch.randperm(N, generator=g)]
+    keys = torch.randn(P, N, 128, generator=g).to(torch.bfloat16)
+    cent = torch.randn(P, nc, 128, generator=g).to(torch.bfloat16)
+    ad, kd, cd = assign.to(dev), keys.to(dev), cent.to(dev).clone()
+    counts = torch.empty(P, nc, dtype=torch.int32, device=dev)
+    offsets = torch.empty(P, nc + 1, dtype=torch.int32, device=dev)
+    members = torch.empty(P, N, dtype=torch.int32, device=dev)
+    kernels.kmeans_build_lists(ad, counts, offsets, members, P, N, nc)
+    kernels.kmeans_update(kd, counts, offsets, members, cd, P, N, nc, 1, N, True)
+    vs = torch.full((P, nc, 128), 7.0, dtype=torch.bfloat16, device=dev)
+    kernels.kmeans_value_sum(kd, counts, offsets, members, vs, P, N, nc)
+    torch.cuda.synchronize()
+    for p in range(P):
+        a = assign[p].numpy().astype(np.int64)
+        s, cnt = okm.cluster_sums(keys[p], a, nc)
+        assert np.array_equal(counts[p].cpu().numpy(), cnt)
+        assert torch.equal(cd[p].cpu(), okm.update(cent[p], s, cnt, True))
+        assert torch.equal(vs[p].cpu(), okm.value_sum(keys[p], a, nc))
+
+
+@pytest.mark.parametrize("P,N,nc,seed", [(3, 1000, 64, 0), (2, 16384, 512, 1), (2, 16385, 512, 2), (5, 37, 32, 3),
+                                         (2, 8192, 512, 4), (1, 4100, 1024, 5), (2, 1023, 96, 6), (1, 1, 32, 7)])
+def test_build_lists_is_a_stable_sort(dev, P, N, nc, seed):
+    """Inverted lists over the sizes on either side of the single-workgroup path (problems of at most
+    16384 tokens with at most 512 clusters) and of the one- and two-pass paths: members are the stable
+    argsort of the assignment, offsets and counts its CSR bounds; some clusters are empty."""
+    from retrievalattention_amd import kernels
+    g = torch.Generator().manual_seed(seed)
+    assign = torch.randint(0, max(nc - 3, 1), (P, N), generator=g, dtype=torch.int32)
+    assign[0, N // 2:] = nc - 1                     # one long run, and the highest id in use
+    ad = assign.to(dev)
+    counts = torch.full((P, nc), -1, dtype=torch.int32, device=dev)
+    offsets = torch.full((P, nc + 1), -1, dtype=torch.int32, device=dev)
+    members = torch.full((P, N), -1, dtype=torch.int32, device=dev)
+    kernels.kmeans_build_lists(ad, counts, offsets, members, P, N, nc)
+    torch.cuda.synchronize()
+    for p in range(P):
+        a = assign[p].numpy()
+        cnt = np.bincount(a, minlength=nc)
+        assert np.array_equal(members[p].cpu().numpy(), np.argsort(a, kind="stable"))
+        assert np.array_equal(counts[p].cpu().numpy(), cnt)
+        assert np.array_equal(offsets[p].cpu().numpy(), np.concatenate([[0], np.cumsum(cnt)]))
+
+
 @pytest.mark.parametrize("G,N,nc,S,seed", [(2, 4096, 256, 4, 0), (1, 8192, 512, 1, 1), (2, 3001, 192, 3, 2)])
 def test_segment_k_means_teacher_forced(dev, G, N, nc, S, seed):
     """Whole driver against the oracle, iteration by iteration: every step is checked on the
