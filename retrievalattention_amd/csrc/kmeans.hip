@@ -159,10 +159,6 @@ __global__ __launch_bounds__(KM_WAVES * 64) void km_assign_kernel(const uint16_t
 // ------------------------------------------------------------------------------------
 // inverted lists
 // ------------------------------------------------------------------------------------
-__global__ void km_zero_kernel(int32_t* a, size_t n) {
-  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) a[i] = 0;
-}
-
 // Inverted lists are a stable sort of the token ids by cluster id: one or two least-significant-
 // digit counting passes of at most 9 bits.  A pass is three launches: per-chunk digit histograms
 // (one wave per chunk of KM_SORT_CHUNK tokens, wave-private LDS counters), an exclusive scan of
