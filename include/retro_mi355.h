@@ -354,6 +354,11 @@ typedef struct ri_wavebuf ri_wavebuf;
 
 /* Replaces ThreadPool / MyThreadPool (wave_buffer_cpu.cpp:17-35, thread_pool.hpp:27-141). */
 ri_threadpool* ri_threadpool_create(int num_threads);
+/* The same pool with worker i bound to core first_core + i, as set_affinity does for core i
+ * (thread_pool.hpp:18-23, 65-66).  A worker whose core the process may not use stays unbound;
+ * ri_threadpool_pinned_workers tells how many were bound.  NULL for first_core < 0. */
+ri_threadpool* ri_threadpool_create_pinned(int num_threads, int first_core);
+int ri_threadpool_pinned_workers(const ri_threadpool* pool);
 void ri_threadpool_destroy(ri_threadpool* pool);
 
 /* Replaces WaveBufferCPU (wave_buffer_cpu.cpp:328-383 ctor; pybind surface :822-849). */

@@ -41,6 +41,8 @@ SIGNATURES = {
     "ri_kmeans_value_sum": (I, [P, P, P, P, P, I, I, I, P, SZ, P]),
     "ri_permute_rows": (I, [P, P, P, I, I, I64, I64, P]),
     "ri_threadpool_create": (P, [I]),
+    "ri_threadpool_create_pinned": (P, [I, I]),
+    "ri_threadpool_pinned_workers": (I, [P]),
     "ri_threadpool_destroy": (None, [P]),
     "ri_wavebuf_create": (P, [I] * 10 + [P]),
     "ri_wavebuf_destroy": (None, [P]),

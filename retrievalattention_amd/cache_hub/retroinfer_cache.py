@@ -38,7 +38,8 @@ class retroinfer_cache(KV_Cache):
                  head_dim, dtype, layer_mapping, max_new_length, static_pattern_start, static_pattern_end, core,
                  n_centroids, n_segment, nprobe, max_compute_cluster_num, cache_unit_size, cache_cluster_num,
                  num_gpus, model_size, use_cluster_estimation=False, kv_residency="auto",
-                 block_cache="device", device_positions=False, overlap_miss_staging=False):
+                 block_cache="device", device_positions=False, overlap_miss_staging=False, pin_workers=False,
+                 profiler_ranges=False):
         super().__init__(layer_num, batch_size, max_length, num_key_value_heads, num_heads, head_dim, dtype,
                          layer_mapping, num_gpus, model_size)
         if head_dim != 128 or dtype != torch.bfloat16:
@@ -67,6 +68,11 @@ class retroinfer_cache(KV_Cache):
         # more than the overlap returns (measured at B=8, 8 KV heads, 120K tokens: 287 vs 270 us per
         # layer-step at 70 % hits, 93 vs 66 us with every block a hit)
         self.overlap_miss_staging = bool(overlap_miss_staging)
+        # the reference's NVTX ranges (retroinfer_cache.py:558-678) as roctx ranges of the same names
+        self.profiler_ranges = bool(profiler_ranges)
+        self.pin_workers = bool(pin_workers)
+        if self.profiler_ranges:
+            kernels.PROFILER_RANGES = True
 
         self.input_length = self.max_length - max_new_length
         self.max_new_length = min(max_new_length - 1, THRESHOLD_LENGTH)  # one token comes out of prefill
@@ -159,7 +165,9 @@ class retroinfer_cache(KV_Cache):
         zeros = lambda shape, dt, d: torch.zeros(shape, dtype=dt, device=d)
         BG, D = self.batch_groups, self.head_dim
         L = range(self.layer_num)
-        self.thread_pool = kernels.ThreadPool(self.core)
+        # pin_workers: worker i on core i like the reference's pool (thread_pool.hpp:65-66); off by default,
+        # because cores 0..n-1 are also where the interpreter's own thread usually runs
+        self.thread_pool = kernels.ThreadPool(self.core, 0 if self.pin_workers else None)
         pool = self.thread_pool.get()
         self.wave_buffer = [kernels.WaveBufferCPU(
             self.batch_size, self.kv_head, D, self.nprobe, self.page_size, self.n_centroids,
@@ -503,7 +511,11 @@ class retroinfer_cache(KV_Cache):
         queries [batch, 1, heads, dim] on the device; returns the same shape."""
         last = layer_idx == self.layer_num - 1
         static_len = self.static_pattern_total if last else self.static_pattern_total + 1
+        if self.profiler_ranges:
+            torch.cuda.nvtx.range_push("kv_cache_compute")
         out = self._compute(queries, layer_idx, queries_next, static_len)
+        if self.profiler_ranges:
+            torch.cuda.nvtx.range_pop()
         if last and self.device_positions:   # the token is done: its row now belongs to the steady zone
             self.steady_len_dev.add_(1)
             self.steady_pos_dev.add_(1)

@@ -5,6 +5,8 @@
 // thread_pool.hpp; the data structures are this library's own: the LRU order is an
 // index-linked list over cluster ids and free blocks are a stack, which makes the block ids
 // handed out deterministic.
+#include <sched.h>
+
 #include <atomic>
 #include <condition_variable>
 #include <cstdint>
@@ -21,11 +23,25 @@ namespace {
 
 class WorkerPool {
  public:
-  explicit WorkerPool(int n) {
+  // first_core >= 0: worker i runs on core first_core + i only (thread_pool.hpp:18-23, 65-66 pins worker i
+  // to core i); a core the process may not use leaves that worker unpinned
+  explicit WorkerPool(int n, int first_core = -1) {
     if (n <= 0) n = (int)std::thread::hardware_concurrency();
     if (n <= 0) n = 1;
-    for (int i = 0; i < n; ++i) workers_.emplace_back([this] { loop(); });
+    for (int i = 0; i < n; ++i)
+      workers_.emplace_back([this, i, first_core] {
+        if (first_core >= 0) {
+          cpu_set_t set;
+          CPU_ZERO(&set);
+          CPU_SET((first_core + i) % CPU_SETSIZE, &set);
+          if (sched_setaffinity(0, sizeof(set), &set) == 0) pinned_.fetch_add(1);
+        }
+        ready_.fetch_add(1);
+        loop();
+      });
+    while (ready_.load() < n) std::this_thread::yield();
   }
+  int pinned() const { return pinned_.load(); }
   ~WorkerPool() {
     {
       std::lock_guard<std::mutex> lk(mu_);
@@ -50,6 +66,7 @@ class WorkerPool {
   int size() const { return (int)workers_.size(); }
 
  private:
+  std::atomic<int> pinned_{0}, ready_{0};
   void loop() {
     for (;;) {
       std::function<void()> job;
@@ -147,7 +164,7 @@ struct GroupCache {
 
 struct ri_threadpool {
   WorkerPool pool;
-  explicit ri_threadpool(int n) : pool(n) {}
+  explicit ri_threadpool(int n, int first_core = -1) : pool(n, first_core) {}
 };
 
 struct ri_wavebuf {
@@ -278,6 +295,11 @@ struct ri_wavebuf {
 extern "C" {
 
 ri_threadpool* ri_threadpool_create(int num_threads) { return new ri_threadpool(num_threads); }
+ri_threadpool* ri_threadpool_create_pinned(int num_threads, int first_core) {
+  if (first_core < 0) return nullptr;
+  return new ri_threadpool(num_threads, first_core);
+}
+int ri_threadpool_pinned_workers(const ri_threadpool* pool) { return pool ? pool->pool.pinned() : 0; }
 void ri_threadpool_destroy(ri_threadpool* pool) { delete pool; }
 
 ri_wavebuf* ri_wavebuf_create(int batch_size, int group_num, int dim, int nprobe, int block_size,

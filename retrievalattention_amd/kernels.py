@@ -5,6 +5,7 @@ against the reference runs unchanged; the second block exposes the fused MI355X 
 
 Tensors only provide memory and the current stream; all arithmetic happens in the library.
 """
+import functools
 import math
 
 import torch
@@ -12,6 +13,26 @@ import torch
 from ._lib import lib, check
 
 _DT = (torch.bfloat16,)
+
+# Named profiler ranges around the stages of a decode step, with the names the reference gives its NVTX
+# ranges (cache_hub/retroinfer_cache.py:558-678); torch's nvtx calls are roctx ranges on ROCm, so
+# rocprofv3 --marker-trace shows them.  Off unless a cache is built with profiler_ranges=True.
+PROFILER_RANGES = False
+
+
+def _ranged(name):
+    def deco(fn):
+        @functools.wraps(fn)
+        def wrapper(*args, **kwargs):
+            if not PROFILER_RANGES:
+                return fn(*args, **kwargs)
+            torch.cuda.nvtx.range_push(name)
+            try:
+                return fn(*args, **kwargs)
+            finally:
+                torch.cuda.nvtx.range_pop()
+        return wrapper
+    return deco
 
 
 def _stream():
@@ -92,6 +113,7 @@ def gather_copy_vectors(key_data, key_buffer, value_data, value_buffer, src_meta
           "gather_copy_vectors")
 
 
+@_ranged("gather_copy_and_concat")
 def gather_copy_and_concat(key_data1, key_data2, key_data3, key_buffer, value_data1, value_data2, value_data3,
                            value_buffer, data_offsets2, data_copy_sizes2, buffer_offsets2, copy_chunks2,
                            data_offsets3, data_copy_sizes3, buffer_offsets3, copy_chunks3, valid_lengths,
@@ -128,6 +150,7 @@ def gather_copy_and_scatter(key_data, key_buffer, value_data, value_buffer, s_of
           "gather_copy_and_scatter")
 
 
+@_ranged("flash_attention")
 def weighted_flash_decoding(q, k, v, weight=None, previous_out=None, previous_lse=None, cache_seqlens=None,
                             return_softmax_lse=False):
     """Signature of the calls at cache_hub/retroinfer_cache.py:611-617 and :666-674.
@@ -158,13 +181,19 @@ def weighted_flash_decoding(q, k, v, weight=None, previous_out=None, previous_ls
 
 
 class ThreadPool:
-    """wave_buffer_cpu.cpp:17-35."""
+    """wave_buffer_cpu.cpp:17-35.  first_core (None: workers run where the scheduler puts them): worker i is
+    bound to core first_core + i, which is what the reference does with first_core = 0
+    (thread_pool.hpp:18-23, 65-66); pinned_workers tells how many the system accepted."""
 
-    def __init__(self, num_threads):
+    def __init__(self, num_threads, first_core=None):
         self._destroy = lib().ri_threadpool_destroy   # bound now: module globals may be gone at interpreter exit
-        self._h = lib().ri_threadpool_create(int(num_threads))
+        if first_core is None:
+            self._h = lib().ri_threadpool_create(int(num_threads))
+        else:
+            self._h = lib().ri_threadpool_create_pinned(int(num_threads), int(first_core))
         if not self._h:
             raise RuntimeError("ri_threadpool_create failed")
+        self.pinned_workers = lib().ri_threadpool_pinned_workers(self._h)
 
     def get(self):
         return self
@@ -242,6 +271,7 @@ class WaveBufferCPU:
 # ----------------------------------------------------------------------------------------
 # fused MI355X entry points
 # ----------------------------------------------------------------------------------------
+@_ranged("search_topk_clusters")
 def score_select(q, centroids, mask, cluster_size_i32, cluster_start, logits, dist, cI, ret_ids, est_ids,
                  ret_tok_off, row_src, meta, nprobe, es, page, max_pages, scale, slot=0, ret_start=None):
     """Centroid scoring + retrieval/estimation selection + token layout.  `slot` names the
@@ -268,6 +298,7 @@ def score_logits(q, centroids, logits, scale, slot=0):
                                 _stream()), "score_logits")
 
 
+@_ranged("flash_attention")
 def wave_attention(q, steady_k, steady_v, static_len, store_k, store_v, row_src, meta, est_ids, logits,
                    value_sum, cluster_size_bf16, out, valid_lengths, es, scale, slot=0, ret_tok_off=None,
                    ret_start=None, est_centroids=None, static_len_dev=None):
@@ -292,6 +323,7 @@ def wave_attention(q, steady_k, steady_v, static_len, store_k, store_v, row_src,
           "wave_attention")
 
 
+@_ranged("flash_attention")
 def wave_attention_part(q, steady_k, steady_v, static_len, store_k, store_v, row_src, src_row_lo, src_row_hi, meta,
                         est_ids, logits, value_sum, cluster_size_bf16, out, lse_out, es, scale, prev_out=None,
                         prev_lse=None, valid_lengths=None, slot=0):
@@ -307,6 +339,7 @@ def wave_attention_part(q, steady_k, steady_v, static_len, store_k, store_v, row
         _p(valid_lengths), BG, gs, nc, es, float(scale), _p(ws), ws.numel(), _stream()), "wave_attention_part")
 
 
+@_ranged("flash_attention")
 def wave_attention_static(q, steady_k, steady_v, static_len, store_k, store_v, row_src, meta, est_ids, logits,
                           value_sum, cluster_size_bf16, out, valid_lengths, es, scale, ret_tok_off=None,
                           ret_start=None, est_centroids=None, static_len_dev=None):

@@ -35,7 +35,9 @@ def _make_cache(dev, residency, layers, B, Hkv, gs, ctx, n_centroids, n_segment,
         n_segment=n_segment, nprobe=nprobe, max_compute_cluster_num=nprobe + es, cache_unit_size=8,
         cache_cluster_num=cache_cluster_num if cache_cluster_num is not None else 3 * nprobe, num_gpus=1,
         model_size=8, use_cluster_estimation=use_cluster_estimation, kv_residency=residency,
-        block_cache=block_cache, device_positions=device_positions, overlap_miss_staging=overlap)
+        block_cache=block_cache, device_positions=device_positions, overlap_miss_staging=overlap,
+        # the options that change no result ride along on two of the modes
+        pin_workers=block_cache == "host", profiler_ranges=overlap)
 
 
 def _prefill(cache, K, V, layers, B):

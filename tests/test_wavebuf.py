@@ -164,6 +164,19 @@ def test_bad_arguments_are_rejected():
         wb.batch_access()
 
 
+def test_pinned_workers():
+    """Worker i bound to core first_core + i (thread_pool.hpp:18-23, 65-66): as many workers report a
+    binding as there are cores the process may use among those asked for; the pool then works as usual."""
+    import os
+    from retrievalattention_amd import kernels
+    allowed = os.sched_getaffinity(0)
+    pool = kernels.ThreadPool(3, first_core=0)
+    assert pool.pinned_workers == len(allowed & {0, 1, 2})
+    assert kernels.ThreadPool(2).pinned_workers == 0
+    wb = kernels.WaveBufferCPU(1, 1, 128, 1, 8, 4, 4, 4, 4, 2, pool.get())
+    del wb, pool
+
+
 def test_device_lru_model_invariants():
     """The policy the device-side manager implements, on its Python restatement: every requested
     cluster is a hit or a miss exactly once (until the buffer cut-off), hit <=> resident, block ids
