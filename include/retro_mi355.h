@@ -70,6 +70,11 @@ int ri_probe_stream_read(const void* buf, size_t bytes, int workgroups, int load
 int ri_batch_gemm_softmax(const void* A, const void* B, void* D, float* Norm, float* Sum,
                           void* Softmax, int batch_count, int m, int n, int k, float alpha,
                           float beta, ri_stream_t stream);
+/* The same operator on IEEE half inputs and outputs (batch_gemm_softmax.cu:185-197 accepts Half as
+ * well as BFloat16): A, B, D and Softmax hold fp16, everything else as above. */
+int ri_batch_gemm_softmax_f16(const void* A, const void* B, void* D, float* Norm, float* Sum,
+                              void* Softmax, int batch_count, int m, int n, int k, float alpha,
+                              float beta, ri_stream_t stream);
 
 /* Fused scoring + selection: replaces the sequence batch_gemm_softmax → torch.sum →
  * masked_fill_ → torch.topk → cluster_ids.copy_ (cache_hub/retroinfer_cache.py:569-575).

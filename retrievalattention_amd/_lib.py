@@ -18,6 +18,7 @@ SIGNATURES = {
     "ri_null_launch": (I, [P]),
     "ri_probe_stream_read": (I, [P, SZ, I, I, P, P]),
     "ri_batch_gemm_softmax": (I, [P, P, P, P, P, P, I, I, I, I, F, F, P]),
+    "ri_batch_gemm_softmax_f16": (I, [P, P, P, P, P, P, I, I, I, I, F, F, P]),
     "ri_score_select_workspace_bytes": (SZ, [I, I, I]),
     "ri_score_select": (I, [P] * 13 + [I, P, I, I, I, I, I, I, I, F, P, SZ, P]),
     "ri_score_logits": (I, [P, P, P, I, I, I, F, P, SZ, P]),

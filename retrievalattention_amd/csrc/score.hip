@@ -15,7 +15,23 @@
 // MFMA 16x16x32: A = 16 centroid rows, B = query heads (columns >= gs are zero).
 // Accumulator register i of lane l holds row 4*(l/16)+i, column l%16.
 // ------------------------------------------------------------------------------------
-__global__ __launch_bounds__(256) void score_kernel(
+// HALF: the 16-bit element type of q, cent and the 16-bit logits is IEEE half instead of bfloat16
+// (batch_gemm_softmax.cu:185-197 dispatches on Half and BFloat16).
+typedef _Float16 f16x8_t __attribute__((ext_vector_type(8)));
+
+template <bool HALF>
+__device__ __forceinline__ uint16_t score_f32_to_16(float f) {
+  if (HALF) return __builtin_bit_cast(uint16_t, (_Float16)f);   // round to nearest even
+  return ri_f32_to_bf16(f);
+}
+template <bool HALF>
+__device__ __forceinline__ float score_16_to_f32(uint16_t v) {
+  if (HALF) return (float)__builtin_bit_cast(_Float16, v);
+  return ri_bf16_to_f32(v);
+}
+
+template <bool HALF>
+__device__ __forceinline__ void score_body(
     const uint16_t* __restrict__ q, const uint16_t* __restrict__ cent, float* __restrict__ logits,
     uint16_t* __restrict__ logits_bf16, float* __restrict__ tile_max, float* __restrict__ tile_sum,
     int gs, int nc, int ntiles, float scale) {
@@ -50,8 +66,10 @@ __global__ __launch_bounds__(256) void score_kernel(
     acc[t] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int kk = 0; kk < 4; ++kk)
-      acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ri_as_bf16x8(a[t][kk]), ri_as_bf16x8(bq[kk]),
-                                                       acc[t], 0, 0, 0);
+      acc[t] = HALF ? __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8_t, a[t][kk]),
+                                                             __builtin_bit_cast(f16x8_t, bq[kk]), acc[t], 0, 0, 0)
+                    : __builtin_amdgcn_mfma_f32_16x16x32_bf16(ri_as_bf16x8(a[t][kk]), ri_as_bf16x8(bq[kk]),
+                                                              acc[t], 0, 0, 0);
   }
 
   // scale, and the partial row max over this lane's valid centroids.  The logits are stored at
@@ -103,12 +121,25 @@ __global__ __launch_bounds__(256) void score_kernel(
         *reinterpret_cast<float4*>(logits + o) = make_float4(acc[t][0], acc[t][1], acc[t][2], acc[t][3]);
       if (logits_bf16) {
         uint2 pk;
-        pk.x = (uint32_t)ri_f32_to_bf16(acc[t][0]) | ((uint32_t)ri_f32_to_bf16(acc[t][1]) << 16);
-        pk.y = (uint32_t)ri_f32_to_bf16(acc[t][2]) | ((uint32_t)ri_f32_to_bf16(acc[t][3]) << 16);
+        pk.x = (uint32_t)score_f32_to_16<HALF>(acc[t][0]) | ((uint32_t)score_f32_to_16<HALF>(acc[t][1]) << 16);
+        pk.y = (uint32_t)score_f32_to_16<HALF>(acc[t][2]) | ((uint32_t)score_f32_to_16<HALF>(acc[t][3]) << 16);
         *reinterpret_cast<uint2*>(logits_bf16 + o) = pk;
       }
     }
   }
+}
+
+__global__ __launch_bounds__(256) void score_kernel(
+    const uint16_t* __restrict__ q, const uint16_t* __restrict__ cent, float* __restrict__ logits,
+    uint16_t* __restrict__ logits_bf16, float* __restrict__ tile_max, float* __restrict__ tile_sum,
+    int gs, int nc, int ntiles, float scale) {
+  score_body<false>(q, cent, logits, logits_bf16, tile_max, tile_sum, gs, nc, ntiles, scale);
+}
+
+__global__ __launch_bounds__(256) void score_kernel_f16(
+    const uint16_t* __restrict__ q, const uint16_t* __restrict__ cent, uint16_t* __restrict__ logits_f16,
+    float* __restrict__ tile_max, float* __restrict__ tile_sum, int gs, int nc, int ntiles, float scale) {
+  score_body<true>(q, cent, nullptr, logits_f16, tile_max, tile_sum, gs, nc, ntiles, scale);
 }
 
 // batch_gemm_softmax tail: finals into slot 0 of Norm/Sum, then the bf16 softmax.
@@ -126,6 +157,7 @@ __global__ void softmax_reduce_kernel(float* norm, float* sum, int ntiles, int g
   }
 }
 
+template <bool HALF>
 __global__ __launch_bounds__(256) void softmax_apply_kernel(const uint16_t* __restrict__ d,
                                                             const float* __restrict__ norm,
                                                             const float* __restrict__ sum,
@@ -141,7 +173,7 @@ __global__ __launch_bounds__(256) void softmax_apply_kernel(const uint16_t* __re
                             (uint16_t)(v.y >> 16)};
     uint16_t o[4];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) o[i] = ri_f32_to_bf16(__expf(ri_bf16_to_f32(in[i]) - m) * iz);
+    for (int i = 0; i < 4; ++i) o[i] = score_f32_to_16<HALF>(__expf(score_16_to_f32<HALF>(in[i]) - m) * iz);
     uint2 w;
     w.x = (uint32_t)o[0] | ((uint32_t)o[1] << 16);
     w.y = (uint32_t)o[2] | ((uint32_t)o[3] << 16);
@@ -157,9 +189,10 @@ static int check_score_shape(int BG, int gs, int nc, int k) {
   return RI_OK;
 }
 
-extern "C" int ri_batch_gemm_softmax(const void* A, const void* B, void* D, float* Norm, float* Sum,
-                                     void* Softmax, int batch_count, int m, int n, int k, float alpha,
-                                     float beta, ri_stream_t stream) {
+template <bool HALF>
+static int batch_gemm_softmax_impl(const void* A, const void* B, void* D, float* Norm, float* Sum, void* Softmax,
+                                   int batch_count, int m, int n, int k, float alpha, float beta,
+                                   ri_stream_t stream) {
   if (!A || !B || !D || !Norm || !Sum || !Softmax || beta != 0.f) return RI_ERR_ARG;
   if (ri_any_misaligned16(A, B, D, Softmax)) return RI_ERR_ARG;
   int rc = check_score_shape(batch_count, m, n, k);
@@ -167,18 +200,34 @@ extern "C" int ri_batch_gemm_softmax(const void* A, const void* B, void* D, floa
   hipStream_t s = (hipStream_t)stream;
   const int ntiles = (n + SCORE_TILE - 1) / SCORE_TILE;
   // fp32 logits are not part of this interface: the partial statistics come from the fp32
-  // accumulators inside the kernel, the softmax from the bf16 D, as in the reference.
-  score_kernel<<<dim3(ntiles, batch_count), 256, 0, s>>>((const uint16_t*)A, (const uint16_t*)B, nullptr,
-                                                         (uint16_t*)D, Norm, Sum, m, n, ntiles, alpha);
+  // accumulators inside the kernel, the softmax from the 16-bit D, as in the reference.
+  if (HALF)
+    score_kernel_f16<<<dim3(ntiles, batch_count), 256, 0, s>>>((const uint16_t*)A, (const uint16_t*)B,
+                                                               (uint16_t*)D, Norm, Sum, m, n, ntiles, alpha);
+  else
+    score_kernel<<<dim3(ntiles, batch_count), 256, 0, s>>>((const uint16_t*)A, (const uint16_t*)B, nullptr,
+                                                           (uint16_t*)D, Norm, Sum, m, n, ntiles, alpha);
   RI_HIP_CHECK_LAUNCH();
   softmax_reduce_kernel<<<batch_count, 64 * m, 0, s>>>(Norm, Sum, ntiles, m);
   RI_HIP_CHECK_LAUNCH();
   int bx = (n + 1023) / 1024;
   if (bx > 16) bx = 16;
-  softmax_apply_kernel<<<dim3(bx, m, batch_count), 256, 0, s>>>((const uint16_t*)D, Norm, Sum,
-                                                                (uint16_t*)Softmax, ntiles, m, n);
+  softmax_apply_kernel<HALF><<<dim3(bx, m, batch_count), 256, 0, s>>>((const uint16_t*)D, Norm, Sum,
+                                                                      (uint16_t*)Softmax, ntiles, m, n);
   RI_HIP_CHECK_LAUNCH();
   return RI_OK;
+}
+
+extern "C" int ri_batch_gemm_softmax(const void* A, const void* B, void* D, float* Norm, float* Sum,
+                                     void* Softmax, int batch_count, int m, int n, int k, float alpha,
+                                     float beta, ri_stream_t stream) {
+  return batch_gemm_softmax_impl<false>(A, B, D, Norm, Sum, Softmax, batch_count, m, n, k, alpha, beta, stream);
+}
+
+extern "C" int ri_batch_gemm_softmax_f16(const void* A, const void* B, void* D, float* Norm, float* Sum,
+                                         void* Softmax, int batch_count, int m, int n, int k, float alpha,
+                                         float beta, ri_stream_t stream) {
+  return batch_gemm_softmax_impl<true>(A, B, D, Norm, Sum, Softmax, batch_count, m, n, k, alpha, beta, stream);
 }
 
 

@@ -12,7 +12,9 @@ import torch
 
 from ._lib import lib, check
 
-_DT = (torch.bfloat16,)
+# 16-bit element types of the reference's operators (batch_gemm_softmax.cu:185-197, gather_copy.cu:63-67).
+# The fused decode path and the k-means are bfloat16 only.
+_DT = (torch.bfloat16, torch.float16)
 
 # Named profiler ranges around the stages of a decode step, with the names the reference gives its NVTX
 # ranges (cache_hub/retroinfer_cache.py:558-678); torch's nvtx calls are roctx ranges on ROCm, so
@@ -83,25 +85,28 @@ def _workspace(nbytes, device, tag):
 def batch_gemm_softmax(A, B, D, Norm, Sum, Softmax, batch_count, m, n, k, alpha=1.0, beta=0.0):
     """batch_gemm_softmax.cu:201-209.  A [bc, m, k], B [bc, n, k]; D/Softmax [bc, m, n]."""
     if A.dtype not in _DT:
-        raise RuntimeError("Only BFloat16 is supported by the gfx950 kernels")
+        raise RuntimeError("Only Half and BFloat16 are supported")      # batch_gemm_softmax.cu:196
     for t, nm in ((A, "A"), (B, "B"), (D, "D"), (Softmax, "Softmax")):
-        _need(t, torch.bfloat16, nm)
+        _need(t, A.dtype, nm)
     _need(Norm, torch.float32, "Norm"); _need(Sum, torch.float32, "Sum")
     ntiles = (n + 255) // 256
     if A.numel() < batch_count * m * k or B.numel() < batch_count * n * k or \
             D.numel() < batch_count * m * n or Softmax.numel() < batch_count * m * n or \
             Norm.numel() < batch_count * ntiles * m or Sum.numel() < batch_count * ntiles * m:
         raise ValueError("batch_gemm_softmax: a buffer is smaller than its shape arguments")
-    check(lib().ri_batch_gemm_softmax(_p(A), _p(B), _p(D), _p(Norm), _p(Sum), _p(Softmax), batch_count, m, n, k,
-                                      float(alpha), float(beta), _stream()), "batch_gemm_softmax")
+    fn = lib().ri_batch_gemm_softmax_f16 if A.dtype == torch.float16 else lib().ri_batch_gemm_softmax
+    check(fn(_p(A), _p(B), _p(D), _p(Norm), _p(Sum), _p(Softmax), batch_count, m, n, k, float(alpha), float(beta),
+             _stream()), "batch_gemm_softmax")
 
 
 def gather_copy_vectors(key_data, key_buffer, value_data, value_buffer, src_metadata, dst_metadata,
                         data_offsets, groups, data_length, buffer_length, index_size, copy_start, copy_num):
-    """gather_copy.cu:288-292."""
+    """gather_copy.cu:288-292.  The rows are moved as 16-bit elements: Half or BFloat16 (gather_copy.cu:63-67)."""
+    if key_data.dtype not in _DT:
+        raise RuntimeError("Only Half and BFloat16 are supported")
     for t, nm in ((key_data, "key_data"), (key_buffer, "key_buffer"), (value_data, "value_data"),
                   (value_buffer, "value_buffer"), (src_metadata, "src_metadata"), (dst_metadata, "dst_metadata")):
-        _need(t, torch.bfloat16, nm)
+        _need(t, key_data.dtype, nm)
     _need(data_offsets, torch.int64, "data_offsets")
     if key_data.numel() < groups * data_length * 128 or key_buffer.numel() < groups * buffer_length * 128 or \
             data_offsets.numel() < groups * index_size or src_metadata.numel() < groups * data_length or \

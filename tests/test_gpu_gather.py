@@ -94,7 +94,9 @@ def test_gather_copy_scatter(dev, seed):
     assert torch.equal(kc.cpu(), kc2) and torch.equal(vc.cpu(), vc2)
 
 
-def test_gather_copy_vectors(dev):
+@pytest.mark.parametrize("DT", [torch.bfloat16, torch.float16])
+def test_gather_copy_vectors(dev, DT):
+    """Half and BFloat16, the two element types gather_copy.cu:63-67 accepts."""
     from retrievalattention_amd import kernels
     torch.manual_seed(3)
     groups, n, dim, nprobe, idx_size = 8, 8192, 128, 150, 2048

@@ -54,6 +54,40 @@ def test_batch_gemm_softmax_matches_reference_test(dev):
     assert int(ulp_distance_bf16(S.cpu(), Sg).max()) <= 1
 
 
+def test_batch_gemm_softmax_half(dev):
+    """The operator on IEEE half tensors (batch_gemm_softmax.cu:185-197 accepts Half): the reference's test
+    oracle and tolerance (test_batch_gemm_softmax.py: bmm / sqrt(d) -> softmax, atol 1e-3), and stage by
+    stage: D is the fp16 rounding of the fp32 logits up to accumulation order, the statistics come from the
+    fp32 logits, the softmax from the kernel's own D within one fp16 ulp."""
+    from retrievalattention_amd import kernels
+    BG, gs, n, d = 6, 5, 4104, 128
+    g = torch.Generator().manual_seed(1)
+    q = torch.randn(BG, gs, d, generator=g).to(torch.float16)
+    c = torch.randn(BG, n, d, generator=g).to(torch.float16)
+    nt = (n + 255) // 256
+    D = torch.zeros(BG, gs, n, dtype=torch.float16, device=dev)
+    S = torch.zeros_like(D)
+    norm = torch.zeros(BG, gs, nt, dtype=torch.float32, device=dev)
+    ssum = torch.zeros_like(norm)
+    kernels.batch_gemm_softmax(q.to(dev), c.to(dev), D, norm, ssum, S, BG, gs, n, d, 1 / math.sqrt(d), 0)
+    torch.cuda.synchronize()
+    logits = torch.bmm(q.double(), c.double().transpose(1, 2)) / math.sqrt(d)
+    ref = torch.softmax(logits, dim=-1)
+    assert torch.allclose(S.cpu().double(), ref, atol=1e-3)
+    # D: fp16(fp32 logits); an fp16 ulp at |x| is 2^-10 |x| (2^-24 below the normal range)
+    err = (D.cpu().double() - logits).abs()
+    assert bool((err <= logits.abs() * 2.0 ** -10 + 2.0 ** -24 + 1e-5).all())
+    fm = norm.view(BG, -1)[:, :gs].cpu().double()
+    fi = ssum.view(BG, -1)[:, :gs].cpu().double()
+    assert torch.allclose(fm, logits.max(dim=-1).values, rtol=0, atol=1e-5)
+    assert torch.allclose(fi, 1.0 / torch.exp(logits - logits.max(dim=-1, keepdim=True).values).sum(-1), rtol=1e-5)
+    Sg = torch.exp(D.cpu().double() - fm[..., None]) * fi[..., None]
+    assert bool(((S.cpu().double() - Sg).abs() <= Sg * 2.0 ** -10 + 2.0 ** -24).all())
+    # mixing element types is refused
+    with pytest.raises(TypeError):
+        kernels.batch_gemm_softmax(q.to(dev), c.to(dev).to(torch.bfloat16), D, norm, ssum, S, BG, gs, n, d, 1.0, 0)
+
+
 @pytest.mark.parametrize("BG,gs,nc,nprobe,es,seed", [
     (8, 4, 512, 9, 118, 0),       # config-1 shape
     (4, 4, 8192, 147, 1900, 1),   # config-2 shape, fewer groups
