@@ -134,12 +134,14 @@ def test_benchmark_shape_decode(dev, name):
     assert torch.equal(out3, out2)
 
 
-def test_kmeans_full_size_properties(dev):
+@pytest.mark.parametrize("S", [16, 1])
+def test_kmeans_full_size_properties(dev, S):
     """Prefill clustering at the k-means benchmark shape: 8 heads x 131072 tokens, 8192 centroids,
-    16 segments, 10 iterations, seeded random-token initialisation."""
+    10 iterations, seeded random-token initialisation; with the 16 segments the cache uses, and
+    unsegmented (every iteration scores all 8192 centroids)."""
     from retrievalattention_amd import synth, kernels
     from retrievalattention_amd.cache_hub.kmeans import segment_k_means_csr
-    G, N, nc, S = 8, 131072, 8192, 16
+    G, N, nc = 8, 131072, 8192
     ks, vs = [], []
     for h in range(G):
         k, v, _ = synth.make_group(0, 0, h, N, nc, 4, outliers=False, device=dev)
