@@ -96,6 +96,7 @@ def test_batch_gemm_softmax_half(dev):
     (3, 1, 64, 1, 0, 4),          # smallest: one probe, no estimation zone
     (2, 16, 1000, 20, 980, 5),    # nc not a multiple of 256, zones cover every cluster
     (1, 4, 32768, 300, 3000, 6),  # more clusters than the select kernel stages in LDS
+    (1, 16, 65536, 1023, 20000, 7),  # the largest shape the entry point takes: 65536 clusters, 1023 probes, 16 heads
 ])
 def test_score_select(dev, BG, gs, nc, nprobe, es, seed):
     from retrievalattention_amd import kernels
@@ -158,6 +159,48 @@ def test_score_select(dev, BG, gs, nc, nprobe, es, seed):
         exp_rows = torch.cat([start[gi, c] + torch.arange(int(size[gi, c])) for c in ret[gi, :int(kept[gi])]]
                              + [torch.zeros(0, dtype=torch.int64)])
         assert torch.equal(o["rows"][gi, :exp_rows.numel()].long(), exp_rows.long())
+
+
+@pytest.mark.parametrize("kind", ["all_equal", "mostly_masked", "two_values"])
+def test_score_select_degenerate_scores(dev, kind):
+    """Score distributions that put (nearly) every cluster on one score: identical centroids, 97 % of the
+    clusters masked as empty, two distinct scores.  The zones are then decided by the id order of ties alone and
+    must equal the oracle's selection on the kernel's own scores exactly."""
+    from retrievalattention_amd import kernels
+    BG, gs, nc, nprobe, es = 3, 4, 2048, 37, 480
+    g = torch.Generator().manual_seed(11)
+    q = torch.randn(BG, gs, 128, generator=g).to(torch.bfloat16)
+    base = torch.randn(BG, 1, 128, generator=g)
+    cent = base.expand(BG, nc, 128).clone()
+    mask = torch.zeros(BG, nc, dtype=torch.bool)
+    if kind == "mostly_masked":
+        cent = torch.randn(BG, nc, 128, generator=g)
+        mask = torch.rand(BG, nc, generator=g) < 0.97
+        mask[:, :nprobe + es + 5] = False          # enough live clusters for both zones, at the low ids
+    elif kind == "two_values":
+        cent[:, ::3] = -cent[:, ::3]
+    cent = cent.to(torch.bfloat16)
+    size = torch.randint(1, 20, (BG, nc), generator=g, dtype=torch.int32)
+    size[mask] = 0
+    start = (torch.cumsum(size, 1) - size).to(torch.int32)
+    k2 = nprobe + es
+    logits = torch.empty(BG, gs, nc, dtype=torch.float32, device=dev)
+    dist = torch.empty(BG, nc, dtype=torch.bfloat16, device=dev)
+    cI = torch.empty(BG, k2, dtype=torch.int64, device=dev)
+    ret = torch.empty(BG, nprobe, dtype=torch.int32, device=dev)
+    est = torch.empty(BG, es, dtype=torch.int32, device=dev)
+    off = torch.empty(BG, nprobe + 1, dtype=torch.int32, device=dev)
+    meta = torch.empty(BG, 4, dtype=torch.int32, device=dev)
+    kernels.score_select(q.to(dev), cent.to(dev), mask.to(torch.uint8).to(dev), size.to(dev), start.to(dev), logits,
+                         dist, cI, ret, est, off, None, meta, nprobe, es, 8, 4096, 1 / math.sqrt(128))
+    torch.cuda.synchronize()
+    ret_x, est_x = scoring.select(dist.cpu(), nprobe, es)
+    assert torch.equal(ret.cpu().long(), ret_x) and torch.equal(est.cpu().long(), est_x)
+    if kind == "all_equal":      # every score the same: the zones are the lowest ids
+        assert torch.equal(ret_x, torch.arange(nprobe).expand(BG, nprobe))
+        assert torch.equal(est_x, torch.arange(nprobe, k2).expand(BG, es))
+    kept, offs = scoring.retrieval_layout(ret.cpu().long(), size, 8, 4096)
+    assert torch.equal(meta.cpu()[:, 0].long(), kept) and torch.equal(off.cpu().long(), offs)
 
 
 def test_score_select_page_cutoff(dev):
