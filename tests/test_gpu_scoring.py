@@ -161,6 +161,14 @@ def test_score_select(dev, BG, gs, nc, nprobe, es, seed):
         assert torch.equal(o["rows"][gi, :exp_rows.numel()].long(), exp_rows.long())
 
 
+def test_score_select_many_seeds(dev):
+    """The benchmark shape's selection over 24 more seeds: every check of test_score_select, so the tally
+    printed at the end of the run counts how often a zone boundary is decided by a tie inside the one-ulp band
+    (and that none needs more)."""
+    for seed in range(200, 224):
+        test_score_select(dev, 4, 4, 8192, 147, 1900, seed)
+
+
 @pytest.mark.parametrize("kind", ["all_equal", "mostly_masked", "two_values"])
 def test_score_select_degenerate_scores(dev, kind):
     """Score distributions that put (nearly) every cluster on one score: identical centroids, 97 % of the
