@@ -155,7 +155,9 @@ __device__ __forceinline__ void combine_group(const AttendParams& P, int g, int 
 #define ATT_DESC_MAX 128  // rows of one wave whose descriptors are staged in LDS at a time
 
 // PF = chunks (of 16 rows) in flight per wave: the loads of chunk j+PF are issued before chunk j
-// is computed
+// is computed.  Launched with PF = 1: with eight to twelve waves per compute unit one chunk ahead already
+// keeps the memory system busy, and the deeper pipelines only add registers and ramp (step time at 32 groups
+// of 4 heads: 52.8 us with one chunk ahead, 53.4 with two, 56.0 with three).
 template <int GS_PAD, int PF>
 __global__ __launch_bounds__(256, GS_PAD == 16 ? 1 : 3) void attend_kernel(AttendParams P) {
   constexpr int NH = GS_PAD / 4;
@@ -509,13 +511,18 @@ static int launch_attend(AttendParams& P, int BG, int gs, hipStream_t s) {
   const int S = P.S_kv + P.S_es;
   const dim3 grid(S, BG);
   switch (gs_pad_of(gs)) {
-    case 4: attend_kernel<4, 2><<<grid, 256, 0, s>>>(P); break;
-    case 8: attend_kernel<8, 2><<<grid, 256, 0, s>>>(P); break;
-    default: attend_kernel<16, 2><<<grid, 256, 0, s>>>(P); break;
+    case 4: attend_kernel<4, 1><<<grid, 256, 0, s>>>(P); break;
+    case 8: attend_kernel<8, 1><<<grid, 256, 0, s>>>(P); break;
+    default: attend_kernel<16, 1><<<grid, 256, 0, s>>>(P); break;
   }
   RI_HIP_CHECK_LAUNCH();
   return RI_OK;
 }
+
+// Memory traffic of one estimation row: its value-sum row, the 32-byte sector around its cluster size, and
+// either one 32-byte sector per query head around its logit or, when the scores are computed in the launch,
+// its centroid row.
+static int est_row_bytes(int gs, bool scored_here) { return 256 + 32 + (scored_here ? 256 : 32 * gs); }
 
 // Split plan: about two workgroups per compute unit in total (an even load over the 256 CUs,
 // all resident at once), at least 128 rows per workgroup, the budget shared between the
@@ -523,11 +530,6 @@ static int launch_attend(AttendParams& P, int BG, int gs, hipStream_t s) {
 // against the 512 bytes of a K and a V row (the launch is bound by its traffic: weighing a key/value
 // row twice an estimation row, by its arithmetic, left the estimation workgroups finishing last,
 // 20.2 against 19.5 us at 32 groups of 4 heads and 60.4 against 54.9 us at 64 groups of 8).
-// Memory traffic of one estimation row: its value-sum row, the 32-byte sector around its cluster size, and
-// either one 32-byte sector per query head around its logit or, when the scores are computed in the launch,
-// its centroid row.
-static int est_row_bytes(int gs, bool scored_here) { return 256 + 32 + (scored_here ? 256 : 32 * gs); }
-
 static void plan_splits(int64_t kv_rows, int64_t es_rows, int es_row_bytes, int BG, int* S_kv, int* S_es) {
   // two workgroups per compute unit while the launch is short (latency counts); three once every
   // workgroup has more than 512 rows to stream (throughput counts)
