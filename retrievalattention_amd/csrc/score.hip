@@ -117,8 +117,13 @@ __device__ __forceinline__ void score_body(
     const int cbase = c0 + t * 16 + 4 * h;
     if (r < gs && cbase < nc) {  // nc % 4 == 0, so the four columns are valid together
       const size_t o = ((size_t)g * gs + r) * nc + cbase;
-      if (logits)
-        *reinterpret_cast<float4*>(logits + o) = make_float4(acc[t][0], acc[t][1], acc[t][2], acc[t][3]);
+      if (logits) {
+        // streaming store: the 4 MB of logits leave the cache as they are written instead of waiting, dirty,
+        // for the write-back at the end of the kernel (about 1 us per step at 32 groups of 8192 centroids)
+        typedef float score_f4 __attribute__((ext_vector_type(4)));
+        const score_f4 val = {acc[t][0], acc[t][1], acc[t][2], acc[t][3]};
+        __builtin_nontemporal_store(val, reinterpret_cast<score_f4*>(logits + o));
+      }
       if (logits_bf16) {
         uint2 pk;
         pk.x = (uint32_t)score_f32_to_16<HALF>(acc[t][0]) | ((uint32_t)score_f32_to_16<HALF>(acc[t][1]) << 16);
