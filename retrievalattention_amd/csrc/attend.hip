@@ -152,7 +152,7 @@ __device__ __forceinline__ void combine_group(const AttendParams& P, int g, int 
   if (threadIdx.x == 0 && P.valid_lengths) P.valid_lengths[g] = lenA + lenB;
 }
 
-#define ATT_DESC_MAX 128  // rows of one wave whose descriptors are staged in LDS at a time
+#define ATT_DESC_MAX 64  // rows of one wave whose descriptors are staged in LDS at a time (32 and 128 measured slower)
 
 // PF = chunks (of 16 rows) in flight per wave: the loads of chunk j+PF are issued before chunk j
 // is computed.  Launched with PF = 1: with eight to twelve waves per compute unit one chunk ahead already
