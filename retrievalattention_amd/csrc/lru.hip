@@ -44,33 +44,26 @@ struct LruParams {
   int np, ncl, meta_stride, blk_off_stride, stamp_stride, blk_ids_stride, buffer_size, capacity, block;
 };
 
-// exclusive prefix sums of N values over the 1024 threads; totals in tot
+// exclusive prefix sums of N values over the 1024 threads; totals in tot.  Wave scans on DPP, the sixteen
+// wave totals scanned by the lanes of every wave (one LDS read, one DPP scan, two lane reads).
 template <int N>
 __device__ __forceinline__ void lru_scan(const int (&v)[N], int (&pre)[N], int (&tot)[N], int* sh) {
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   int inc[N];
 #pragma unroll
   for (int k = 0; k < N; ++k) {
-    inc[k] = v[k];
-#pragma unroll
-    for (int d = 1; d < 64; d <<= 1) {
-      const int o = __shfl_up(inc[k], d);
-      if (lane >= d) inc[k] += o;
-    }
+    inc[k] = (int)ri_wave_incl_scan((uint32_t)v[k]);
     if (lane == 63) sh[k * LRU_WAVES + wave] = inc[k];
   }
   __syncthreads();
+  const int wv = __builtin_amdgcn_readfirstlane(wave);
 #pragma unroll
   for (int k = 0; k < N; ++k) {
-    int woff = 0, t = 0;
-#pragma unroll
-    for (int w = 0; w < LRU_WAVES; ++w) {
-      const int x = sh[k * LRU_WAVES + w];
-      if (w < wave) woff += x;
-      t += x;
-    }
+    const uint32_t x = (lane < LRU_WAVES) ? (uint32_t)sh[k * LRU_WAVES + lane] : 0u;
+    const uint32_t sc = ri_wave_incl_scan(x);
+    tot[k] = __builtin_amdgcn_readlane((int)sc, LRU_WAVES - 1);
+    const int woff = wv > 0 ? __builtin_amdgcn_readlane((int)sc, wv - 1) : 0;
     pre[k] = woff + inc[k] - v[k];
-    tot[k] = t;
   }
   __syncthreads();
 }

@@ -92,3 +92,19 @@ __device__ __forceinline__ void ri_wave_reduce_partials(const float* pm, const f
   *m_out = m;
   *invz_out = 1.0f / z;
 }
+
+// Inclusive prefix sum over the 64 lanes of a wave with DPP row shifts and row broadcasts
+// (no LDS traffic): shifts by 1, 2, 3 build sums of four neighbours, shifts by 4 and 8 finish the
+// 16-lane rows, the two broadcasts carry row totals into the rows behind.
+__device__ __forceinline__ uint32_t ri_wave_incl_scan(uint32_t v) {
+  uint32_t r = v;
+  r += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x111, 0xf, 0xf, true);   // row_shr:1
+  r += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x112, 0xf, 0xf, true);   // row_shr:2
+  r += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x113, 0xf, 0xf, true);   // row_shr:3
+  r += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)r, 0x114, 0xf, 0xe, false);  // row_shr:4, banks 1-3
+  r += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)r, 0x118, 0xf, 0xc, false);  // row_shr:8, banks 2-3
+  r += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)r, 0x142, 0xa, 0xf, false);  // row_bcast:15 -> rows 1, 3
+  r += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)r, 0x143, 0xc, 0xf, false);  // row_bcast:31 -> rows 2, 3
+  return r;
+}
+

@@ -96,21 +96,6 @@ __global__ __launch_bounds__(256) void dist_kernel(const float* __restrict__ log
 // ------------------------------------------------------------------------------------
 // select_kernel helpers
 // ------------------------------------------------------------------------------------
-// Inclusive prefix sum over the 64 lanes of a wave with DPP row shifts and row broadcasts
-// (no LDS traffic): shifts by 1, 2, 3 build sums of four neighbours, shifts by 4 and 8 finish the
-// 16-lane rows, the two broadcasts carry row totals into the rows behind.
-__device__ __forceinline__ uint32_t wave_incl_scan(uint32_t v) {
-  uint32_t r = v;
-  r += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x111, 0xf, 0xf, true);   // row_shr:1
-  r += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x112, 0xf, 0xf, true);   // row_shr:2
-  r += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x113, 0xf, 0xf, true);   // row_shr:3
-  r += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)r, 0x114, 0xf, 0xe, false);  // row_shr:4, banks 1-3
-  r += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)r, 0x118, 0xf, 0xc, false);  // row_shr:8, banks 2-3
-  r += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)r, 0x142, 0xa, 0xf, false);  // row_bcast:15 -> rows 1, 3
-  r += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)r, 0x143, 0xc, 0xf, false);  // row_bcast:31 -> rows 2, 3
-  return r;
-}
-
 // Exclusive prefix sums of N values over the threads of the block with one barrier.
 // sh: N * SEL_WAVES words that no other scan of the same parity is still reading: callers
 // alternate between two buffers.  tot[] receives the block totals.
@@ -121,20 +106,20 @@ __device__ __forceinline__ void block_excl_scan(const uint32_t (&v)[N], uint32_t
   uint32_t inc[N];
 #pragma unroll
   for (int k = 0; k < N; ++k) {
-    inc[k] = wave_incl_scan(v[k]);
+    inc[k] = ri_wave_incl_scan(v[k]);
     if (lane == 63) sh[k * SEL_WAVES + wave] = inc[k];
   }
   __syncthreads();
+  // the sixteen wave totals are scanned by the lanes (one LDS read, one DPP scan, two lane reads) instead of
+  // being walked by every thread: a third of the kernel's vector instructions were that walk, and the kernel
+  // is bound by instruction issue on its one compute unit as much as by latency
+  const int wv = __builtin_amdgcn_readfirstlane(wave);
 #pragma unroll
   for (int k = 0; k < N; ++k) {
-    uint32_t woff = 0, t = 0;
-#pragma unroll
-    for (int w = 0; w < SEL_WAVES; ++w) {
-      const uint32_t x = sh[k * SEL_WAVES + w];
-      if (w < wave) woff += x;
-      t += x;
-    }
-    tot[k] = t;
+    const uint32_t x = (lane < SEL_WAVES) ? sh[k * SEL_WAVES + lane] : 0u;
+    const uint32_t sc = ri_wave_incl_scan(x);
+    tot[k] = (uint32_t)__builtin_amdgcn_readlane((int)sc, SEL_WAVES - 1);
+    const uint32_t woff = wv > 0 ? (uint32_t)__builtin_amdgcn_readlane((int)sc, wv - 1) : 0u;
     pre[k] = woff + inc[k] - v[k];
   }
 }
