@@ -549,8 +549,9 @@ def main():
                          "HIP graph per token) instead of the attention-only layer-step")
     ap.add_argument("--repeats", type=int, default=21,
                     help="repetitions of the timed region of --steps layer-steps; the median is reported")
-    ap.add_argument("--read-probe", action="store_true",
-                    help="also measure what a read-only streaming kernel reaches on this part (ri_probe_stream_read)")
+    ap.add_argument("--no-read-probe", action="store_true",
+                    help="skip the read-only streaming probe (the measured read ceiling of the part, reported as read_probe)")
+    ap.add_argument("--read-probe", action="store_true", help="kept for older command lines: the probe runs by default")
     ap.add_argument("--copy-probe", action="store_true",
                     help="also run 8 device copies of 256 MiB (a known-size kernel to scale rocprofv3 byte counters by)")
     args = ap.parse_args()
@@ -773,7 +774,7 @@ def main():
         result["stages"]["wave_attention"]["us_in_step"] = t_attn_in_step * 1e6
     if est_next:
         result["next_layer_estimation"] = bench_estimate_next(args, cache, queries, outs, L, static_len)
-    if args.read_probe:
+    if not args.no_read_probe:
         result["read_probe"] = read_probe(dev)
     if not args.no_kmeans:
         result["prefill_kmeans"] = bench_kmeans(cfg, dev)
