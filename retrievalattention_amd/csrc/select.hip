@@ -143,6 +143,10 @@ __device__ __forceinline__ uint32_t sel_bin(uint32_t key) {
 // Thread t owns the contiguous id range [t*E, t*E+E) and keeps those keys in registers: ties
 // are ranked by ascending id with plain prefix sums.
 // ------------------------------------------------------------------------------------
+// E8: eights of keys a thread owns (1 up to 8192 clusters, 2 up to 16384, 4 up to 32768, 8 up to 65536): the
+// loops over the owned keys are unrolled E8 times, so the common sizes do not carry (and fetch) the code of
+// sixty-four keys per thread.
+template <int E8>
 __global__ __launch_bounds__(SEL_THREADS) void select_kernel(
     const uint16_t* __restrict__ keys, const int32_t* __restrict__ cluster_size,
     const int32_t* __restrict__ cluster_start, int64_t* __restrict__ cI, int32_t* __restrict__ ret_ids,
@@ -161,12 +165,12 @@ __global__ __launch_bounds__(SEL_THREADS) void select_kernel(
 
   // ---- loads: this thread's keys (registers) ----
   // thread t owns the contiguous id range [t*E, t*E+E), E a multiple of 8 (nc % 8 == 0), E <= 64
-  const int E = (((nc + SEL_THREADS - 1) / SEL_THREADS) + 7) & ~7;
+  const int E = 8 * E8;  // >= ceil(nc / SEL_THREADS), a multiple of 8
   const int cbeg = min(tid * E, nc);
   const int cend = min(cbeg + E, nc);
-  uint4 kreg[8];
+  uint4 kreg[E8];
 #pragma unroll
-  for (int i = 0; i < 8; ++i)
+  for (int i = 0; i < E8; ++i)
     kreg[i] = (cbeg + 8 * i < cend) ? *reinterpret_cast<const uint4*>(keys + (size_t)g * nc + cbeg + 8 * i)
                                      : ri_zero16();
 #pragma unroll
@@ -176,7 +180,7 @@ __global__ __launch_bounds__(SEL_THREADS) void select_kernel(
   // calls f(id, key) for every owned key in ascending id order
   auto for_each_key = [&](auto&& f) {
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
+    for (int i = 0; i < E8; ++i) {
       if (cbeg + 8 * i < cend) {
         const uint32_t w[4] = {kreg[i].x, kreg[i].y, kreg[i].z, kreg[i].w};
 #pragma unroll
@@ -393,11 +397,15 @@ extern "C" int ri_score_select(const void* q, const void* centroids, const uint8
   else
     dist_kernel<16><<<dgrid, 256, 0, s>>>(logits, tmax, tsum, mask, keys, (uint16_t*)dist, gs, nc, ntiles);
   RI_HIP_CHECK_LAUNCH();
-  // all cluster sizes fit in LDS next to the histogram up to 16384 clusters
-  select_kernel<<<BG, SEL_THREADS, 0, s>>>(
-      keys, cluster_size_i32, cluster_start, cI, ret_ids, est_ids, ret_tok_off, ret_start, row_src, row_src_stride, meta,
-      nc,
-      np, es, page, max_pages);
+  const int per_thread = (nc + SEL_THREADS - 1) / SEL_THREADS;
+#define RI_SELECT_LAUNCH(E8)                                                                                          \
+  select_kernel<E8><<<BG, SEL_THREADS, 0, s>>>(keys, cluster_size_i32, cluster_start, cI, ret_ids, est_ids, ret_tok_off, \
+                                               ret_start, row_src, row_src_stride, meta, nc, np, es, page, max_pages)
+  if (per_thread <= 8) RI_SELECT_LAUNCH(1);
+  else if (per_thread <= 16) RI_SELECT_LAUNCH(2);
+  else if (per_thread <= 32) RI_SELECT_LAUNCH(4);
+  else RI_SELECT_LAUNCH(8);
+#undef RI_SELECT_LAUNCH
   RI_HIP_CHECK_LAUNCH();
   return RI_OK;
 }
