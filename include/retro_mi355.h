@@ -183,7 +183,9 @@ int ri_wave_attention(const void* q, const void* steady_k, const void* steady_v,
  * lse_out [BG, gs] fp32 or NULL receives this part's log-sum-exp.  static_len = 0 leaves the steady zone
  * out, es = 0 the estimation zone.  Two calls over complementary windows, the second with the first's
  * (out, lse_out) as its previous result, equal one ri_wave_attention up to the bf16 rounding of the
- * intermediate output.  Workspace as for ri_wave_attention. */
+ * intermediate output.  A part that attends nothing (no steady zone, no estimation zone, no row inside the
+ * window) writes zeros and a log-sum-exp of -inf, and such a previous result is ignored by the part that
+ * merges it.  Workspace as for ri_wave_attention. */
 int ri_wave_attention_part(const void* q, const void* steady_k, const void* steady_v,
                            int64_t steady_stride, int static_len, const int32_t* static_len_dev,
                            const void* store_k, const void* store_v, int64_t store_stride,

@@ -120,8 +120,8 @@ __device__ __forceinline__ void combine_group(const AttendParams& P, int g, int 
 #pragma unroll
     for (int o = 32; o > 0; o >>= 1) L += __shfl_xor(L, o);
     float A0 = 0.f, A1 = 0.f;
-    if (P.prev_lse) {
-      const float fp = (pl == -INFINITY) ? 0.f : __expf(pl - M);
+    if (P.prev_lse && pl != -INFINITY) {  // an empty earlier part carries no weight, whatever its output holds
+      const float fp = __expf(pl - M);
       L += fp;
       A0 = fp * __uint_as_float(po << 16);
       A1 = fp * __uint_as_float(po & 0xffff0000u);
@@ -145,7 +145,9 @@ __device__ __forceinline__ void combine_group(const AttendParams& P, int g, int 
         A1 += b2[u].y * fs;
       }
     }
-    const uint32_t o = (uint32_t)ri_f32_to_bf16(A0 / L) | ((uint32_t)ri_f32_to_bf16(A1 / L) << 16);
+    // nothing attended at all (an empty part): zeros and a log-sum-exp of -inf, not 0/0
+    const bool any = L > 0.f;
+    const uint32_t o = (uint32_t)ri_f32_to_bf16(any ? A0 / L : 0.f) | ((uint32_t)ri_f32_to_bf16(any ? A1 / L : 0.f) << 16);
     *reinterpret_cast<uint32_t*>(P.out + ((size_t)g * gs + j) * RI_DIM + 2 * lane) = o;
     if (lane == 0 && P.lse_out) P.lse_out[(size_t)g * gs + j] = M + __logf(L);
   }

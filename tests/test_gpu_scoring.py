@@ -6,7 +6,8 @@ import torch
 
 from oracle import scoring
 from oracle.numerics import bf16_ulp
-from tests.parity import check_zone_sets, check_rank_order, ulp_distance_bf16
+from tests.parity import (bf16_bits_i, check_zone_sets, check_rank_order, flip_slack, score_interval,
+                          ulp_distance_bf16)
 
 pytestmark = pytest.mark.gpu
 
@@ -130,11 +131,15 @@ def test_score_select(dev, BG, gs, nc, nprobe, es, seed):
     x_ref = scoring.logits_fp32(q, cent, scale)
     assert torch.allclose(o["logits"], x_ref, rtol=2e-5, atol=2e-5)
 
-    # (2) score pipeline on the kernel's own logits: <= 1 bf16 ulp from the oracle
+    # (2) score pipeline on the kernel's own logits: inside the interval that a 4e-6 relative tolerance of the
+    # fp32 probabilities leaves open (the oracle's own value wherever no head sits on a bf16 rounding boundary)
     _, _, _, soft = scoring.softmax_from_logits(o["logits"])
     dist_ref = scoring.dist_from_softmax(soft, mask)
     dd = ulp_distance_bf16(o["dist"], dist_ref)
-    assert int(dd.max()) <= 1
+    lo, hi = score_interval(o["logits"], mask)
+    kb = bf16_bits_i(o["dist"])
+    assert bool(((kb >= bf16_bits_i(lo)) & (kb <= bf16_bits_i(hi))).all())
+    assert int(ulp_distance_bf16(lo, hi).max()) <= 2 and int(dd.max()) <= 2
     assert float((dd > 0).float().mean()) < 0.02
 
     # (3) selection is exact on the kernel's own scores (ties by ascending id)
@@ -144,11 +149,14 @@ def test_score_select(dev, BG, gs, nc, nprobe, es, seed):
     assert torch.equal(o["cI"][:, :nprobe], ret_x) and torch.equal(o["cI"][:, nprobe:], est_x)
 
     # (4) end to end against the oracle's scores: identical up to boundary ties
-    _, _, _, soft_o = scoring.softmax_from_logits(x_ref)
-    dist_o = scoring.dist_from_softmax(soft_o, mask)
+    dist_of = lambda x: scoring.dist_from_softmax(scoring.softmax_from_logits(x)[3], mask)
+    dist_o = dist_of(x_ref)
     ret_o, est_o = scoring.select(dist_o, nprobe, es)
-    check_zone_sets(dist_o, ret, est, ret_o, est_o, nprobe, es, band=1.0, label=f"score_select BG{BG} gs{gs} nc{nc}")
-    check_rank_order(dist_o, ret, band=1.0)
+    # the band, plus what a bf16 rounding flip of a logit inside the logits' own tolerance can move a score
+    slack = flip_slack(x_ref, dist_of, delta=2e-5)
+    label = f"score_select BG{BG} gs{gs} nc{nc}"
+    check_zone_sets(dist_o, ret, est, ret_o, est_o, nprobe, es, band=1.0, label=label, slack=slack)
+    check_rank_order(dist_o, ret, band=1.0, slack=slack, label=label)
 
     # (5) token layout of the retrieved clusters
     kept, offs = scoring.retrieval_layout(ret, size, page, max_pages)
@@ -167,6 +175,21 @@ def test_score_select_many_seeds(dev):
     (and that none needs more)."""
     for seed in range(200, 224):
         test_score_select(dev, 4, 4, 8192, 147, 1900, seed)
+
+
+def test_score_select_random_shapes(dev):
+    """Every check of test_score_select over 60 shapes drawn from a fixed seed: 1..5 groups, group sizes 1..16
+    (not only the powers of two the models use), 32..48000 clusters in steps of 8, any retrieval zone up to the
+    1023 the selection supports and any estimation zone, including none."""
+    import random
+    rnd = random.Random(777)
+    for it in range(60):
+        BG = rnd.choice([1, 2, 3, 5])
+        gs = rnd.choice([1, 2, 3, 4, 5, 7, 8, 9, 12, 16])
+        nc = 8 * rnd.randint(4, rnd.choice([64, 600, 3000, 6000]))
+        nprobe = rnd.randint(1, min(1023, max(1, nc // 4)))
+        es = 0 if rnd.random() < 0.2 else rnd.randint(0, nc - nprobe)
+        test_score_select(dev, BG, gs, nc, nprobe, es, 1000 + it)
 
 
 @pytest.mark.parametrize("kind", ["all_equal", "mostly_masked", "two_values"])

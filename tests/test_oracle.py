@@ -41,6 +41,23 @@ def test_softmax_uses_bf16_logits_for_the_final_value():
     assert float(soft[0, 0, 0]) == float(expect)
 
 
+def test_score_interval_brackets_the_oracle_scores():
+    """The interval the GPU score check uses is a float64 restatement with a 4e-6 relative tolerance: the oracle's
+    fp32 pipeline must fall inside it, and the interval must be a single value for nearly every cluster (else it
+    would pin nothing)."""
+    from tests.parity import bf16_bits_i, score_interval, ulp_distance_bf16
+    g = torch.Generator().manual_seed(5)
+    x = torch.randn(3, 4, 6000, generator=g) * 2.0
+    mask = torch.rand(3, 6000, generator=g) < 0.02
+    d = scoring.dist_from_softmax(scoring.softmax_from_logits(x)[3], mask)
+    lo, hi = score_interval(x, mask)
+    b = bf16_bits_i(d)
+    assert bool(((b >= bf16_bits_i(lo)) & (b <= bf16_bits_i(hi))).all())
+    w = ulp_distance_bf16(lo, hi)
+    assert int(w.max()) <= 2 and float((w > 0).float().mean()) < 0.01
+    assert bool((lo[mask] == BF16_MIN).all()) and bool((hi[mask] == BF16_MIN).all())
+
+
 def test_select_agrees_with_torch_topk_and_brute_force():
     """retroinfer_cache.py:572-574.  Values must equal torch.topk's; ids equal a brute-force
     sort by (-score, id)."""
