@@ -197,6 +197,48 @@ def test_host_and_device_residency_agree_and_cache_warms(dev, host_kind):
         assert checked > 0
 
 
+def test_residencies_agree_random_shapes(dev):
+    """The four ways to hold the clustered K/V (device store; host store with the device-side block cache, with and
+    without the cached rows attended beside the miss staging; host store with the worker-thread block cache) on 16
+    shapes drawn from a fixed seed: 1-2 layers, batch 1-3, 1-4 kv heads, group sizes 1-8, 1-4 k-means segments,
+    block caches from exactly one probe list (every step evicts) to ten, repeated and fresh queries.  Selections
+    and valid lengths identical, outputs within tolerance of the device store's."""
+    import random
+    rnd = random.Random(4711)
+    kinds = ["device", "host", "host-overlap", "host-cpu"]
+    for it in range(16):
+        layers, B, Hkv, gs = rnd.choice([1, 2]), rnd.choice([1, 2, 3]), rnd.choice([1, 2, 4]), rnd.choice([1, 2, 4, 7, 8])
+        S = rnd.choice([1, 1, 2, 4])
+        nc = 32 * S * rnd.randint(1, 6)
+        ctx = 68 + S * rnd.randint(max(nc // S, 64), 1200)
+        nprobe = rnd.randint(1, max(1, nc // 6))
+        es = rnd.choice([0, rnd.randint(0, nc - nprobe)])
+        ccn = rnd.choice([nprobe, nprobe + 1, 2 * nprobe, 3 * nprobe, 10 * nprobe])
+        label = (layers, B, Hkv, gs, ctx, nc, S, nprobe, es, ccn)
+        K, V = _gen(layers, B, Hkv, gs, ctx, max(nc // 2, 8), dev, 40 + it)
+        caches = [_make_cache(dev, k, layers, B, Hkv, gs, ctx, nc, S, nprobe, es, cache_cluster_num=ccn) for k in kinds]
+        for c in caches:
+            _prefill(c, K, V, layers, B)
+        g = torch.Generator().manual_seed(it)
+        draw = lambda *shape: torch.randn(*shape, generator=g).to(torch.bfloat16).to(dev)
+        qs = [draw(B, 1, Hkv * gs, 128) for _ in range(3)]
+        for step in range(rnd.randint(2, 6)):
+            for l in range(layers):
+                q = qs[rnd.randrange(3)] if rnd.random() < 0.6 else draw(B, 1, Hkv * gs, 128)
+                kn, vn = draw(B, 1, Hkv, 128), draw(B, 1, Hkv, 128)
+                outs = []
+                for c in caches:
+                    c.decode_update_kv_cache(kn, vn, l)
+                    outs.append(c.compute(q, l).clone())
+                torch.cuda.synchronize()
+                for k, c, o in zip(kinds[1:], caches[1:], outs[1:]):
+                    assert bool(torch.isfinite(o.float()).all()), (label, k, step, l)
+                    _close(o.cpu(), outs[0].cpu())
+                    assert torch.equal(caches[0].cI[l % 2].cpu(), c.cI[l % 2].cpu()), (label, k, step, l)
+                    assert torch.equal(caches[0].valid_lengths[l % 2].cpu(), c.valid_lengths[l % 2].cpu()), (label, k, step, l)
+        del caches
+
+
 @pytest.mark.parametrize("residency", ["device", "host", "host-overlap", "host-cpu"])
 def test_next_layer_cluster_estimation(dev, residency):
     """use_cluster_estimation (reference: retroinfer_cache.py:565, 582-595): layers 0 and 1 choose their
