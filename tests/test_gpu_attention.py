@@ -60,6 +60,33 @@ def test_weighted_flash_decoding(dev, BG, gs, S, weighted, prev, ragged):
     assert torch.allclose(lse.cpu(), rl, atol=2e-3, rtol=1e-4)
 
 
+def test_weighted_flash_decoding_with_an_empty_group(dev):
+    """cache_seqlens = 0 for one group: zeros and a log-sum-exp of -inf without a previous partial, the previous
+    partial itself (rounded to bf16) with one; the other groups are unaffected."""
+    from retrievalattention_amd import kernels
+    BG, gs, S = 3, 4, 700
+    g = torch.Generator().manual_seed(21)
+    q, k, v = _rand((BG, gs, 128), g), _rand((BG, S, 128), g), _rand((BG, S, 128), g)
+    po, pl = _rand((BG, gs, 128), g, 0.3), torch.randn(BG, gs, generator=g) + 6.0
+    sl = torch.tensor([S, 0, 311], dtype=torch.int32)
+    args = (q.view(BG, 1, gs, 128).to(dev), k.view(BG, S, 1, 128).to(dev), v.view(BG, S, 1, 128).to(dev), None)
+    out, lse = kernels.weighted_flash_decoding(*args, cache_seqlens=sl.to(dev), return_softmax_lse=True)
+    out2, lse2 = kernels.weighted_flash_decoding(*args, previous_out=po.view(BG, 1, gs, 128).to(dev),
+                                                 previous_lse=pl.to(dev), cache_seqlens=sl.to(dev),
+                                                 return_softmax_lse=True)
+    torch.cuda.synchronize()
+    out, out2 = out.cpu().view(BG, gs, 128), out2.cpu().view(BG, gs, 128)
+    assert bool((out[1] == 0).all()) and bool((lse.cpu()[1] == float("-inf")).all())
+    assert torch.equal(out2[1], po[1]) and torch.allclose(lse2.cpu()[1], pl[1], atol=1e-5)
+    for b in (0, 2):
+        n = int(sl[b])
+        ro, rl = attention.weighted_flash_decoding(q[b:b + 1], k[b:b + 1, :n], v[b:b + 1, :n])
+        _close(out[b:b + 1], ro)
+        assert torch.allclose(lse.cpu()[b:b + 1], rl, atol=2e-3, rtol=1e-4)
+        ro, rl = attention.weighted_flash_decoding(q[b:b + 1], k[b:b + 1, :n], v[b:b + 1, :n], None, po[b:b + 1], pl[b:b + 1])
+        _close(out2[b:b + 1], ro)
+
+
 def test_closed_form_plain_softmax_attention(dev):
     """w = 1 and no previous partial: ordinary softmax attention (torch SDPA on the CPU)."""
     from retrievalattention_amd import kernels
