@@ -8,17 +8,17 @@ typedef float f32x16_t __attribute__((ext_vector_type(16)));
 typedef __attribute__((address_space(3))) void* km_lds_ptr;
 typedef const __attribute__((address_space(1))) void* km_glb_ptr;
 
-#ifndef KM_CT
-#define KM_CT 128         // centroid rows per LDS tile (32-row MFMA sub-tiles)
-#endif
-#ifndef KM_TT
-#define KM_TT 4           // 32-token MFMA columns per wave, held in registers
-#endif
-#ifndef KM_WAVES
 #define KM_WAVES 4        // waves per workgroup sharing one centroid tile
-#endif
-#define KM_WG_TOKENS (KM_WAVES * 32 * KM_TT)
-static_assert(KM_CT % (4 * KM_WAVES) == 0 && KM_CT % 32 == 0, "a tile is whole 1 KiB wave loads and whole sub-tiles");
+// The assignment kernel comes in two tilings (KM_TT 32-token MFMA columns per wave held in registers,
+// KM_CT centroid rows per LDS tile):
+//   4 x 128  long centroid loops (more than KM_WIDE_MIN_NC centroids per problem): most reuse of every LDS read,
+//            256 VGPRs and 64 KiB of LDS, two workgroups per CU;
+//   2 x 32   short loops (the segmented iterations: 512 centroids per problem): the load of the tokens in
+//            front of the loop is a large part of the kernel, and 126 VGPRs / 16 KiB let four workgroups per
+//            CU overlap one's loads with the others' MFMAs.
+// Measured with 8 x 131072 tokens: 512 centroids per problem 125.6 against 135.4 us, 1024: 228 against 252,
+// 2048: 433 against 457, 4096: 836 against 845, 8192: 1639 against 1611 us.
+#define KM_WIDE_MIN_NC 4096
 
 // 16 bytes per lane from global memory straight into LDS: lane l lands at lds_base + 16 l
 // (lds_base: byte address inside the workgroup's LDS, the same in every lane).  The wait for the
@@ -34,21 +34,24 @@ __device__ __forceinline__ size_t km_row0(int p, int seg, int64_t head_rows, int
 }
 
 // ------------------------------------------------------------------------------------
-// assign: grid (ceil(N / KM_WG_TOKENS), P), KM_WAVES waves; a wave keeps KM_TT columns of 32
+// assign: grid (ceil(N / (KM_WAVES * 32 * KM_TT)), P), KM_WAVES waves; a wave keeps KM_TT columns of 32
 // tokens in registers for the whole kernel (KM_TT independent accumulator chains).  Centroid
 // tiles of KM_CT rows go through two LDS buffers shared by all waves of the workgroup: the next
 // tile is requested from global memory straight into the other buffer (no registers, no LDS
-// stores) before the MFMAs of the current one, one wait and one barrier per tile.  (4 token
-// columns x 4 waves measured fastest on the full-size pass against 2x4, 2x8, 2x12, 3x8, and
-// 128-row tiles against 64 and 256, with clocks warmed up and runs interleaved.)
+// stores) before the MFMAs of the current one, one wait and one barrier per tile.  (On the full-size
+// pass 4 token columns x 4 waves measured fastest against 2x4, 2x8, 2x12, 3x8, and 128-row tiles
+// against 64 and 256, with clocks warmed up and runs interleaved.)
 // MFMA 32x32x16: A = centroid rows, B = token columns; accumulator i of lane l is
 // row (i/4)*8 + (l/32)*4 + i%4, column l%32.  nc is a multiple of 32; the last tile may hold
 // fewer sub-tiles.
 // ------------------------------------------------------------------------------------
+template <int KM_TT, int KM_CT>
 __global__ __launch_bounds__(KM_WAVES * 64) void km_assign_kernel(const uint16_t* __restrict__ data,
                                                                   const uint16_t* __restrict__ cent,
                                                                   int32_t* __restrict__ assign, int N, int nc,
                                                                   int seg, int64_t head_rows) {
+  static_assert(KM_CT % (4 * KM_WAVES) == 0 && KM_CT % 32 == 0, "a tile is whole 1 KiB wave loads and whole sub-tiles");
+  constexpr int KM_WG_TOKENS = KM_WAVES * 32 * KM_TT;
   __shared__ __attribute__((aligned(1024))) uint16_t sh_c[2][KM_CT][RI_DIM];
   const int p = blockIdx.y;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -636,8 +639,15 @@ extern "C" int ri_kmeans_assign(const void* data, const void* centroids, int32_t
                                 int nc, int seg, int64_t head_rows, ri_stream_t stream) {
   int rc = km_assign_args(data, centroids, assign, P, N, nc, seg);
   if (rc) return rc;
-  km_assign_kernel<<<dim3((N + KM_WG_TOKENS - 1) / KM_WG_TOKENS, P), KM_WAVES * 64, 0, (hipStream_t)stream>>>(
-      (const uint16_t*)data, (const uint16_t*)centroids, assign, N, nc, seg, head_rows);
+  if (nc > KM_WIDE_MIN_NC) {
+    constexpr int wg_tokens = KM_WAVES * 32 * 4;
+    km_assign_kernel<4, 128><<<dim3((N + wg_tokens - 1) / wg_tokens, P), KM_WAVES * 64, 0, (hipStream_t)stream>>>(
+        (const uint16_t*)data, (const uint16_t*)centroids, assign, N, nc, seg, head_rows);
+  } else {
+    constexpr int wg_tokens = KM_WAVES * 32 * 2;
+    km_assign_kernel<2, 32><<<dim3((N + wg_tokens - 1) / wg_tokens, P), KM_WAVES * 64, 0, (hipStream_t)stream>>>(
+        (const uint16_t*)data, (const uint16_t*)centroids, assign, N, nc, seg, head_rows);
+  }
   RI_HIP_CHECK_LAUNCH();
   return RI_OK;
 }
