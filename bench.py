@@ -125,7 +125,10 @@ def algorithmic_bytes(cache, cfg, nprobe, es, layer, static_len):
     """HBM bytes one decode layer-step has to touch: centroids once, queries, mask, value-sum rows
     and sizes of the estimation zone, K and V of retrieved + steady tokens once, output."""
     BG, gs, nc, D, e = cfg["B"] * cfg["Hkv"], cfg["gs"], cfg["nc"], 128, 2
-    t_ret = cache.meta[:, 1].sum().item()
+    if getattr(cache, "meta", None) is not None:
+        t_ret = cache.meta[:, 1].sum().item()
+    else:   # worker-thread block cache manager: no device-side layout record, the valid lengths hold the same count
+        t_ret = int((cache.valid_lengths[layer % 2] - static_len).sum().item())
     parts = {
         "centroids": BG * nc * D * e + BG * gs * D * e + BG * nc,
         "estimation": BG * es * (D * e + e),
