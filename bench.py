@@ -464,13 +464,32 @@ def bench_host(args, cfg, cache, queries, L, nprobe, es, static_len):
                 torch.cuda.synchronize()
         torch.cuda.synchronize()
         stage_us = {nm: sum(e[k].elapsed_time(e[k + 1]) for e in ev) * 1e3 / n_k for k, nm in enumerate(names)}
+    elif es > 0:
+        # worker-thread manager: the attention launch over the execution buffer as the last warm step left it
+        # (hits and staged misses assembled behind the steady zone), an event pair around each eager launch
+        from retrievalattention_amd import kernels
+        l, n_k = L - 1, 32
+        buf = l % 2
+        out_tmp = torch.empty((BG, gs, 128), dtype=torch.bfloat16, device=queries[0].device)
+        ev = [[torch.cuda.Event(enable_timing=True) for _ in range(2)] for _ in range(n_k)]
+        for e in ev:
+            e[0].record()
+            kernels.buffer_attention(queries[l].view(BG, gs, 128), cache.execution_buffer_keys[buf],
+                                     cache.execution_buffer_values[buf], cache.valid_lengths[buf], cache.est_ids[buf],
+                                     cache.logits, cache.value_sum[l], cache.cluster_size[l], out_tmp, es,
+                                     cache.RSQRT_DIM)
+            e[1].record()
+        torch.cuda.synchronize()
+        stage_us = {"attention": sum(e[0].elapsed_time(e[1]) for e in ev) * 1e3 / n_k}
     parts, t_ret = algorithmic_bytes(cache, cfg, nprobe, es, (L - 1), static_len)
     attn_bytes = parts["estimation"] + parts["kv"] + parts["out"]
     total_bytes = sum(parts.values())
     roofline = None
     if stage_us is not None:
         t_attn = stage_us["attention"] * 1e-6
-        roofline = {"bound": "hbm", "kernel": "attend_kernel (ri_wave_attention over the block cache, every block a hit)",
+        where = ("ri_wave_attention over the block cache, every block a hit" if cache.block_cache == "device"
+                 else "ri_buffer_attention over the assembled execution buffer")
+        roofline = {"bound": "hbm", "kernel": f"attend_kernel ({where})",
                     "achieved": attn_bytes / t_attn / 1e9, "peak": HBM_PEAK / 1e9, "unit": "GB/s",
                     "frac": attn_bytes / t_attn / HBM_PEAK, "traffic": None,
                     "traffic_source": "no counter run recorded for the host-resident path",
