@@ -12,6 +12,8 @@
 //                  membership with ties resolved by ascending id, rank order of the retrieval
 //                  zone straight from the histogram prefix, and the token layout (page
 //                  cut-off; token prefix and first store row per rank, a row per token on request).
+#include <type_traits>
+
 #include "ri_common.h"
 
 #define SEL_THREADS 1024
@@ -223,16 +225,25 @@ __global__ __launch_bounds__(SEL_THREADS) void select_kernel(
   // ---- one scan ranks everything: ties at T1, ties at T2 and the keys strictly between ----
   // Tied keys are taken in ascending id order: tie rank r at T1 belongs to the retrieval zone
   // while g1 + r < np, then to the estimation zone while g1 + r < k2; at T2 while g2 + r < k2.
-  uint32_t n1 = 0, n2 = 0, nmid = 0;
-  for_each_key([&](int, uint32_t key) {
-    const uint32_t b = sel_bin(key);
-    n1 += (b == B1);
-    n2 += (b == B2 && B2 != B1);
-    nmid += (b < B1 && b > B2);
+  // The owned keys are classified once, without branches, into four bit masks (bit i = owned key i); the
+  // rare cases (keys of the retrieval zone: np of nc; ties at a threshold) are then walked bit by bit.
+  typedef typename std::conditional<(E8 <= 4), uint32_t, uint64_t>::type mask_t;
+  mask_t m_gt1 = 0, m_eq1 = 0, m_gt2 = 0, m_eq2 = 0;
+  for_each_key([&](int c, uint32_t key) {
+    const uint32_t bin = sel_bin(key);
+    const int i = c - cbeg;
+    m_gt1 |= (mask_t)(bin > B1) << i;
+    m_eq1 |= (mask_t)(bin == B1) << i;
+    m_gt2 |= (mask_t)(bin > B2) << i;
+    m_eq2 |= (mask_t)(bin == B2) << i;
   });
-  uint32_t cnt3[3] = {n1, n2, nmid}, pre3[3], tot3[3];
+  if (B2 == B1) m_eq2 = 0;
+  const mask_t m_mid = m_gt2 & ~m_gt1 & ~m_eq1;  // strictly between the thresholds: estimation zone
+  auto popc = [](mask_t m) { return (uint32_t)(sizeof(mask_t) == 8 ? __popcll((unsigned long long)m) : __popc((unsigned)m)); };
+  auto lowest = [](mask_t m) { return sizeof(mask_t) == 8 ? __ffsll((long long)m) - 1 : __ffs((int)m) - 1; };
+  uint32_t cnt3[3] = {popc(m_eq1), popc(m_eq2), popc(m_mid)}, pre3[3], tot3[3];
   block_excl_scan<3>(cnt3, pre3, tot3, sh_scan[1]);
-  uint32_t r1 = pre3[0], r2 = pre3[1];
+  const uint32_t r1 = pre3[0], r2 = pre3[1];
   const uint32_t mid_before = pre3[2];
   const uint32_t lo1 = (uint32_t)np > g1 ? (uint32_t)np - g1 : 0u;   // first tie rank of T1 in the est zone
   const uint32_t hi1r = (uint32_t)k2 > g1 ? (uint32_t)k2 - g1 : 0u;  // one past the last
@@ -241,29 +252,34 @@ __global__ __launch_bounds__(SEL_THREADS) void select_kernel(
   // memory operation of the wave, stores included, so a store issued here would put its round
   // trip on the critical path of each later phase.
   const uint32_t est_first = mid_before + (min(max(r1, lo1), hi1r) - lo1) + min(r2, hi2r);
-  uint64_t est_bits = 0;  // bit i: owned key i is in the estimation zone (E <= 64)
-  for_each_key([&](int c, uint32_t key) {
-    const uint32_t b = sel_bin(key);
-    bool in_ret, in_est;
-    uint32_t slot;
-    if (b == B1) {
-      in_ret = r1 < lo1;
-      in_est = !in_ret && r1 < hi1r;
-      slot = g1 + r1;  // ties enter in id order
-      ++r1;
-    } else if (b == B2) {
-      in_ret = false;
-      in_est = r2 < hi2r;
-      slot = 0;
-      ++r2;
-    } else {
-      in_ret = b > B1;
-      in_est = !in_ret && b > B2;
-      slot = in_ret ? atomicAdd(&hist[b], 1u) : 0u;  // hist[b] = keys above b: ranks of b start there
+  // owned key i (a register half chosen at run time: only the rare walks below need it)
+  auto key_at = [&](int i) {
+    uint32_t w = 0;
+#pragma unroll
+    for (int v = 0; v < E8; ++v) {
+      const uint32_t q[4] = {kreg[v].x, kreg[v].y, kreg[v].z, kreg[v].w};
+#pragma unroll
+      for (int u = 0; u < 4; ++u) w = ((i >> 1) == 4 * v + u) ? q[u] : w;
     }
-    if (in_ret) sh_ret[slot] = (key << 16) | (0xffffu - (uint32_t)c);
-    if (in_est) est_bits |= 1ull << (c - cbeg);
-  });
+    return (i & 1) ? (w >> 16) : (w & 0xffffu);
+  };
+  mask_t est_bits = m_mid;  // bit i: owned key i is in the estimation zone
+  for (mask_t m = m_gt1; m; m &= m - 1) {  // above T1: the ranks of a bin start at hist[bin] = keys above it
+    const int i = lowest(m);
+    const uint32_t key = key_at(i);
+    const uint32_t slot = atomicAdd(&hist[sel_bin(key)], 1u);
+    sh_ret[slot] = (key << 16) | (0xffffu - (uint32_t)(cbeg + i));
+  }
+  {
+    uint32_t rk = r1;  // ties at T1 enter in id order
+    for (mask_t m = m_eq1; m; m &= m - 1, ++rk) {
+      const int i = lowest(m);
+      if (rk < lo1) sh_ret[g1 + rk] = (key_at(i) << 16) | (0xffffu - (uint32_t)(cbeg + i));
+      else if (rk < hi1r) est_bits |= (mask_t)1 << i;
+    }
+    rk = r2;
+    for (mask_t m = m_eq2; m && rk < hi2r; m &= m - 1, ++rk) est_bits |= (mask_t)1 << lowest(m);
+  }
   __syncthreads();
 
   // ---- rank order: sh_ret is ordered by score; order runs of equal scores by ascending id ----
@@ -331,7 +347,7 @@ __global__ __launch_bounds__(SEL_THREADS) void select_kernel(
   {
     uint32_t est_off = est_first;
     for (int i = 0; i < E; ++i) {
-      if ((est_bits >> i) & 1ull) {
+      if ((est_bits >> i) & 1u) {
         est_ids[(size_t)g * es + est_off] = cbeg + i;
         if (cI) cI[(size_t)g * k2 + np + est_off] = cbeg + i;
         ++est_off;

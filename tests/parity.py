@@ -33,7 +33,7 @@ def ulp_distance_bf16(a, b):
 def score_interval(logits, mask=None, rel=4e-6):
     """(lo, hi) bf16 [BG, nc]: the scores bf16(sum_j bf16(p_j)) with every head's probability
     p_j = exp(bf16(x_j) - m_j) / Z_j (evaluated in float64 from fp32 logits [BG, gs, nc]) scaled by
-    (1 - rel) and (1 + rel).  rel covers a fast fp32 exp, the order of the fp32 sum behind Z and a
+    (1 - rel) and (1 + rel), the bf16 probabilities added in fp32 in head order.  rel covers a fast fp32 exp, the order of the fp32 sum behind Z and a
     reciprocal instead of a division (each around 1e-7 .. 1e-6 relative).  Both roundings are monotone,
     so any implementation within that tolerance lands in [lo, hi]; lo == hi for all but the few clusters
     with a head sitting on a rounding boundary."""
@@ -43,7 +43,11 @@ def score_interval(logits, mask=None, rel=4e-6):
     p = torch.exp(logits.to(torch.bfloat16).double() - m) / z
     out = []
     for f in (1.0 - rel, 1.0 + rel):
-        d = (p * f).float().to(torch.bfloat16).double().sum(dim=1).float().to(torch.bfloat16)
+        pb = (p * f).float().to(torch.bfloat16).float()
+        d = torch.zeros_like(pb[:, 0])
+        for j in range(pb.shape[1]):   # fp32 sum in head order: a head of 2^-24 of the sum can decide a tie
+            d = d + pb[:, j]
+        d = d.to(torch.bfloat16)
         if mask is not None:
             d = d.masked_fill(mask.bool(), torch.finfo(torch.bfloat16).min)
         out.append(d)
