@@ -159,6 +159,8 @@ __global__ __launch_bounds__(SEL_THREADS) void select_kernel(
   __shared__ uint32_t sh_sel[4];  // bin of T1, entries above it, bin of T2, entries above it
   __shared__ uint32_t sh_ret[1024];
   __shared__ uint32_t sh_sorted[1024];
+  __shared__ uint32_t sh_size[1024];   // size and first store row of the cluster at each rank
+  __shared__ int32_t sh_start[1024];
   __shared__ uint32_t sh_pages, sh_tret, sh_nkeep;
 
   const int g = blockIdx.x;
@@ -283,14 +285,26 @@ __global__ __launch_bounds__(SEL_THREADS) void select_kernel(
   __syncthreads();
 
   // ---- rank order: sh_ret is ordered by score; order runs of equal scores by ascending id ----
+  // The size and first store row of the entry's cluster are requested before the walk over its run and
+  // travel to the entry's final rank through LDS: their round trip to global memory runs under the walk
+  // instead of after the next barrier.
   for (int r = tid; r < np; r += SEL_THREADS) {
     const uint32_t mine = sh_ret[r];
     const uint32_t kk = mine >> 16;
+    uint32_t sz_e = 0;
+    int32_t st_e = 0;
+    if (cluster_size) {
+      const size_t at = (size_t)g * nc + (0xffffu - (mine & 0xffffu));
+      sz_e = (uint32_t)cluster_size[at];
+      if (cluster_start) st_e = cluster_start[at];
+    }
     int lo = r, rank_in_run = 0;
     while (lo > 0 && (sh_ret[lo - 1] >> 16) == kk) { --lo; rank_in_run += (sh_ret[lo] > mine); }
     int hi = r;
     while (hi + 1 < np && (sh_ret[hi + 1] >> 16) == kk) { ++hi; rank_in_run += (sh_ret[hi] > mine); }
     sh_sorted[lo + rank_in_run] = mine;
+    sh_size[lo + rank_in_run] = sz_e;
+    sh_start[lo + rank_in_run] = st_e;
   }
   __syncthreads();
 
@@ -302,11 +316,9 @@ __global__ __launch_bounds__(SEL_THREADS) void select_kernel(
   int my_c = -1;
   if (r < np) {
     my_c = (int)(0xffffu - (sh_sorted[r] & 0xffffu));
-    if (cluster_size) {
-      if (cluster_start) st = cluster_start[(size_t)g * nc + my_c];
-      sz = (uint32_t)cluster_size[(size_t)g * nc + my_c];
-      pg = (sz + page - 1) / page;
-    }
+    st = sh_start[r];
+    sz = sh_size[r];
+    pg = (sz + page - 1) / page;
   }
   bool keep = false;
   uint32_t tok_run = 0;
@@ -322,12 +334,7 @@ __global__ __launch_bounds__(SEL_THREADS) void select_kernel(
     keep = r < np && pg_run + pg <= (uint32_t)max_pages;
     // the kept clusters are the ranks 0 .. nkeep-1: the last of them publishes the totals
     if (keep) {
-      bool next_keep = false;
-      if (r + 1 < np) {
-        const int nc_ = (int)(0xffffu - (sh_sorted[r + 1] & 0xffffu));
-        const uint32_t sz_n = (uint32_t)cluster_size[(size_t)g * nc + nc_];
-        next_keep = pg_run + pg + (sz_n + page - 1) / page <= (uint32_t)max_pages;
-      }
+      const bool next_keep = r + 1 < np && pg_run + pg + (sh_size[r + 1] + page - 1) / page <= (uint32_t)max_pages;
       if (!next_keep) {
         sh_pages = pg_run + pg;
         sh_tret = tok_run + sz;
