@@ -87,13 +87,18 @@ __global__ __launch_bounds__(LRU_THREADS) void lru_kernel(LruParams P) {
   const int F0 = P.free_count[g];
 
   // ---- access: thread r looks at the cluster of rank r ----
-  int c = -1, nb = 0, sz = 0;
+  // (everything the rank needs to know about its cluster is requested in one go: loads issued after a
+  // barrier would each put another round trip to global memory on the kernel's critical path)
+  int c = -1, nb = 0, sz = 0, stamp_c = 0, boff_c = 0, start_c = 0;
   if (tid < P.np) {
     c = P.ret_ids[(size_t)g * P.np + tid];
     if (c < 0 || c >= P.ncl) {
       c = -1;
     } else {
       sz = sizes[c];
+      stamp_c = stamp[c];
+      boff_c = boff[c];
+      start_c = starts[c];
       nb = (sz + block - 1) / block;
     }
   }
@@ -101,7 +106,7 @@ __global__ __launch_bounds__(LRU_THREADS) void lru_kernel(LruParams P) {
   lru_scan<1>(v1, p1, t1, sh_scan);
   // the walk stops at the first cluster whose blocks no longer fit: everything after it is dropped
   const bool keep = c >= 0 && nb > 0 && p1[0] + nb <= P.buffer_size;
-  const bool hit = keep && stamp[c] != 0;
+  const bool hit = keep && stamp_c != 0;
   const bool miss = keep && !hit;
   int v4[4] = {hit ? nb : 0, keep ? sz : 0, miss ? nb : 0, miss ? sz : 0}, p4[4], t4[4];
   lru_scan<4>(v4, p4, t4, sh_scan);
@@ -124,7 +129,7 @@ __global__ __launch_bounds__(LRU_THREADS) void lru_kernel(LruParams P) {
     // row table: every thread takes tokens t, t + 1024, ... and finds the rank that owns them by
     // bisection over the token offsets of the ranks (clusters that were dropped have no tokens)
     sh_off[tid] = p4[1];
-    sh_src[tid] = hit ? -(boff[c] + 1) : P.stage_row0 + p4[3];  // hits: where their block ids are
+    sh_src[tid] = hit ? -(boff_c + 1) : P.stage_row0 + p4[3];  // hits: where their block ids are
     __syncthreads();
     int32_t* table = P.row_src + (size_t)g * P.row_src_stride;
     for (int t = tid; t < t4[1]; t += LRU_THREADS) {
@@ -138,7 +143,7 @@ __global__ __launch_bounds__(LRU_THREADS) void lru_kernel(LruParams P) {
     }
   }
   if (hit) {
-    const int32_t* ids = bids + boff[c];
+    const int32_t* ids = bids + boff_c;
     if (!rows) {
       for (int j = 0; j < nb; ++j) {
         P.hit_ids[lo + p4[0] + j] = ids[j];
@@ -149,7 +154,7 @@ __global__ __launch_bounds__(LRU_THREADS) void lru_kernel(LruParams P) {
     stamp[c] = E;
   }
   if (miss) {
-    const int row = starts[c];
+    const int row = start_c;
     for (int j = 0; j < nb; ++j) {
       P.miss_ids[lo + p4[2] + j] = row + j * block;
       P.miss_sizes[lo + p4[2] + j] = (j == nb - 1) ? sz - (nb - 1) * block : block;
@@ -238,7 +243,7 @@ __global__ __launch_bounds__(LRU_THREADS) void lru_kernel(LruParams P) {
   int vb[1] = {adm ? nb : 0}, pb[1], tb[1];
   lru_scan<1>(vb, pb, tb, sh_scan);
   if (adm) {
-    int32_t* ids = bids + boff[c];
+    int32_t* ids = bids + boff_c;
     for (int j = 0; j < nb; ++j) {
       const int id = flist[F - 1 - (pa[0] + j)];
       ids[j] = id;
