@@ -243,6 +243,9 @@ class retroinfer_cache(KV_Cache):
         if self.kv_residency != "device" and self.block_cache == "device":
             self._part_out = torch.zeros((BG, gs, D), dtype=self.dtype, device=d0)
             self._part_lse = torch.zeros((BG, gs), dtype=torch.float32, device=d0)
+            # the miss staging reports the rows it assembled; the attention launch writes the real valid lengths,
+            # and the staging may run on the copy stream beside it, so its report goes to a tensor of its own
+            self._staged_rows = i32(BG)
         if self.kv_residency != "device":
             shape = (BG, self.execution_stride, 1, D)
             self.execution_buffer_keys = [torch.zeros(shape, dtype=self.dtype, device=d0) for _ in range(2)]
@@ -576,7 +579,7 @@ class retroinfer_cache(KV_Cache):
             self.steady_zone_values[layer], self.list_values[layer], self.cache_values[layer], stage_v,
             self.miss_unit_idices[layer], self.miss_unit_sizes[layer], self.miss_unit_sizes_cumsum[layer],
             self.miss_num_units[layer], self.hit_unit_idices[layer], self.hit_unit_sizes[layer],
-            self.hit_unit_sizes_cumsum[layer], self.hit_num_units[layer], self.valid_lengths[buf], BG,
+            self.hit_unit_sizes_cumsum[layer], self.hit_num_units[layer], self._staged_rows, BG,
             self.static_stride, self.list_stride, self.cache_stride, rows, self.buffer_size, 0)
         return stage_k, stage_v
 
