@@ -710,8 +710,16 @@ class retroinfer_cache(KV_Cache):
             with torch.cuda.stream(self.copystream):
                 self._assemble(layer_idx + 1, nbuf, static_len)
         if not search_here:
-            # this layer's buffer was assembled on the copy stream during the previous layer
+            # this layer's buffer was assembled on the copy stream during the previous layer, before this
+            # layer's new token was appended to its steady zone (as in the reference, retroinfer_cache.py:644-652
+            # against :541-542, whose attention then sees a stale row there): the token's row is brought in now,
+            # so that every residency attends the same rows
             torch.cuda.current_stream().wait_stream(self.copystream)
+            BGd = (BG, -1, D)
+            self.execution_buffer_keys[buf][:, static_len - 1, 0] = \
+                self.steady_zone_keys[layer_idx].view(BGd)[:, static_len - 1]
+            self.execution_buffer_values[buf][:, static_len - 1, 0] = \
+                self.steady_zone_values[layer_idx].view(BGd)[:, static_len - 1]
         if fuse_est:
             attn = torch.empty((BG, gs, D), dtype=self.dtype, device=queries.device)
             kernels.buffer_attention(

@@ -239,6 +239,50 @@ def test_residencies_agree_random_shapes(dev):
         del caches
 
 
+def test_residencies_agree_with_cluster_estimation_random_shapes(dev):
+    """use_cluster_estimation through the four residencies on 12 shapes drawn from a fixed seed (3-5 layers, 1-3
+    tokens, short contexts, so that the one new token of a layer carries weight): zones from a predicted query
+    from the third layer on.  Selections and valid lengths identical, outputs within tolerance of the device
+    store's.  (The worker-thread mode assembles a layer's buffer during the previous layer, before the layer's
+    new token exists; the token's row is brought in before the attention.)"""
+    import random
+    rnd = random.Random(77)
+    kinds = ["device", "host", "host-overlap", "host-cpu"]
+    for it in range(12):
+        layers, B, Hkv, gs = rnd.choice([3, 4, 5]), rnd.choice([1, 2, 3]), rnd.choice([1, 2, 4]), rnd.choice([1, 2, 4, 7, 8])
+        S = rnd.choice([1, 1, 2, 4])
+        nc = 32 * S * rnd.randint(1, 6)
+        ctx = 68 + S * rnd.randint(max(nc // S, 64), 1200)
+        nprobe = rnd.randint(1, max(1, nc // 6))
+        es = rnd.choice([0, rnd.randint(0, nc - nprobe)])
+        ccn = rnd.choice([nprobe, 2 * nprobe, 3 * nprobe, 10 * nprobe])
+        tokens = rnd.randint(1, 3)
+        label = (layers, B, Hkv, gs, ctx, nc, S, nprobe, es, ccn, tokens)
+        K, V = _gen(layers, B, Hkv, gs, ctx, max(nc // 2, 8), dev, 140 + it)
+        caches = [_make_cache(dev, k, layers, B, Hkv, gs, ctx, nc, S, nprobe, es, cache_cluster_num=ccn,
+                              use_cluster_estimation=True) for k in kinds]
+        for c in caches:
+            _prefill(c, K, V, layers, B)
+        g = torch.Generator().manual_seed(it)
+        draw = lambda *shape: torch.randn(*shape, generator=g).to(torch.bfloat16).to(dev)
+        for tok in range(tokens):
+            qs = [draw(B, 1, Hkv * gs, 128) for _ in range(layers)]
+            qp = [(q.float() + 0.5 * torch.randn(q.shape, generator=g).to(dev)).to(torch.bfloat16) for q in qs]
+            for l in range(layers):
+                kn, vn = draw(B, 1, Hkv, 128), draw(B, 1, Hkv, 128)
+                outs = []
+                for c in caches:
+                    c.decode_update_kv_cache(kn, vn, l)
+                    outs.append(c.compute(qs[l], l, qp[l + 1] if l + 1 < layers else None).clone())
+                torch.cuda.synchronize()
+                for k, c, o in zip(kinds[1:], caches[1:], outs[1:]):
+                    assert bool(torch.isfinite(o.float()).all()), (label, k, tok, l)
+                    _close(o.cpu(), outs[0].cpu())
+                    assert torch.equal(caches[0].cI[l % 2].cpu(), c.cI[l % 2].cpu()), (label, k, tok, l)
+                    assert torch.equal(caches[0].valid_lengths[l % 2].cpu(), c.valid_lengths[l % 2].cpu()), (label, k, tok, l)
+        del caches
+
+
 @pytest.mark.parametrize("residency", ["device", "host", "host-overlap", "host-cpu"])
 def test_next_layer_cluster_estimation(dev, residency):
     """use_cluster_estimation (reference: retroinfer_cache.py:565, 582-595): layers 0 and 1 choose their
