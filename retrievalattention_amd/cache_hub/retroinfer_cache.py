@@ -15,6 +15,7 @@ Two residencies of the clustered K/V:
 Buffer names follow the reference so that code poking at them keeps working.
 """
 import math
+import warnings
 
 import torch
 
@@ -46,6 +47,22 @@ class retroinfer_cache(KV_Cache):
             raise ValueError("the gfx950 kernels are built for head_dim 128 and bfloat16")
         if cache_unit_size != 8:
             raise ValueError("cache_unit_size must be 8 (block size of the copy kernels)")
+        # limits of the kernels, checked here so that they surface at construction and not at the first decode step
+        n_new = ((max_new_length - 2) // THRESHOLD_LENGTH) * (((THRESHOLD_LENGTH // 16) // 32) * 32)
+        if num_heads % num_key_value_heads != 0 or num_heads // num_key_value_heads > kernels.MAX_GROUP_SIZE:
+            raise ValueError(f"at most {kernels.MAX_GROUP_SIZE} query heads per KV head (got {num_heads} / "
+                             f"{num_key_value_heads})")
+        if not 1 <= nprobe <= kernels.MAX_PROBES:
+            raise ValueError(f"nprobe must be in 1..{kernels.MAX_PROBES} (got {nprobe})")
+        if n_centroids % 8 != 0 or n_centroids + n_new > kernels.MAX_CLUSTERS:
+            raise ValueError(f"n_centroids must be a multiple of 8 and, with the clusters of generated tokens "
+                             f"({n_new}), at most {kernels.MAX_CLUSTERS} (got {n_centroids})")
+        if not nprobe <= max_compute_cluster_num <= n_centroids:
+            raise ValueError(f"max_compute_cluster_num must lie between nprobe ({nprobe}) and n_centroids "
+                             f"({n_centroids}) (got {max_compute_cluster_num})")
+        if cache_cluster_num < 0:
+            raise ValueError("cache_cluster_num must not be negative (0: no block cache, every retrieved cluster "
+                             "is read from the host store)")
         self.valid_start = valid_start
         self.static_pattern_start = static_pattern_start
         self.static_pattern_end = static_pattern_end
@@ -71,8 +88,6 @@ class retroinfer_cache(KV_Cache):
         # the reference's NVTX ranges (retroinfer_cache.py:558-678) as roctx ranges of the same names
         self.profiler_ranges = bool(profiler_ranges)
         self.pin_workers = bool(pin_workers)
-        if self.profiler_ranges:
-            kernels.PROFILER_RANGES = True
 
         self.input_length = self.max_length - max_new_length
         self.max_new_length = min(max_new_length - 1, THRESHOLD_LENGTH)  # one token comes out of prefill
@@ -103,6 +118,10 @@ class retroinfer_cache(KV_Cache):
             store_gib = 2 * layer_num * self.batch_groups * self.list_stride * head_dim * 2 / 1024 ** 3
             kv_residency = "device" if store_gib * 1.25 < self.free_memory else "host"
         self.kv_residency = kv_residency
+        if self.overlap_miss_staging and not (kv_residency == "host" and block_cache == "device"):
+            warnings.warn("overlap_miss_staging only applies to a host-resident store with the device-side block "
+                          "cache manager: ignored")
+            self.overlap_miss_staging = False
         self.allocated = True  # the GPU side is always allocated up front on a 288 GB part
 
         dev = lambda ldx: self.layer_mapping[str(ldx)]
@@ -203,8 +222,9 @@ class retroinfer_cache(KV_Cache):
         # with the device-side manager the staging blocks of the misses sit behind the cache blocks in the
         # same tensor, so that attention can read hits in place and staged misses through one row table
         self.cache_blocks = self.cache_size + (self.buffer_size if self.block_cache == "device" else 0)
-        self.cache_stride = self.cache_blocks
-        self.cache_keys = [torch.zeros((self.batch_size, self.kv_head, self.cache_blocks, self.page_size, D),
+        self.cache_stride = max(self.cache_blocks, 1)
+        # (a cache without blocks still gets one physical block: the copy kernels take a base address)
+        self.cache_keys = [torch.zeros((self.batch_size, self.kv_head, max(self.cache_blocks, 1), self.page_size, D),
                                        dtype=self.dtype, device=dev(l)) for l in L]
         self.cache_values = [torch.zeros_like(self.cache_keys[l]) for l in L]
         n_in = self.input_length - self.static_pattern_total
@@ -272,6 +292,10 @@ class retroinfer_cache(KV_Cache):
         self.clusters_cpu = self.cluster_size_cpu = None
         self.temp_keys = self.temp_values = None
         self._centred_keys.clear()
+        # the clusterings captured during this prefill replay with the addresses of the buffers just dropped
+        # (scratch tensors that were outgrown stay: a decode graph of another cache may still replay with them)
+        if not torch.cuda.is_current_stream_capturing():
+            kernels.release_cached_graphs(retired_workspaces=False)
 
     # ------------------------------------------------------------------ prefill
     def prefill_update_kv_cache(self, query_states, key_states, value_states, layer_idx, batch_idx):
@@ -515,10 +539,14 @@ class retroinfer_cache(KV_Cache):
         last = layer_idx == self.layer_num - 1
         static_len = self.static_pattern_total if last else self.static_pattern_total + 1
         if self.profiler_ranges:
-            torch.cuda.nvtx.range_push("kv_cache_compute")
-        out = self._compute(queries, layer_idx, queries_next, static_len)
-        if self.profiler_ranges:
-            torch.cuda.nvtx.range_pop()
+            with kernels.profiler_ranges(True):
+                torch.cuda.nvtx.range_push("kv_cache_compute")
+                try:
+                    out = self._compute(queries, layer_idx, queries_next, static_len)
+                finally:
+                    torch.cuda.nvtx.range_pop()
+        else:
+            out = self._compute(queries, layer_idx, queries_next, static_len)
         if last and self.device_positions:   # the token is done: its row now belongs to the steady zone
             self.steady_len_dev.add_(1)
             self.steady_pos_dev.add_(1)

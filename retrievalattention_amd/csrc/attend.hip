@@ -91,13 +91,13 @@ __device__ __forceinline__ void wave_rows(int total, int nwaves, int wid, int* r
 }
 
 // Merges the S split partials of group g (and the optional previous result) and writes the
-// output: wave w of the calling workgroup takes heads w, w+4, ...; lanes first cover the splits
+// output: wave w of the calling workgroup takes heads w, w+NW, ...; lanes first cover the splits
 // (statistics), then two dims each.
-template <int GS_PAD>
+template <int GS_PAD, int NW>
 __device__ __forceinline__ void combine_group(const AttendParams& P, int g, int S, int lenA, int lenB) {
   const int gs = P.gs;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  for (int j = wave; j < gs; j += 4) {
+  for (int j = wave; j < gs; j += NW) {
     const float* ml = P.part_ml + ((size_t)g * S * GS_PAD + j) * 2;
     const float* pa = P.part_acc + ((size_t)g * S * GS_PAD + j) * RI_DIM + 2 * lane;
     // every load of the merge is issued up front: the statistics (one split per lane) and the
@@ -160,20 +160,29 @@ __device__ __forceinline__ void combine_group(const AttendParams& P, int g, int 
 // is computed.  Launched with PF = 1: with eight to twelve waves per compute unit one chunk ahead already
 // keeps the memory system busy, and the deeper pipelines only add registers and ramp (step time at 32 groups
 // of 4 heads: 52.8 us with one chunk ahead, 53.4 with two, 56.0 with three).
-template <int GS_PAD, int PF>
-__global__ __launch_bounds__(256, GS_PAD == 16 ? 1 : 3) void attend_kernel(AttendParams P) {
+//
+// NW = waves per workgroup (4 or 8).  The waves of a workgroup merge in LDS, so a group split over S workgroups
+// hands S partials to its last arriver whatever NW is: eight-wave workgroups halve the partials (and the
+// arrivals) of a launch with the same number of waves per compute unit.
+// The rank tables of the retrieval zone (np + 1 token offsets, np first rows) live in dynamic LDS, sized by
+// the launch, so that any number of probes the selection accepts can be attended.
+template <int GS_PAD, int NW, int PF>
+__global__ __launch_bounds__(64 * NW, GS_PAD == 16 ? 1 : 3) void attend_kernel(AttendParams P) {
   constexpr int NH = GS_PAD / 4;
-  __shared__ __attribute__((aligned(16))) uint16_t sh_vt[4][16 * ATT_VT_STRIDE];
-  __shared__ __attribute__((aligned(16))) uint16_t sh_pb[4][16 * 16];
-  __shared__ float sh_al[4][16];
-  __shared__ float sh_m[4][GS_PAD];
-  __shared__ float sh_l[4][GS_PAD];
-  __shared__ float sh_acc[4][GS_PAD][RI_DIM];
+  constexpr int NT = 64 * NW;
+  __shared__ __attribute__((aligned(16))) uint16_t sh_vt[NW][16 * ATT_VT_STRIDE];
+  __shared__ __attribute__((aligned(16))) uint16_t sh_pb[NW][16 * 16];
+  __shared__ float sh_al[NW][16];
+  __shared__ float sh_m[NW][GS_PAD];
+  __shared__ float sh_l[NW][GS_PAD];
+  __shared__ float sh_acc[NW][GS_PAD][RI_DIM];
   __shared__ __attribute__((aligned(16))) uint16_t sh_q[GS_PAD][RI_DIM];
-  __shared__ int sh_desc[4][ATT_DESC_MAX];
-  __shared__ float sh_w[4][ATT_DESC_MAX];
+  __shared__ int sh_desc[NW][ATT_DESC_MAX];
+  __shared__ float sh_w[NW][ATT_DESC_MAX];
   __shared__ int sh_last;
-  __shared__ int sh_roff[1025], sh_rst[1024];
+  extern __shared__ __attribute__((aligned(16))) int sh_tab[];
+  int* const sh_roff = sh_tab;              // [np + 1]
+  int* const sh_rst = sh_tab + P.np + 1;    // [np]
 
   const int g = blockIdx.y;
   const int split = blockIdx.x;
@@ -207,30 +216,39 @@ __global__ __launch_bounds__(256, GS_PAD == 16 ? 1 : 3) void attend_kernel(Atten
     // rank tables (requested together with everything else the prologue loads: no dependent round trip)
     const bool tab = !est_split && P.ret_off != nullptr;
     // every global load of the prologue is requested before the first of them is consumed
-    int t_off[4], t_st[4];
-    if (tab) {
+    // (up to 1023 probes the table entries pass through registers, TAB_U per thread; longer tables are
+    // staged by a plain loop after the query)
+    constexpr int TAB_U = 1024 / NT;
+    const bool tab_fast = tab && P.np < 1024;
+    int t_off[TAB_U], t_st[TAB_U];
+    if (tab_fast) {
 #pragma unroll
-      for (int u = 0; u < 4; ++u) {
-        const int i = threadIdx.x + u * 256;
+      for (int u = 0; u < TAB_U; ++u) {
+        const int i = threadIdx.x + u * NT;
         t_off[u] = (i <= P.np) ? P.ret_off[(size_t)g * (P.np + 1) + i] : 0;
         t_st[u] = (i < P.np) ? P.ret_start[(size_t)g * P.np + i] : 0;
       }
     }
     // A operand: query heads through LDS (read again per chunk: registers go to the loads);
     // row m of the MFMA holds head m % GS_PAD, zero if >= gs
-    static_assert(GS_PAD * (RI_DIM / 8) <= 256, "one piece of the query per thread");
+    static_assert(GS_PAD * (RI_DIM / 8) <= NT, "one piece of the query per thread");
     {
       const int head = threadIdx.x / (RI_DIM / 8), piece = threadIdx.x % (RI_DIM / 8);
       uint4 qv = ri_zero16();
       if (head < gs) qv = ri_ld16(P.q + ((size_t)g * gs + head) * RI_DIM + piece * 8);
       if (head < GS_PAD) *reinterpret_cast<uint4*>(&sh_q[head][piece * 8]) = qv;
     }
-    if (tab) {
+    if (tab_fast) {
 #pragma unroll
-      for (int u = 0; u < 4; ++u) {
-        const int i = threadIdx.x + u * 256;
+      for (int u = 0; u < TAB_U; ++u) {
+        const int i = threadIdx.x + u * NT;
         if (i <= P.np) sh_roff[i] = t_off[u];
         if (i < P.np) sh_rst[i] = t_st[u];
+      }
+    } else if (tab) {
+      for (int i = threadIdx.x; i <= P.np; i += NT) {
+        sh_roff[i] = P.ret_off[(size_t)g * (P.np + 1) + i];
+        if (i < P.np) sh_rst[i] = P.ret_start[(size_t)g * P.np + i];
       }
     }
     // (the row count is consumed only now: the loads above went out together with its load)
@@ -238,9 +256,9 @@ __global__ __launch_bounds__(256, GS_PAD == 16 ? 1 : 3) void attend_kernel(Atten
     const int total = est_split ? P.es : lenA_all + lenB;
     int r0, r1;
     if (est_split)
-      wave_rows(total, P.S_es * 4, (split - P.S_kv) * 4 + wave, &r0, &r1);
+      wave_rows(total, P.S_es * NW, (split - P.S_kv) * NW + wave, &r0, &r1);
     else
-      wave_rows(total, P.S_kv * 4, split * 4 + wave, &r0, &r1);
+      wave_rows(total, P.S_kv * NW, split * NW + wave, &r0, &r1);
     const uint16_t* qrow = &sh_q[n % GS_PAD][h * 8];
     const uint16_t* kA = P.kA + (size_t)g * P.strideA * RI_DIM;
     const uint16_t* vA = P.vA + (size_t)g * P.strideA * RI_DIM;
@@ -349,7 +367,7 @@ __global__ __launch_bounds__(256, GS_PAD == 16 ? 1 : 3) void attend_kernel(Atten
     // ---------------- estimation rows ----------------
     const int es = P.es;
     int r0, r1;
-    wave_rows(es, P.S_es * 4, (split - P.S_kv) * 4 + wave, &r0, &r1);
+    wave_rows(es, P.S_es * NW, (split - P.S_kv) * NW + wave, &r0, &r1);
     const int32_t* ids = P.est_ids + (size_t)g * es;
     const uint16_t* vs = P.value_sum + (size_t)g * P.nc * RI_DIM;
     const uint16_t* cs = P.csize + (size_t)g * P.nc;
@@ -429,14 +447,16 @@ __global__ __launch_bounds__(256, GS_PAD == 16 ? 1 : 3) void attend_kernel(Atten
   }
   __syncthreads();
 
-  // ---------------- merge the four waves, write the split partial ----------------
+  // ---------------- merge the waves, write the split partial ----------------
   const int S = P.S_kv + P.S_es;
-  for (int idx = threadIdx.x; idx < GS_PAD * RI_DIM; idx += 256) {
+  for (int idx = threadIdx.x; idx < GS_PAD * RI_DIM; idx += NT) {
     const int j = idx / RI_DIM, d = idx % RI_DIM;
-    const float M = fmaxf(fmaxf(sh_m[0][j], sh_m[1][j]), fmaxf(sh_m[2][j], sh_m[3][j]));
+    float M = sh_m[0][j];
+#pragma unroll
+    for (int w = 1; w < NW; ++w) M = fmaxf(M, sh_m[w][j]);
     float a = 0.f, l = 0.f;
 #pragma unroll
-    for (int w = 0; w < 4; ++w) {
+    for (int w = 0; w < NW; ++w) {
       const float f = (sh_m[w][j] == -INFINITY) ? 0.f : __expf(sh_m[w][j] - M);
       a += sh_acc[w][j][d] * f;
       l += sh_l[w][j] * f;
@@ -466,6 +486,9 @@ __global__ __launch_bounds__(256, GS_PAD == 16 ? 1 : 3) void attend_kernel(Atten
   // was measured at +15 us per launch (35.2 us instead of 20.0 us at the benchmark shape), while the
   // data that must be ordered is only this workgroup's own 2 KB.  The asm statement keeps the compiler
   // from moving the stores below the wait.
+#if defined(__HIP_DEVICE_COMPILE__) && !defined(__gfx950__)
+#error "the partial hand-off below relies on gfx950 cache behaviour: build this file for gfx950 only"
+#endif
   asm volatile("" ::: "memory");
   __builtin_amdgcn_s_waitcnt(0);
   __syncthreads();
@@ -473,7 +496,7 @@ __global__ __launch_bounds__(256, GS_PAD == 16 ? 1 : 3) void attend_kernel(Atten
     sh_last = (__hip_atomic_fetch_add(&P.counters[g], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == S - 1);
   __syncthreads();
   if (!sh_last) return;
-  combine_group<GS_PAD>(P, g, S, lenA_all, lenB);
+  combine_group<GS_PAD, NW>(P, g, S, lenA_all, lenB);
   // ready for the next launch (every arrival of this launch has been counted; launches that share the
   // workspace do not overlap)
   if (threadIdx.x == 0) __hip_atomic_store(&P.counters[g], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -483,6 +506,7 @@ __global__ __launch_bounds__(256, GS_PAD == 16 ? 1 : 3) void attend_kernel(Atten
 // host side
 // ------------------------------------------------------------------------------------
 #define RI_MAX_SPLITS 64
+#define RI_MAX_PROBES 8192  // rank tables of a launch: (2 * np + 1) * 4 bytes of LDS
 #define RI_MAX_GROUPS 4096  // size of the counter area at the head of the workspace
 
 static inline int gs_pad_of(int gs) { return gs <= 4 ? 4 : (gs <= 8 ? 8 : 16); }
@@ -509,16 +533,35 @@ static void carve_workspace(AttendParams& P, void* workspace, int BG, int gp) {
   P.part_acc = P.part_ml + (size_t)BG * S * gp * 2;
 }
 
-static int launch_attend(AttendParams& P, int BG, int gs, hipStream_t s) {
+static int launch_attend(AttendParams& P, int BG, int gs, int nw, hipStream_t s) {
   const int S = P.S_kv + P.S_es;
   const dim3 grid(S, BG);
-  switch (gs_pad_of(gs)) {
-    case 4: attend_kernel<4, 1><<<grid, 256, 0, s>>>(P); break;
-    case 8: attend_kernel<8, 1><<<grid, 256, 0, s>>>(P); break;
-    default: attend_kernel<16, 1><<<grid, 256, 0, s>>>(P); break;
-  }
+  const size_t tab_bytes = P.ret_off ? (size_t)(2 * P.np + 1) * sizeof(int) : 0;
+  const int gp = gs_pad_of(gs);
+  if (nw == 8 && gp == 4) attend_kernel<4, 8, 1><<<grid, 512, tab_bytes, s>>>(P);
+  else if (nw == 8 && gp == 8) attend_kernel<8, 8, 1><<<grid, 512, tab_bytes, s>>>(P);
+  else if (gp == 4) attend_kernel<4, 4, 1><<<grid, 256, tab_bytes, s>>>(P);
+  else if (gp == 8) attend_kernel<8, 4, 1><<<grid, 256, tab_bytes, s>>>(P);
+  else attend_kernel<16, 4, 1><<<grid, 256, tab_bytes, s>>>(P);
   RI_HIP_CHECK_LAUNCH();
   return RI_OK;
+}
+
+// Waves per workgroup of a launch.  Eight for groups of up to four query heads: half the split partials and
+// arrivals per group at the same number of waves per compute unit (32 groups of 4 heads over 8192 clusters:
+// 18.7 against 19.3 us per launch).  Four otherwise: with eight or more heads the wave partials of an
+// eight-wave workgroup take so much LDS that only one workgroup fits a compute unit (64 groups of 8 heads over
+// 16384 clusters: 71 against 53 us).  RI_ATTEND_WAVES=4|8 in the environment overrides the choice for groups of
+// up to eight heads (read once, for measurements).
+static int attend_waves(int gs) {
+  static const int forced = [] {
+    const char* e = getenv("RI_ATTEND_WAVES");
+    return e ? atoi(e) : 0;
+  }();
+  const int gp = gs_pad_of(gs);
+  if (gp == 16) return 4;
+  if (forced == 4 || forced == 8) return forced;
+  return gp == 4 ? 8 : 4;
 }
 
 // Memory traffic of one estimation row: its value-sum row, the 32-byte sector around its cluster size, and
@@ -532,16 +575,16 @@ static int est_row_bytes(int gs, bool scored_here) { return 256 + 32 + (scored_h
 // against the 512 bytes of a K and a V row (the launch is bound by its traffic: weighing a key/value
 // row twice an estimation row, by its arithmetic, left the estimation workgroups finishing last,
 // 20.2 against 19.5 us at 32 groups of 4 heads and 60.4 against 54.9 us at 64 groups of 8).
-static void plan_splits(int64_t kv_rows, int64_t es_rows, int es_row_bytes, int BG, int* S_kv, int* S_es) {
-  // two workgroups per compute unit while the launch is short (latency counts); three once every
-  // workgroup has more than 512 rows to stream (throughput counts)
+static void plan_splits(int64_t kv_rows, int64_t es_rows, int es_row_bytes, int BG, int nw, int* S_kv, int* S_es) {
+  // eight waves per compute unit while the launch is short (latency counts); twelve once every
+  // wave has more than 128 rows to stream (throughput counts)
   const int64_t all_rows = (kv_rows + es_rows) * BG;
-  const int target_wgs = all_rows > 512 * 512 ? 768 : 512;
+  const int target_wgs = (all_rows > 512 * 512 ? 768 : 512) * 4 / nw;
   int per_group = target_wgs / BG;
   if (per_group < 1) per_group = 1;
   if (per_group > RI_MAX_SPLITS) per_group = RI_MAX_SPLITS;
   const int64_t rows = kv_rows + es_rows;
-  int64_t by_rows = (rows + 127) / 128;
+  int64_t by_rows = (rows + 32 * nw - 1) / (32 * nw);
   if (by_rows < 1) by_rows = 1;
   if (per_group > by_rows) per_group = (int)by_rows;
   if (es_rows <= 0) {
@@ -580,7 +623,8 @@ extern "C" int ri_weighted_flash_decoding(const void* q, const void* k, const vo
   P.lenB_const = S;
   P.weightB = (const uint16_t*)weight;
   P.weight_stride = S;
-  plan_splits(S, 0, 0, BG, &P.S_kv, &P.S_es);
+  const int nw = attend_waves(gs);
+  plan_splits(S, 0, 0, BG, nw, &P.S_kv, &P.S_es);
   P.gs = gs;
   P.scale = scale;
   P.prev_out = (const uint16_t*)prev_out;
@@ -588,7 +632,7 @@ extern "C" int ri_weighted_flash_decoding(const void* q, const void* k, const vo
   P.out = (uint16_t*)out;
   P.lse_out = lse_out;
   carve_workspace(P, workspace, BG, gp);
-  return launch_attend(P, BG, gs, (hipStream_t)stream);
+  return launch_attend(P, BG, gs, nw, (hipStream_t)stream);
 }
 
 // Shared body of ri_wave_attention and ri_wave_attention_static.  `scratch` holds the arrival
@@ -613,7 +657,7 @@ static int wave_attention_impl(const void* q, const void* steady_k, const void* 
   if ((prev_out == nullptr) != (prev_lse == nullptr) || ri_misaligned16(prev_out)) return RI_ERR_ARG;
   if (ri_any_misaligned16(q, steady_k, steady_v, store_k, store_v, value_sum, est_centroids, out, scratch))
     return RI_ERR_ARG;
-  if (!row_src && (!ret_tok_off || !ret_start || np <= 0 || np > 1023)) return RI_ERR_ARG;
+  if (!row_src && (!ret_tok_off || !ret_start || np <= 0 || np > RI_MAX_PROBES)) return RI_ERR_ARG;
   if (BG <= 0 || BG > RI_MAX_GROUPS || gs <= 0 || gs > 16 || static_len < 0 || static_len > steady_stride ||
       es < 0 || nc <= 0)
     return RI_ERR_ARG;
@@ -657,15 +701,16 @@ static int wave_attention_impl(const void* q, const void* steady_k, const void* 
   // the retrieved-token count is only known on the device: size the split for the row table
   // capacity scaled by the usual fill (a quarter) or for 16 tokens per rank, the estimation zone by
   // its exact size
+  const int nw = attend_waves(gs);
   plan_splits(static_len + (row_src ? row_src_stride / 4 : np * 16), es, est_row_bytes(gs, est_centroids != nullptr), BG,
-              &P.S_kv, &P.S_es);
+              nw, &P.S_kv, &P.S_es);
   if (scratch_bytes < attn_scratch_used(BG, gp, P.S_kv + P.S_es)) return RI_ERR_WORKSPACE;
   carve_workspace(P, scratch, BG, gp);
   if (clear_counters) {
     attend_clear_counters_kernel<<<(BG + 255) / 256, 256, 0, stream>>>(P.counters, BG);
     RI_HIP_CHECK_LAUNCH();
   }
-  return launch_attend(P, BG, gs, stream);
+  return launch_attend(P, BG, gs, nw, stream);
 }
 
 extern "C" int ri_wave_attention(const void* q, const void* steady_k, const void* steady_v,
@@ -791,8 +836,9 @@ extern "C" int ri_buffer_attention(const void* q, const void* buf_k, const void*
   P.scale = scale;
   P.out = (uint16_t*)out;
   // the valid lengths are only known on the device: size the split for a quarter of the buffer
-  plan_splits(max_len / 4 + 64, es, est_row_bytes(gs, false), BG, &P.S_kv, &P.S_es);
+  const int nw = attend_waves(gs);
+  plan_splits(max_len / 4 + 64, es, est_row_bytes(gs, false), BG, nw, &P.S_kv, &P.S_es);
   carve_workspace(P, workspace, BG, gp);
-  return launch_attend(P, BG, gs, (hipStream_t)stream);
+  return launch_attend(P, BG, gs, nw, (hipStream_t)stream);
 }
 

@@ -68,11 +68,14 @@ __device__ __forceinline__ void lru_scan(const int (&v)[N], int (&pre)[N], int (
   __syncthreads();
 }
 
+// R: ranks of the probe list a thread owns (thread t: ranks [t*R, t*R + R)); 1 up to 1023 probes, 4 up to 4096.
+template <int R>
 __global__ __launch_bounds__(LRU_THREADS) void lru_kernel(LruParams P) {
-  __shared__ int sh_scan[4 * LRU_WAVES];
+  constexpr int NPMAX = LRU_THREADS * R;
+  __shared__ int sh_scan[5 * LRU_WAVES];
   __shared__ int sh_hist[LRU_AGES];
   __shared__ int sh_cut[2];  // boundary age, blocks freed by strictly older clusters
-  __shared__ int sh_off[LRU_THREADS], sh_src[LRU_THREADS];
+  __shared__ int sh_off[NPMAX], sh_src[NPMAX];
   const int g = blockIdx.x;
   const int tid = threadIdx.x;
   const int block = P.block;
@@ -85,55 +88,109 @@ __global__ __launch_bounds__(LRU_THREADS) void lru_kernel(LruParams P) {
   const size_t lo = (size_t)g * P.buffer_size;
   const int E = P.epoch[g] + 1;
   const int F0 = P.free_count[g];
+  const int rb = tid * R;
 
-  // ---- access: thread r looks at the cluster of rank r ----
+  // ---- access: every rank looks at its cluster ----
   // (everything the rank needs to know about its cluster is requested in one go: loads issued after a
   // barrier would each put another round trip to global memory on the kernel's critical path)
-  int c = -1, nb = 0, sz = 0, stamp_c = 0, boff_c = 0, start_c = 0;
-  if (tid < P.np) {
-    c = P.ret_ids[(size_t)g * P.np + tid];
-    if (c < 0 || c >= P.ncl) {
-      c = -1;
-    } else {
-      sz = sizes[c];
-      stamp_c = stamp[c];
-      boff_c = boff[c];
-      start_c = starts[c];
-      nb = (sz + block - 1) / block;
+  int c[R], nb[R], sz[R], stamp_c[R], boff_c[R], start_c[R];
+  int nb_sum = 0;
+#pragma unroll
+  for (int i = 0; i < R; ++i) {
+    c[i] = -1; nb[i] = 0; sz[i] = 0; stamp_c[i] = 0; boff_c[i] = 0; start_c[i] = 0;
+    if (rb + i < P.np) {
+      c[i] = P.ret_ids[(size_t)g * P.np + rb + i];
+      if (c[i] < 0 || c[i] >= P.ncl) {
+        c[i] = -1;
+      } else {
+        sz[i] = sizes[c[i]];
+        stamp_c[i] = stamp[c[i]];
+        boff_c[i] = boff[c[i]];
+        start_c[i] = starts[c[i]];
+        nb[i] = (sz[i] + block - 1) / block;
+      }
     }
+    nb_sum += nb[i];
   }
-  int v1[1] = {nb}, p1[1], t1[1];
+  int v1[1] = {nb_sum}, p1[1], t1[1];
   lru_scan<1>(v1, p1, t1, sh_scan);
   // the walk stops at the first cluster whose blocks no longer fit: everything after it is dropped
-  const bool keep = c >= 0 && nb > 0 && p1[0] + nb <= P.buffer_size;
-  const bool hit = keep && stamp_c != 0;
-  const bool miss = keep && !hit;
-  int v4[4] = {hit ? nb : 0, keep ? sz : 0, miss ? nb : 0, miss ? sz : 0}, p4[4], t4[4];
-  lru_scan<4>(v4, p4, t4, sh_scan);
-  // p4[1]: tokens of kept clusters of lower rank (position in the row table); the hit list's own
-  // token offsets are only needed without a row table
-  int hit_tok = 0;
-  if (!P.row_src) {
-    int vh[1] = {hit ? sz : 0}, ph[1], th[1];
-    lru_scan<1>(vh, ph, th, sh_scan);
-    hit_tok = ph[0];
+  bool keep[R], hit[R], miss[R];
+  int v5[5] = {0, 0, 0, 0, 0}, p5[5], t5[5];
+  {
+    int run = p1[0];
+#pragma unroll
+    for (int i = 0; i < R; ++i) {
+      keep[i] = c[i] >= 0 && nb[i] > 0 && run + nb[i] <= P.buffer_size;
+      hit[i] = keep[i] && stamp_c[i] != 0;
+      miss[i] = keep[i] && !hit[i];
+      run += nb[i];
+      v5[0] += hit[i] ? nb[i] : 0;
+      v5[1] += keep[i] ? sz[i] : 0;
+      v5[2] += miss[i] ? nb[i] : 0;
+      v5[3] += miss[i] ? sz[i] : 0;
+      v5[4] += keep[i] ? 1 : 0;
+    }
   }
-  // the longest prefix of the misses whose blocks fit the whole cache may be admitted
-  bool adm = miss && p4[2] + nb <= P.capacity;
-  int va[1] = {adm ? nb : 0}, pa[1], ta[1];
+  lru_scan<5>(v5, p5, t5, sh_scan);
+  // per rank: hit blocks, kept tokens, miss blocks, miss tokens of the lower ranks
+  int hb_pre[R], tok_pre[R], mb_pre[R], mt_pre[R];
+  {
+    int a = p5[0], b = p5[1], cc = p5[2], d = p5[3];
+#pragma unroll
+    for (int i = 0; i < R; ++i) {
+      hb_pre[i] = a; tok_pre[i] = b; mb_pre[i] = cc; mt_pre[i] = d;
+      a += hit[i] ? nb[i] : 0;
+      b += keep[i] ? sz[i] : 0;
+      cc += miss[i] ? nb[i] : 0;
+      d += miss[i] ? sz[i] : 0;
+    }
+  }
+  // tok_pre: tokens of kept clusters of lower rank (position in the row table); the hit list's own
+  // token offsets are only needed without a row table
+  int hit_tok[R];
+#pragma unroll
+  for (int i = 0; i < R; ++i) hit_tok[i] = 0;
+  if (!P.row_src) {
+    int vh[1] = {0}, ph[1], th[1];
+#pragma unroll
+    for (int i = 0; i < R; ++i) vh[0] += hit[i] ? sz[i] : 0;
+    lru_scan<1>(vh, ph, th, sh_scan);
+    int a = ph[0];
+#pragma unroll
+    for (int i = 0; i < R; ++i) { hit_tok[i] = a; a += hit[i] ? sz[i] : 0; }
+  }
+  // the longest prefix of the misses whose blocks fit the whole cache may be admitted (none when the cache
+  // has no blocks: every retrieved cluster then stays a miss, wave_buffer_cpu.cpp:119-130 with capacity 0)
+  bool adm[R];
+  int va[1] = {0}, pa[1], ta[1];
+#pragma unroll
+  for (int i = 0; i < R; ++i) {
+    adm[i] = miss[i] && mb_pre[i] + nb[i] <= P.capacity;
+    va[0] += adm[i] ? nb[i] : 0;
+  }
   lru_scan<1>(va, pa, ta, sh_scan);
   const int need = ta[0];
+  int adm_pre[R];
+  {
+    int a = pa[0];
+#pragma unroll
+    for (int i = 0; i < R; ++i) { adm_pre[i] = a; a += adm[i] ? nb[i] : 0; }
+  }
 
   const bool rows = P.row_src != nullptr;
   if (rows) {
     // row table: every thread takes tokens t, t + 1024, ... and finds the rank that owns them by
     // bisection over the token offsets of the ranks (clusters that were dropped have no tokens)
-    sh_off[tid] = p4[1];
-    sh_src[tid] = hit ? -(boff_c + 1) : P.stage_row0 + p4[3];  // hits: where their block ids are
+#pragma unroll
+    for (int i = 0; i < R; ++i) {
+      sh_off[rb + i] = tok_pre[i];
+      sh_src[rb + i] = hit[i] ? -(boff_c[i] + 1) : P.stage_row0 + mt_pre[i];  // hits: where their block ids are
+    }
     __syncthreads();
     int32_t* table = P.row_src + (size_t)g * P.row_src_stride;
-    for (int t = tid; t < t4[1]; t += LRU_THREADS) {
-      int lo_r = 0, hi_r = LRU_THREADS;  // first rank whose offset exceeds t
+    for (int t = tid; t < t5[1]; t += LRU_THREADS) {
+      int lo_r = 0, hi_r = NPMAX;  // first rank whose offset exceeds t
       while (lo_r < hi_r) {
         const int mid = (lo_r + hi_r) >> 1;
         if (sh_off[mid] > t) hi_r = mid; else lo_r = mid + 1;
@@ -142,35 +199,35 @@ __global__ __launch_bounds__(LRU_THREADS) void lru_kernel(LruParams P) {
       table[t] = src < 0 ? bids[-src - 1 + i / block] * block + i % block : src + i;
     }
   }
-  if (hit) {
-    const int32_t* ids = bids + boff_c;
-    if (!rows) {
-      for (int j = 0; j < nb; ++j) {
-        P.hit_ids[lo + p4[0] + j] = ids[j];
-        P.hit_sizes[lo + p4[0] + j] = (j == nb - 1) ? sz - (nb - 1) * block : block;
-        P.hit_cumsum[lo + p4[0] + j] = hit_tok + j * block;
+#pragma unroll
+  for (int i = 0; i < R; ++i) {
+    if (hit[i]) {
+      const int32_t* ids = bids + boff_c[i];
+      if (!rows) {
+        for (int j = 0; j < nb[i]; ++j) {
+          P.hit_ids[lo + hb_pre[i] + j] = ids[j];
+          P.hit_sizes[lo + hb_pre[i] + j] = (j == nb[i] - 1) ? sz[i] - (nb[i] - 1) * block : block;
+          P.hit_cumsum[lo + hb_pre[i] + j] = hit_tok[i] + j * block;
+        }
       }
+      stamp[c[i]] = E;
     }
-    stamp[c] = E;
-  }
-  if (miss) {
-    const int row = start_c;
-    for (int j = 0; j < nb; ++j) {
-      P.miss_ids[lo + p4[2] + j] = row + j * block;
-      P.miss_sizes[lo + p4[2] + j] = (j == nb - 1) ? sz - (nb - 1) * block : block;
-      P.miss_cumsum[lo + p4[2] + j] = p4[3] + j * block;
+    if (miss[i]) {
+      const int row = start_c[i];
+      for (int j = 0; j < nb[i]; ++j) {
+        P.miss_ids[lo + mb_pre[i] + j] = row + j * block;
+        P.miss_sizes[lo + mb_pre[i] + j] = (j == nb[i] - 1) ? sz[i] - (nb[i] - 1) * block : block;
+        P.miss_cumsum[lo + mb_pre[i] + j] = mt_pre[i] + j * block;
+      }
     }
   }
   if (tid == 0) {
-    P.hit_num[g] = rows ? 0 : t4[0];
-    P.miss_num[g] = t4[2];
-  }
-  if (P.meta) {
-    const int nkept = __syncthreads_count(keep);
-    if (tid == 0) {
-      P.meta[g * 4 + 0] = nkept;
-      P.meta[g * 4 + 1] = t4[1];
-      P.meta[g * 4 + 2] = t4[0] + t4[2];
+    P.hit_num[g] = rows ? 0 : t5[0];
+    P.miss_num[g] = t5[2];
+    if (P.meta) {
+      P.meta[g * 4 + 0] = t5[4];
+      P.meta[g * 4 + 1] = t5[1];
+      P.meta[g * 4 + 2] = t5[0] + t5[2];
       P.meta[g * 4 + 3] = 0;
     }
   }
@@ -239,19 +296,26 @@ __global__ __launch_bounds__(LRU_THREADS) void lru_kernel(LruParams P) {
   }
 
   // ---- admission: block ids come off the end of the free list in rank order ----
-  adm = adm && pa[0] + nb <= F;  // cut short if the untouched clusters did not cover the request
-  int vb[1] = {adm ? nb : 0}, pb[1], tb[1];
+  int vb[1] = {0}, pb[1], tb[1];
+#pragma unroll
+  for (int i = 0; i < R; ++i) {
+    adm[i] = adm[i] && adm_pre[i] + nb[i] <= F;  // cut short if the untouched clusters did not cover the request
+    vb[0] += adm[i] ? nb[i] : 0;
+  }
   lru_scan<1>(vb, pb, tb, sh_scan);
-  if (adm) {
-    int32_t* ids = bids + boff_c;
-    for (int j = 0; j < nb; ++j) {
-      const int id = flist[F - 1 - (pa[0] + j)];
-      ids[j] = id;
-      P.upd_cache[lo + pa[0] + j] = id;
-      P.upd_sizes[lo + pa[0] + j] = (j == nb - 1) ? sz - (nb - 1) * block : block;
-      P.upd_buf[lo + pa[0] + j] = p4[3] + j * block;  // admitted misses lead the miss list
+#pragma unroll
+  for (int i = 0; i < R; ++i) {
+    if (adm[i]) {
+      int32_t* ids = bids + boff_c[i];
+      for (int j = 0; j < nb[i]; ++j) {
+        const int id = flist[F - 1 - (adm_pre[i] + j)];
+        ids[j] = id;
+        P.upd_cache[lo + adm_pre[i] + j] = id;
+        P.upd_sizes[lo + adm_pre[i] + j] = (j == nb[i] - 1) ? sz[i] - (nb[i] - 1) * block : block;
+        P.upd_buf[lo + adm_pre[i] + j] = mt_pre[i] + j * block;  // admitted misses lead the miss list
+      }
+      stamp[c[i]] = E;
     }
-    stamp[c] = E;
   }
   if (tid == 0) {
     P.upd_num[g] = tb[0];
@@ -269,12 +333,14 @@ extern "C" int ri_lru_access_update(const int32_t* ret_ids, const int32_t* sizes
                                     int32_t* upd_cache, int32_t* upd_num, int32_t* row_src, int row_src_stride,
                                     int stage_row0, int32_t* meta, int BG, int np, int ncl, int buffer_size,
                                     int capacity, int block, ri_stream_t stream) {
-  if (!ret_ids || !sizes || !starts || !blk_off || !stamp || !blk_ids || !free_list || !free_count || !epoch ||
+  // (a cache without blocks has an empty free list: its pointer may be null)
+  if (!ret_ids || !sizes || !starts || !blk_off || !stamp || !blk_ids || (!free_list && capacity > 0) || !free_count ||
+      !epoch ||
       !hit_ids || !hit_sizes || !hit_cumsum || !hit_num || !miss_ids || !miss_sizes || !miss_cumsum || !miss_num ||
       !upd_buf || !upd_sizes || !upd_cache || !upd_num)
     return RI_ERR_ARG;
-  if (BG <= 0 || np <= 0 || np > LRU_THREADS - 1 || ncl <= 0 || ncl > 64 * LRU_THREADS || buffer_size <= 0 ||
-      capacity <= 0 || block <= 0)
+  if (BG <= 0 || np <= 0 || np > 4 * LRU_THREADS || ncl <= 0 || ncl > 64 * LRU_THREADS || buffer_size <= 0 ||
+      capacity < 0 || block <= 0)
     return RI_ERR_ARG;
   if (meta_stride < ncl || blk_off_stride < ncl + 1 || stamp_stride < ncl || blk_ids_stride <= 0) return RI_ERR_ARG;
   if (row_src && (!meta || row_src_stride < buffer_size * block || stage_row0 < capacity * block)) return RI_ERR_ARG;
@@ -282,7 +348,10 @@ extern "C" int ri_lru_access_update(const int32_t* ret_ids, const int32_t* sizes
                  hit_ids, hit_sizes, hit_cumsum, hit_num, miss_ids, miss_sizes, miss_cumsum, miss_num,
                  upd_buf, upd_sizes, upd_cache, upd_num, row_src, meta, row_src_stride, stage_row0,
                  np, ncl, meta_stride, blk_off_stride, stamp_stride, blk_ids_stride, buffer_size, capacity, block};
-  lru_kernel<<<BG, LRU_THREADS, 0, (hipStream_t)stream>>>(P);
+  if (np < LRU_THREADS)
+    lru_kernel<1><<<BG, LRU_THREADS, 0, (hipStream_t)stream>>>(P);
+  else
+    lru_kernel<4><<<BG, LRU_THREADS, 0, (hipStream_t)stream>>>(P);
   RI_HIP_CHECK_LAUNCH();
   return RI_OK;
 }

@@ -17,6 +17,7 @@
 #include "ri_common.h"
 
 #define SEL_THREADS 1024
+#define SEL_MAX_PROBES 4096  // ranks of the retrieval zone one workgroup can lay out (four per thread)
 #define SEL_WAVES (SEL_THREADS / 64)
 #define DIST_IDS 1024  // ids per dist workgroup (4 per thread)
 
@@ -148,7 +149,8 @@ __device__ __forceinline__ uint32_t sel_bin(uint32_t key) {
 // E8: eights of keys a thread owns (1 up to 8192 clusters, 2 up to 16384, 4 up to 32768, 8 up to 65536): the
 // loops over the owned keys are unrolled E8 times, so the common sizes do not carry (and fetch) the code of
 // sixty-four keys per thread.
-template <int E8>
+// R: ranks of the retrieval zone a thread owns in the token-layout phase (1 up to 1023 probes, 4 up to 4096).
+template <int E8, int R>
 __global__ __launch_bounds__(SEL_THREADS) void select_kernel(
     const uint16_t* __restrict__ keys, const int32_t* __restrict__ cluster_size,
     const int32_t* __restrict__ cluster_start, int64_t* __restrict__ cI, int32_t* __restrict__ ret_ids,
@@ -157,10 +159,15 @@ __global__ __launch_bounds__(SEL_THREADS) void select_kernel(
   __shared__ uint32_t hist[SEL_BINS];
   __shared__ uint32_t sh_scan[2][3 * SEL_WAVES];  // two buffers, used alternately
   __shared__ uint32_t sh_sel[4];  // bin of T1, entries above it, bin of T2, entries above it
-  __shared__ uint32_t sh_ret[1024];
-  __shared__ uint32_t sh_sorted[1024];
-  __shared__ uint32_t sh_size[1024];   // size and first store row of the cluster at each rank
-  __shared__ int32_t sh_start[1024];
+  constexpr int NPMAX = SEL_THREADS * R;
+  __shared__ uint32_t sh_ret[NPMAX];
+  // rank-ordered entries, then size and first store row of the cluster at each rank: arrays of their own for
+  // the common case, laid over the histogram (which is dead by then) when a thread owns several ranks
+  __shared__ uint32_t sh_lay[R == 1 ? 3 * NPMAX : 1];
+  static_assert(R == 1 || 3 * NPMAX <= SEL_BINS, "the rank arrays must fit the histogram they are laid over");
+  uint32_t* const sh_sorted = R == 1 ? sh_lay : hist;
+  uint32_t* const sh_size = sh_sorted + NPMAX;
+  int32_t* const sh_start = reinterpret_cast<int32_t*>(sh_sorted + 2 * NPMAX);
   __shared__ uint32_t sh_pages, sh_tret, sh_nkeep;
 
   const int g = blockIdx.x;
@@ -309,37 +316,52 @@ __global__ __launch_bounds__(SEL_THREADS) void select_kernel(
   __syncthreads();
 
   // ---- token layout of the retrieved clusters with the page cut-off ----
-  // thread r owns rank r (np <= 1023 < threads)
-  uint32_t sz = 0, pg = 0;
-  int32_t st = 0;
-  const int r = tid;
-  int my_c = -1;
-  if (r < np) {
-    my_c = (int)(0xffffu - (sh_sorted[r] & 0xffffu));
-    st = sh_start[r];
-    sz = sh_size[r];
-    pg = (sz + page - 1) / page;
+  // thread t owns the ranks [t*R, t*R + R)
+  const int rb = tid * R;
+  uint32_t sz[R], pg[R];
+  int32_t st[R];
+  int my_c[R];
+  uint32_t pg_sum = 0, sz_sum = 0;
+#pragma unroll
+  for (int i = 0; i < R; ++i) {
+    sz[i] = 0; pg[i] = 0; st[i] = 0; my_c[i] = -1;
+    if (rb + i < np) {
+      my_c[i] = (int)(0xffffu - (sh_sorted[rb + i] & 0xffffu));
+      st[i] = sh_start[rb + i];
+      sz[i] = sh_size[rb + i];
+      pg[i] = (sz[i] + page - 1) / page;
+    }
+    pg_sum += pg[i];
+    sz_sum += sz[i];
   }
-  bool keep = false;
-  uint32_t tok_run = 0;
+  uint32_t tok_run[R];
+  uint32_t keep_bits = 0;
   int nkeep = 0;
   int32_t T_ret = 0;
   if (cluster_size) {
-    uint32_t lay[2] = {pg, sz}, layp[2], layt[2];
+    uint32_t lay[2] = {pg_sum, sz_sum}, layp[2], layt[2];
     block_excl_scan<2>(lay, layp, layt, sh_scan[0]);
-    const uint32_t pg_run = layp[0];
-    tok_run = layp[1];
+    uint32_t pg_run = layp[0], tk = layp[1];
     // kept clusters form a prefix because the page prefix is monotone; tokens before a kept
     // cluster all belong to kept clusters
-    keep = r < np && pg_run + pg <= (uint32_t)max_pages;
-    // the kept clusters are the ranks 0 .. nkeep-1: the last of them publishes the totals
-    if (keep) {
-      const bool next_keep = r + 1 < np && pg_run + pg + (sh_size[r + 1] + page - 1) / page <= (uint32_t)max_pages;
-      if (!next_keep) {
-        sh_pages = pg_run + pg;
-        sh_tret = tok_run + sz;
-        sh_nkeep = (uint32_t)r + 1u;
+#pragma unroll
+    for (int i = 0; i < R; ++i) {
+      tok_run[i] = tk;
+      const int r = rb + i;
+      const bool keep = r < np && pg_run + pg[i] <= (uint32_t)max_pages;
+      // the kept clusters are the ranks 0 .. nkeep-1: the last of them publishes the totals
+      if (keep) {
+        keep_bits |= 1u << i;
+        const uint32_t next_pg = (i + 1 < R) ? pg[i + 1] : (r + 1 < np ? (sh_size[r + 1] + page - 1) / page : 0u);
+        const bool next_keep = r + 1 < np && pg_run + pg[i] + next_pg <= (uint32_t)max_pages;
+        if (!next_keep) {
+          sh_pages = pg_run + pg[i];
+          sh_tret = tk + sz[i];
+          sh_nkeep = (uint32_t)r + 1u;
+        }
       }
+      pg_run += pg[i];
+      tk += sz[i];
     }
     __syncthreads();
     nkeep = (int)sh_nkeep;
@@ -347,9 +369,12 @@ __global__ __launch_bounds__(SEL_THREADS) void select_kernel(
   }
 
   // ---- all global stores ----
-  if (r < np) {
-    ret_ids[(size_t)g * np + r] = my_c;
-    if (cI) cI[(size_t)g * k2 + r] = my_c;
+#pragma unroll
+  for (int i = 0; i < R; ++i) {
+    if (rb + i < np) {
+      ret_ids[(size_t)g * np + rb + i] = my_c[i];
+      if (cI) cI[(size_t)g * k2 + rb + i] = my_c[i];
+    }
   }
   {
     uint32_t est_off = est_first;
@@ -362,19 +387,30 @@ __global__ __launch_bounds__(SEL_THREADS) void select_kernel(
     }
   }
   if (!cluster_size) return;
-  if (r <= np) ret_tok_off[(size_t)g * (np + 1) + r] = (r < nkeep) ? (int32_t)tok_run : T_ret;
-  if (ret_start && r < np) ret_start[(size_t)g * np + r] = st;
+#pragma unroll
+  for (int i = 0; i < R; ++i) {
+    const int r = rb + i;
+    if (r < np) {
+      ret_tok_off[(size_t)g * (np + 1) + r] = (r < nkeep) ? (int32_t)tok_run[i] : T_ret;
+      if (ret_start) ret_start[(size_t)g * np + r] = st[i];
+    }
+  }
   if (tid == 0) {
+    ret_tok_off[(size_t)g * (np + 1) + np] = T_ret;
     meta[g * 4 + 0] = nkeep;
     meta[g * 4 + 1] = T_ret;
     meta[g * 4 + 2] = (int32_t)sh_pages;
     meta[g * 4 + 3] = 0;
   }
   // row table: each kept cluster writes the rows of its tokens
-  if (!row_src || !cluster_start || !keep) return;
-  int32_t* dst = row_src + (size_t)g * row_src_stride + tok_run;
-  const int room = row_src_stride - (int)tok_run;
-  for (int i = 0; i < (int)sz && i < room; ++i) dst[i] = st + i;
+  if (!row_src || !cluster_start) return;
+#pragma unroll
+  for (int i = 0; i < R; ++i) {
+    if (!((keep_bits >> i) & 1u)) continue;
+    int32_t* dst = row_src + (size_t)g * row_src_stride + tok_run[i];
+    const int room = row_src_stride - (int)tok_run[i];
+    for (int k = 0; k < (int)sz[i] && k < room; ++k) dst[k] = st[i] + k;
+  }
 }
 
 // ------------------------------------------------------------------------------------
@@ -398,7 +434,7 @@ extern "C" int ri_score_select(const void* q, const void* centroids, const uint8
   if (!q || !centroids || !logits || !ret_ids || !workspace) return RI_ERR_ARG;
   if (ri_any_misaligned16(q, centroids, logits, workspace)) return RI_ERR_ARG;
   if (BG <= 0 || gs <= 0 || gs > 16 || nc <= 0 || (nc % 8) != 0) return RI_ERR_ARG;
-  if (np <= 0 || np > 1023 || es < 0 || np + es > nc || nc > 65536) return RI_ERR_ARG;
+  if (np <= 0 || np > SEL_MAX_PROBES || es < 0 || np + es > nc || nc > 65536) return RI_ERR_ARG;
   if (es > 0 && !est_ids) return RI_ERR_ARG;
   if (cluster_size_i32 && (!ret_tok_off || !meta || page <= 0 || max_pages <= 0)) return RI_ERR_ARG;
   if (workspace_bytes < ri_score_select_workspace_bytes(BG, gs, nc)) return RI_ERR_WORKSPACE;
@@ -421,13 +457,20 @@ extern "C" int ri_score_select(const void* q, const void* centroids, const uint8
     dist_kernel<16><<<dgrid, 256, 0, s>>>(logits, tmax, tsum, mask, keys, (uint16_t*)dist, gs, nc, ntiles);
   RI_HIP_CHECK_LAUNCH();
   const int per_thread = (nc + SEL_THREADS - 1) / SEL_THREADS;
-#define RI_SELECT_LAUNCH(E8)                                                                                          \
-  select_kernel<E8><<<BG, SEL_THREADS, 0, s>>>(keys, cluster_size_i32, cluster_start, cI, ret_ids, est_ids, ret_tok_off, \
-                                               ret_start, row_src, row_src_stride, meta, nc, np, es, page, max_pages)
-  if (per_thread <= 8) RI_SELECT_LAUNCH(1);
-  else if (per_thread <= 16) RI_SELECT_LAUNCH(2);
-  else if (per_thread <= 32) RI_SELECT_LAUNCH(4);
-  else RI_SELECT_LAUNCH(8);
+#define RI_SELECT_LAUNCH(E8, R)                                                                                       \
+  select_kernel<E8, R><<<BG, SEL_THREADS, 0, s>>>(keys, cluster_size_i32, cluster_start, cI, ret_ids, est_ids,       \
+                                                  ret_tok_off, ret_start, row_src, row_src_stride, meta, nc, np, es, \
+                                                  page, max_pages)
+  if (np < SEL_THREADS) {
+    if (per_thread <= 8) RI_SELECT_LAUNCH(1, 1);
+    else if (per_thread <= 16) RI_SELECT_LAUNCH(2, 1);
+    else if (per_thread <= 32) RI_SELECT_LAUNCH(4, 1);
+    else RI_SELECT_LAUNCH(8, 1);
+  } else {  // long probe lists only occur with many clusters
+    if (per_thread <= 16) RI_SELECT_LAUNCH(2, 4);
+    else if (per_thread <= 32) RI_SELECT_LAUNCH(4, 4);
+    else RI_SELECT_LAUNCH(8, 4);
+  }
 #undef RI_SELECT_LAUNCH
   RI_HIP_CHECK_LAUNCH();
   return RI_OK;

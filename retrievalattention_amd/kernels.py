@@ -5,6 +5,7 @@ against the reference runs unchanged; the second block exposes the fused MI355X 
 
 Tensors only provide memory and the current stream; all arithmetic happens in the library.
 """
+import contextlib
 import functools
 import math
 
@@ -18,8 +19,19 @@ _DT = (torch.bfloat16, torch.float16)
 
 # Named profiler ranges around the stages of a decode step, with the names the reference gives its NVTX
 # ranges (cache_hub/retroinfer_cache.py:558-678); torch's nvtx calls are roctx ranges on ROCm, so
-# rocprofv3 --marker-trace shows them.  Off unless a cache is built with profiler_ranges=True.
+# rocprofv3 --marker-trace shows them.  Off except inside `with profiler_ranges(True)`, which a cache built
+# with profiler_ranges=True holds around its own calls (so one cache's ranges do not switch on another's).
 PROFILER_RANGES = False
+
+
+@contextlib.contextmanager
+def profiler_ranges(enabled):
+    global PROFILER_RANGES
+    before, PROFILER_RANGES = PROFILER_RANGES, bool(enabled)
+    try:
+        yield
+    finally:
+        PROFILER_RANGES = before
 
 
 def _ranged(name):
@@ -77,6 +89,27 @@ def _workspace(nbytes, device, tag):
         w = torch.zeros(max(nbytes, 256), dtype=torch.uint8, device=device)
         _workspaces[key] = w
     return w
+
+
+def release_cached_graphs(retired_workspaces=True):
+    """Drops what the library keeps alive for replays: the captured clusterings of segment_k_means_csr (only the
+    library replays those, so this is always safe) and, with retired_workspaces, the scratch tensors that were
+    outgrown.  A graph that a caller captured while such a tensor was current still holds its address: drop the
+    retired tensors only when every graph captured before the last growth of a scratch area is gone, or a replay
+    would write into memory that has been handed back.  Refused during a stream capture."""
+    if torch.cuda.is_current_stream_capturing():
+        raise RuntimeError("release_cached_graphs during a stream capture")
+    from .cache_hub import kmeans as _km
+    _km._GRAPHS.clear()
+    _km._SEEN.clear()
+    if retired_workspaces:
+        _retired_workspaces.clear()
+
+
+# limits of the fused decode path (checked by the entry points; callers can check them up front)
+MAX_PROBES = 4096          # ri_score_select / ri_wave_attention / ri_lru_access_update: retrieval zone per group
+MAX_CLUSTERS = 65536       # ri_score_select / ri_lru_access_update: clusters per group (16-bit ids in the selection)
+MAX_GROUP_SIZE = 16        # query heads per KV head
 
 
 # ----------------------------------------------------------------------------------------

@@ -132,3 +132,24 @@ def check_rank_order(dist, ret, band=1.0, slack=None, label=None):
                 FLIP_TALLY[label] = FLIP_TALLY.get(label, 0) + flips
             lim = lim + sl[1:] + sl[:-1]
         assert bool((viol <= lim).all()), f"group {g}: retrieval zone not in rank order"
+
+
+class BlockIdMap:
+    """Bijection between the cache block ids of two block cache managers that follow the same policy but hand
+    out free ids in different orders: ids are bound when a cluster is admitted, must translate consistently
+    while the cluster is resident, and are forgotten when it is evicted (`retain` keeps the reference ids that
+    are still in use)."""
+
+    def __init__(self):
+        self.fwd, self.back = {}, {}
+
+    def bind(self, got, ref):
+        assert got not in self.fwd and ref not in self.back, "block id handed out twice"
+        self.fwd[got], self.back[ref] = ref, got
+
+    def to_ref(self, got):
+        return self.fwd[got]
+
+    def retain(self, live_ref_ids):
+        for ref in [r for r in self.back if r not in live_ref_ids]:
+            del self.fwd[self.back.pop(ref)]

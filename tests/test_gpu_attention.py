@@ -157,6 +157,9 @@ def test_closed_form_estimation_exact_for_singletons_and_identical_keys(dev):
     (1, 3, 256, 1, 255, 0, 7),       # one probe, no steady zone, zones cover every cluster
     (1, 16, 80, 1, 0, 0, 3065),      # one probe and nothing else: one of the two row windows attends nothing
     (1, 16, 112, 10, 0, 0, 3044),    # ten small clusters only: outputs of the size of single value rows
+    (1, 4, 15000, 1500, 2250, 69, 8),   # probe lists of the reference's throughput harness (10 % of the clusters)
+    (1, 4, 30000, 3000, 1000, 69, 9),
+    (1, 8, 16384, 4096, 0, 10, 10),     # the longest probe list
 ])
 def test_wave_attention(dev, BG, gs, nc, nprobe, es, static_len, seed):
     """score_select + wave_attention against the oracle's composition of steps 4-8 of

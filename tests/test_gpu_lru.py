@@ -1,10 +1,12 @@
-"""Device-side block cache manager against its Python restatement (oracle.wavebuf.DeviceLruModel)."""
+"""Device-side block cache manager against its Python restatement (oracle.wavebuf.DeviceLruModel), and
+against the restatement of the reference's manager (oracle.wavebuf.LruModel) where the two policies coincide."""
 import random
 
 import pytest
 import torch
 
-from oracle.wavebuf import DeviceLruModel
+from oracle.wavebuf import DeviceLruModel, LruModel
+from tests.parity import BlockIdMap
 
 pytestmark = pytest.mark.gpu
 
@@ -14,6 +16,9 @@ pytestmark = pytest.mark.gpu
     (3840, 69, 600, 552, 25, 1),     # config-4 sizes: 5 % cache
     (300, 20, 40, 30, 30, 2),        # buffer cut-off and admissions cut short
     (2500, 40, 4000, 400, 12, 3),    # cache larger than everything requested: no eviction
+    (300, 20, 0, 160, 6, 4),         # a cache without blocks (throughput_eval/test.py:77): all misses, none admitted
+    (20000, 1500, 9000, 12000, 6, 5),   # probe lists past 1023 ranks (four ranks per thread)
+    (40000, 3000, 2000, 20000, 5, 6),   #   with the buffer cut-off and admissions cut short
 ])
 def test_lists_match_the_model_step_by_step(dev, ncl, nprobe, capacity, buffer_size, steps, seed):
     from retrievalattention_amd import kernels
@@ -55,7 +60,58 @@ def test_lists_match_the_model_step_by_step(dev, ncl, nprobe, capacity, buffer_s
             assert lru.free_list[g, :len(models[g].free)].tolist() == models[g].free
             stamp = lru.stamp[g, :ncl].cpu()
             assert [int(x) for x in stamp] == models[g].stamp
-    assert any(len(m.blocks) > 0 for m in models)
+    assert capacity == 0 or any(len(m.blocks) > 0 for m in models)
+
+
+@pytest.mark.parametrize("ncl,capacity,steps,seed", [(40, 24, 250, 0), (300, 64, 250, 1), (12, 10, 200, 2)])
+def test_one_probe_per_step_equals_the_reference_policy(dev, ncl, capacity, steps, seed):
+    """With one retrieved cluster per step every recency stamp is unique, and with fewer than 255 steps no age
+    saturates: step-granular recency is then the reference's touch order, so the kernel's hit / miss / admission
+    lists and its evictions must equal those of the reference's manager (LruModel, itself checked against the
+    reference's own BufferManager build), block id values aside (an id map is kept and must stay a bijection)."""
+    from retrievalattention_amd import kernels
+    BG, block, buffer_size = 2, 8, 16
+    rnd = random.Random(seed)
+    sizes = [[rnd.randint(0, 30) for _ in range(ncl)] for _ in range(BG)]
+    refs = [LruModel(s, block, capacity, buffer_size) for s in sizes]
+    maps = [BlockIdMap() for _ in range(BG)]
+    sz = torch.tensor(sizes, dtype=torch.int32, device=dev)
+    st = (torch.cumsum(sz.long(), 1) - sz.long()).to(torch.int32)
+    lru = kernels.DeviceLru(BG, ncl, int(((sz + block - 1) // block).sum(1).max()) + 1, capacity, buffer_size, block, dev)
+    lru.set_sizes(sz)
+    lists = [torch.full((BG, buffer_size), -7, dtype=torch.int32, device=dev) if i % 4 != 3
+             else torch.zeros(BG, dtype=torch.int32, device=dev) for i in range(12)]
+    hot = [rnd.sample(range(ncl), max(2, ncl // 3)) for _ in range(BG)]
+    evictions = 0
+    for step in range(steps):
+        ids = [[rnd.choice(hot[g]) if rnd.random() < 0.6 else rnd.randrange(ncl)] for g in range(BG)]
+        lru.access_update(torch.tensor(ids, dtype=torch.int32, device=dev), sz, st, lists)
+        torch.cuda.synchronize()
+        host = [x.cpu() for x in lists]
+        for g in range(BG):
+            before = set(refs[g].resident)
+            hit, miss = refs[g].access(ids[g])
+            upd = refs[g].update()
+            evictions += len(before - set(refs[g].resident))
+            # blocks of clusters evicted in this step go back to the free list and may be handed out again at once
+            maps[g].retain({b for ids_c in refs[g].resident.values() for b in ids_c} - {b for b, _, _ in upd})
+            for k, ref in enumerate((hit, miss, upd)):
+                a, b, c, n = host[4 * k:4 * k + 4]
+                assert int(n[g]) == len(ref), (step, g, k)
+                got = list(zip(a[g, :len(ref)].tolist(), b[g, :len(ref)].tolist(), c[g, :len(ref)].tolist()))
+                if k == 2:
+                    got = [(z, y, x) for x, y, z in got]
+                if k == 1:                      # misses: host rows, no block ids involved
+                    assert got == ref, (step, g, k)
+                else:
+                    if k == 2:                  # admission hands out ids: the map learns them
+                        for (bg, _, _), (br, _, _) in zip(got, ref):
+                            maps[g].bind(bg, br)
+                    assert [(maps[g].to_ref(x), y, z) for x, y, z in got] == ref, (step, g, k)
+            # the same clusters are resident: evictions happened in the same order
+            resident = set(torch.nonzero(lru.stamp[g, :ncl]).flatten().tolist())
+            assert resident == set(refs[g].resident), (step, g)
+    assert evictions > 0
 
 
 def test_row_table_for_attention_in_place(dev):
@@ -97,6 +153,6 @@ def test_bad_arguments(dev):
     z = torch.zeros(64, dtype=torch.int32, device=dev)
     p = z.data_ptr()
     ptrs = [p] * 12
-    assert l.ri_lru_access_update(p, p, p, 8, p, 9, p, 8, p, 8, p, p, p, *ptrs, None, 0, 0, None, 1, 1024, 8, 4, 4, 8, None) == -1   # np too large
+    assert l.ri_lru_access_update(p, p, p, 8, p, 9, p, 8, p, 8, p, p, p, *ptrs, None, 0, 0, None, 1, 4097, 8, 4, 4, 8, None) == -1   # np too large
     assert l.ri_lru_access_update(p, p, p, 4, p, 9, p, 8, p, 8, p, p, p, *ptrs, None, 0, 0, None, 1, 2, 8, 4, 4, 8, None) == -1      # stride < ncl
     assert l.ri_lru_access_update(None, p, p, 8, p, 9, p, 8, p, 8, p, p, p, *ptrs, None, 0, 0, None, 1, 2, 8, 4, 4, 8, None) == -1

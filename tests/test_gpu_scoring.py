@@ -97,7 +97,10 @@ def test_batch_gemm_softmax_half(dev):
     (3, 1, 64, 1, 0, 4),          # smallest: one probe, no estimation zone
     (2, 16, 1000, 20, 980, 5),    # nc not a multiple of 256, zones cover every cluster
     (1, 4, 32768, 300, 3000, 6),  # more clusters than the select kernel stages in LDS
-    (1, 16, 65536, 1023, 20000, 7),  # the largest shape the entry point takes: 65536 clusters, 1023 probes, 16 heads
+    (1, 16, 65536, 1023, 20000, 7),  # 65536 clusters (the most the entry point takes), 16 heads
+    (2, 4, 15000, 1500, 2250, 8),    # probe lists of the reference's throughput harness (throughput_eval/test.py:74,
+    (1, 4, 30000, 3000, 4500, 9),    #   nprobe = 10 % of the clusters): 240K and 480K tokens of context
+    (1, 8, 40960, 4096, 100, 10),    # the longest probe list the entry point takes
 ])
 def test_score_select(dev, BG, gs, nc, nprobe, es, seed):
     from retrievalattention_amd import kernels
@@ -179,8 +182,8 @@ def test_score_select_many_seeds(dev):
 
 def test_score_select_random_shapes(dev):
     """Every check of test_score_select over 60 shapes drawn from a fixed seed: 1..5 groups, group sizes 1..16
-    (not only the powers of two the models use), 32..48000 clusters in steps of 8, any retrieval zone up to the
-    1023 the selection supports and any estimation zone, including none."""
+    (not only the powers of two the models use), 32..48000 clusters in steps of 8, any retrieval zone up to
+    1023 clusters and any estimation zone, including none; then 8 shapes with 1024..4096 probes."""
     import random
     rnd = random.Random(777)
     for it in range(60):
@@ -190,6 +193,12 @@ def test_score_select_random_shapes(dev):
         nprobe = rnd.randint(1, min(1023, max(1, nc // 4)))
         es = 0 if rnd.random() < 0.2 else rnd.randint(0, nc - nprobe)
         test_score_select(dev, BG, gs, nc, nprobe, es, 1000 + it)
+    for it in range(8):   # probe lists past 1023 (several ranks per thread in the layout phase)
+        BG, gs = rnd.choice([1, 2]), rnd.choice([1, 4, 7, 8, 16])
+        nc = 8 * rnd.randint(640, 5000)
+        nprobe = rnd.randint(1024, min(4096, nc // 3))
+        es = rnd.randint(0, nc - nprobe)
+        test_score_select(dev, BG, gs, nc, nprobe, es, 1100 + it)
 
 
 @pytest.mark.parametrize("kind", ["all_equal", "mostly_masked", "two_values"])
@@ -265,6 +274,12 @@ def test_score_select_rejects_bad_shapes(dev):
     with pytest.raises(RuntimeError, match="invalid argument"):
         kernels.score_select(q.to(dev), cent.to(dev), None, None, None, logits, None, None, ret, None, None, None,
                              None, 80, 0, 8, 16, 1.0)   # nprobe > nc
+    q, cent = _mixture(1, 4, 8192, 0)
+    logits = torch.empty(1, 4, 8192, dtype=torch.float32, device=dev)
+    ret = torch.empty(1, 4097, dtype=torch.int32, device=dev)
+    with pytest.raises(RuntimeError, match="invalid argument"):
+        kernels.score_select(q.to(dev), cent.to(dev), None, None, None, logits, None, None, ret, None, None, None,
+                             None, 4097, 0, 8, 16, 1.0)   # more probes than the selection lays out
 
 
 def test_misaligned_rows_are_rejected(dev):

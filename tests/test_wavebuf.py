@@ -218,3 +218,37 @@ def test_device_lru_model_invariants():
             assert max(last_touch[c] for c in evicted) <= oldest_kept
         for c in evicted:
             last_touch.pop(c, None)
+
+
+@pytest.mark.parametrize("ncl,capacity,steps,seed", [(40, 24, 250, 0), (300, 64, 250, 1), (12, 10, 200, 2), (30, 0, 50, 3)])
+def test_device_policy_equals_the_reference_policy_with_one_probe_per_step(ncl, capacity, steps, seed):
+    """Where the two block cache policies must coincide they do: with one retrieved cluster per step the
+    step-granular recency of DeviceLruModel is a total order (every stamp unique) and, below 255 steps, no age
+    saturates, so it is the touch order of the reference's list (LruModel, pinned by the reference's own
+    BufferManager build).  Hit, miss and admission lists and the set of resident clusters after every step are
+    identical, block id values aside (the two hand out free ids in different orders; the map must stay a
+    bijection)."""
+    import random
+    from oracle.wavebuf import DeviceLruModel
+    from tests.parity import BlockIdMap
+    rnd = random.Random(seed)
+    sizes = [rnd.randint(0, 30) for _ in range(ncl)]
+    dev_m, ref_m, ids_map = DeviceLruModel(sizes, 8, capacity, 16), LruModel(sizes, 8, capacity, 16), BlockIdMap()
+    hot = rnd.sample(range(ncl), max(2, ncl // 3))
+    evictions = 0
+    for step in range(steps):
+        ids = [rnd.choice(hot) if rnd.random() < 0.6 else rnd.randrange(ncl)]
+        before = set(ref_m.resident)
+        hit_r, miss_r = ref_m.access(ids)
+        upd_r = ref_m.update()
+        evictions += len(before - set(ref_m.resident))
+        hit_d, miss_d, upd_d = dev_m.step(ids)
+        assert miss_d == miss_r
+        ids_map.retain({b for v in ref_m.resident.values() for b in v} - {b for b, _, _ in upd_r})
+        assert len(upd_d) == len(upd_r)
+        for (bd, _, _), (br, _, _) in zip(upd_d, upd_r):
+            ids_map.bind(bd, br)
+        assert [(ids_map.to_ref(b), s, o) for b, s, o in hit_d] == hit_r
+        assert [(ids_map.to_ref(b), s, o) for b, s, o in upd_d] == upd_r
+        assert set(dev_m.blocks) == set(ref_m.resident)
+    assert evictions > 0 or capacity == 0
