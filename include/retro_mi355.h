@@ -90,6 +90,7 @@ int ri_batch_gemm_softmax_f16(const void* A, const void* B, void* D, float* Norm
  *   cI         [BG, np+es] int64 or NULL: retrieval ids in rank order (score descending,
  *              ties by ascending id) followed by estimation ids in ascending id order
  *   ret_ids    [BG, np] int32, est_ids [BG, es] int32 (same content as cI)
+ *   (np: 1..4096 clusters in the retrieval zone; nc <= 65536, a multiple of 8)
  *   ret_tok_off[BG, np+1] int32: exclusive token prefix of the retrieval clusters after
  *              the reference's buffer cut-off (stop before the first cluster whose pages
  *              push the running total over max_pages; wave_buffer_cpu.cpp:207-216)
@@ -159,6 +160,8 @@ int ri_weighted_flash_decoding(const void* q, const void* k, const void* v, cons
  *   es > 0) when the zones were chosen from another query than q (next-layer cluster estimation,
  *   cache_hub/retroinfer_cache.py:582-617): the estimation zone's scores are then computed inside
  *   the launch from the centroid rows of est_ids
+ *   np: 1..4096 probes with the rank tables (their 2 np + 1 words are staged in LDS); any number with
+ *   a row table
  *   value_sum [BG, nc, 128] bf16, cluster_size_bf16 [BG, nc] bf16 (estimation weights)
  *   es may be 0 (no estimation zone).  out [BG, gs, 128] bf16; valid_lengths [BG] int32 or
  *   NULL receives static_len + retrieved tokens (what gather_copy_and_concat reports).
@@ -183,7 +186,9 @@ int ri_wave_attention(const void* q, const void* steady_k, const void* steady_v,
  * lse_out [BG, gs] fp32 or NULL receives this part's log-sum-exp.  static_len = 0 leaves the steady zone
  * out, es = 0 the estimation zone.  Two calls over complementary windows, the second with the first's
  * (out, lse_out) as its previous result, equal one ri_wave_attention up to the bf16 rounding of the
- * intermediate output.  A part that attends nothing (no steady zone, no estimation zone, no row inside the
+ * intermediate output.  static_len_dev only counts for a part that attends the steady zone: with
+ * static_len = 0 it is ignored (a caller that hands the same device length to both parts would otherwise
+ * attend the steady zone twice).  A part that attends nothing (no steady zone, no estimation zone, no row inside the
  * window) writes zeros and a log-sum-exp of -inf, and such a previous result is ignored by the part that
  * merges it.  Workspace as for ri_wave_attention. */
 int ri_wave_attention_part(const void* q, const void* steady_k, const void* steady_v,
@@ -330,7 +335,9 @@ int ri_kmeans_value_sum(const void* values, const int32_t* counts, const int32_t
  * Policy: the walk over the ranks stops at the first cluster whose blocks do not fit
  * buffer_size; the longest prefix of the misses that fits `capacity` is admitted; victims are
  * whole clusters, least recently touched step first, ascending id inside a step, never one
- * touched in this call.  np <= 1023, ncl <= 65536.
+ * touched in this call.  np <= 4096, ncl <= 65536.  capacity may be 0 (no block cache, as
+ * throughput_eval/test.py:77 runs the reference): every kept cluster is then a miss at every call and
+ * nothing is admitted (wave_buffer_cpu.cpp:119-130 with a capacity of 0); free_list may then be NULL.
  * With row_src [BG, row_src_stride] and meta [BG, 4] (both or neither): for attention in place over
  * one tensor that holds the `capacity` cache blocks first and the staging rows of the misses from row
  * stage_row0 on, row_src receives the row of every retrieved token (hits: block id * block + i;

@@ -506,7 +506,7 @@ __global__ __launch_bounds__(64 * NW, GS_PAD == 16 ? 1 : 3) void attend_kernel(A
 // host side
 // ------------------------------------------------------------------------------------
 #define RI_MAX_SPLITS 64
-#define RI_MAX_PROBES 8192  // rank tables of a launch: (2 * np + 1) * 4 bytes of LDS
+#define RI_MAX_PROBES 4096  // rank tables of a launch: (2 * np + 1) * 4 bytes of LDS (what the selection lays out)
 #define RI_MAX_GROUPS 4096  // size of the counter area at the head of the workspace
 
 static inline int gs_pad_of(int gs) { return gs <= 4 ? 4 : (gs <= 8 ? 8 : 16); }
@@ -746,6 +746,8 @@ extern "C" int ri_wave_attention_part(const void* q, const void* steady_k, const
                                       size_t workspace_bytes, ri_stream_t stream) {
   if (!row_src || src_row_lo >= src_row_hi) return RI_ERR_ARG;
   if (workspace && workspace_bytes < attn_workspace_bytes(BG, gs)) return RI_ERR_WORKSPACE;
+  // a part that leaves the steady zone out must not pick its length up from the device either
+  if (static_len == 0) static_len_dev = nullptr;
   return wave_attention_impl(q, steady_k, steady_v, steady_stride, static_len, static_len_dev, store_k, store_v,
                              store_stride, row_src, row_src_stride, nullptr, nullptr, 0, meta, est_ids, logits, nullptr,
                              value_sum, cluster_size_bf16, out, valid_lengths, BG, gs, nc, es, scale, workspace,
@@ -782,7 +784,13 @@ static int static_scratch_ptr(void** out) {
   return RI_OK;
 }
 
-extern "C" size_t ri_wave_attention_static_scratch_bytes(void) { return RI_STATIC_SCRATCH_BYTES; }
+// (also looks the array's address up on the current device, so that a caller who asks for the size before
+// capturing a stream has the first-call work behind it: the look-up can load the code object)
+extern "C" size_t ri_wave_attention_static_scratch_bytes(void) {
+  void* ptr = nullptr;
+  (void)static_scratch_ptr(&ptr);
+  return RI_STATIC_SCRATCH_BYTES;
+}
 
 extern "C" int ri_wave_attention_static(const void* q, const void* steady_k, const void* steady_v,
                                         int64_t steady_stride, int static_len, const int32_t* static_len_dev,
