@@ -222,7 +222,42 @@ def bench_kmeans(cfg, dev, iters=10, reps=3):
                               "frac": flops_as / t_as / MFMA_BF16_PEAK}}
 
 
-def cpu_baseline(cache, cfg, queries, nprobe, es, static_len, max_seconds=10.0, max_samples=100):
+def kmeans_cpu_baseline(cfg, iters=10):
+    """The CPU restatement of the clustering (oracle/kmeans.py) on a bounded sample of the same keys: the nine
+    segmented iterations of ONE 8192-token segment of one head, and the final assignment + update of 8192 of
+    the head's tokens against all its centroids; scaled linearly to one sequence (all heads, all segments, all
+    tokens).  The arithmetic per token and centroid is the same for every segment and head, so the scaling is
+    by counts only."""
+    from oracle import kmeans as okm
+    from retrievalattention_amd import synth
+    torch.set_num_threads(os.cpu_count() or 1)
+    Hkv, N, nc, S = cfg["Hkv"], cfg["N"], cfg["nc"], cfg["S"]
+    nseg, ncs = N // S, nc // S
+    k, _, _ = synth.make_group(0, 0, 0, N, cfg["K"], cfg["gs"], outliers=cfg["outliers"], n_extra=0)
+    k = k.to(torch.bfloat16)
+    k = (k - k.mean(dim=0, keepdim=True)).contiguous()
+    cent = k[okm.init_indices(N, nc)].clone()
+    d, c = k[:nseg], cent[:ncs]
+    t0 = time.time()
+    for _ in range(iters - 1):
+        c, _, _ = okm.train_step(d, c, True)
+    t_seg = time.time() - t0
+    sample = min(N, 8192)
+    t0 = time.time()
+    okm.train_step(k[:sample], cent, False)
+    t_glob = time.time() - t0
+    per_seq = Hkv * (S * t_seg + (N / sample) * t_glob)
+    return {"ms_per_sequence": per_seq * 1e3, "unit": "ms", "cores": torch.get_num_threads(), "kind": "port",
+            "measured_s": {"segment_sweep_9_iterations": t_seg, "final_pass_on_sample_tokens": t_glob},
+            "sample": f"oracle/kmeans.py on head 0 of the same keys: {iters - 1} segmented iterations of one {nseg}-token "
+                      f"segment ({ncs} centroids) and the final pass over {sample} tokens against {nc} centroids, "
+                      f"{t_seg + t_glob:.1f} s of CPU work",
+            "extrapolation": f"{Hkv} heads x ({S} segments x segment sweep + {N // sample} x final-pass sample): linear "
+                             f"in tokens, segments and heads",
+            "note": "the checker's restatement (float64 scores, numpy), not a tuned CPU implementation"}
+
+
+def cpu_baseline(cache, cfg, queries, nprobe, es, static_len, max_seconds=10.0, max_samples=100, min_samples=3):
     """The CPU restatement (oracle/) of the same decode step, layer 0, on the host cores."""
     from oracle import pipeline
     BG, gs = cfg["B"] * cfg["Hkv"], cfg["gs"]
@@ -236,10 +271,11 @@ def cpu_baseline(cache, cfg, queries, nprobe, es, static_len, max_seconds=10.0, 
             cache.value_sum[l].cpu(), cache.centroids_mask[l].cpu(), cache.cluster_size_i32[l].cpu(),
             cache.cluster_size[l].cpu(), sk, sv, cache.cluster_start[l].cpu().long(), nprobe, es, 8,
             cache.buffer_size)
-    pipeline.decode_step(*args)  # warm-up
+    if min_samples > 1:
+        pipeline.decode_step(*args)  # warm-up
     times = []
     t_all = time.time()
-    while len(times) < max_samples and (len(times) < 3 or time.time() - t_all < max_seconds):
+    while len(times) < max_samples and (len(times) < min_samples or time.time() - t_all < max_seconds):
         t0 = time.time()
         ref, _ = pipeline.decode_step(*args)
         times.append(time.time() - t0)
@@ -339,7 +375,7 @@ def bench_end_to_end(args, cfg, dev):
         "roofline": None, "cpu_baseline": None}))
 
 
-def bench_host(args, cfg, cache, queries, L, nprobe, es, static_len):
+def bench_host(args, cfg, cache, queries, L, nprobe, es, static_len, config_name=None, cpu_seconds=10.0):
     """Host-resident clustered K/V: the reference's operator sequence (score+select, id copy to the
     host, block-cache look-up on the worker pool, gather of misses over the host link and hits
     from the device cache, attention, cache admission).  The first pass over the layers runs
@@ -489,21 +525,23 @@ def bench_host(args, cfg, cache, queries, L, nprobe, es, static_len):
         t_attn = stage_us["attention"] * 1e-6
         where = ("ri_wave_attention over the block cache, every block a hit" if cache.block_cache == "device"
                  else "ri_buffer_attention over the assembled execution buffer")
+        traffic, traffic_source = measured_traffic(f"{config_name or args.config}_host")
         roofline = {"bound": "hbm", "kernel": f"attend_kernel ({where})",
                     "achieved": attn_bytes / t_attn / 1e9, "peak": HBM_PEAK / 1e9, "unit": "GB/s",
-                    "frac": attn_bytes / t_attn / HBM_PEAK, "traffic": None,
-                    "traffic_source": "no counter run recorded for the host-resident path",
+                    "frac": attn_bytes / t_attn / HBM_PEAK, "traffic": traffic,
+                    "traffic_source": traffic_source,
                     "launch_us": stage_us["attention"], "algorithmic_bytes": attn_bytes,
                     "note": "event pair around one eager launch (includes its dispatch)"}
     cpu = None
     if not args.no_cpu_baseline:
-        t_cpu, n, ref = cpu_baseline(cache, cfg, queries, nprobe, es, static_len)
+        t_cpu, n, ref = cpu_baseline(cache, cfg, queries, nprobe, es, static_len, max_seconds=cpu_seconds,
+                                     min_samples=3 if cpu_seconds > 0 else 1)
         out0 = step(0)
         torch.cuda.synchronize()
         d = (out0.view(BG, gs, 128).cpu().float() - ref.float()).abs()
         cpu = {"value": B / (cfg["L"] * t_cpu), "unit": "tokens/s", "us_per_layer_step": t_cpu * 1e6,
                "cores": torch.get_num_threads(), "kind": "port",
-               "sample": f"median of {n} full-shape decode layer-steps of layer 0 (oracle/pipeline.py), about 10 s of CPU work",
+               "sample": f"median of {n} full-shape decode layer-steps of layer 0 (oracle/pipeline.py)",
                "note": "the checker's restatement, not a tuned CPU implementation: float64 matrix products and a "
                        "Python loop over the groups",
                "max_abs_vs_gpu": float(d.max()), "mean_abs_vs_gpu": float(d.mean())}
@@ -519,7 +557,8 @@ def bench_host(args, cfg, cache, queries, L, nprobe, es, static_len):
         torch.cuda.synchronize()
         t_copy = min(t_copy, time.perf_counter() - t0)
     link_peak = pin.numel() / t_copy / 1e9
-    print(json.dumps({
+    del pin, dst
+    return ({
         "metric": "decode tokens/s at 128K ctx (attention only, B / (L * t_layer_step)); us/layer-step and % HBM roofline alongside",
         "value": B / (cfg["L"] * t_warm), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": t_warm * 1e3, "us_per_layer_step": t_warm * 1e6, "cold_us_per_layer_step": t_cold * 1e6,
@@ -540,68 +579,34 @@ def bench_host(args, cfg, cache, queries, L, nprobe, es, static_len):
                       "achieved": link, "peak": link_peak, "unit": "GB/s", "frac": link / link_peak if link else None,
                       "note": "achieved = missed K and V bytes per step over the whole step time, best drift level; "
                               "peak = a 256 MiB copy from pinned host memory measured in this run"},
-        "roofline": roofline, "cpu_baseline": cpu}))
+        "roofline": roofline, "cpu_baseline": cpu})
 
 
-def main():
-    ap = argparse.ArgumentParser()
-    ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=640)
-    ap.add_argument("--warmup", type=int, default=64)
-    ap.add_argument("--config", default="c2", choices=sorted(CONFIGS))
-    ap.add_argument("--layers", type=int, default=0, help="distinct layers (default: the config's)")
-    ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--no-graph", action="store_true", help="time eager launches instead of HIP graph replays")
-    ap.add_argument("--residency", default="device", choices=["device", "host"],
-                    help="host: clustered K/V in pinned host memory behind the block cache (staged operator path, "
-                         "eager launches; reports the cold first pass and the warm steady state)")
-    ap.add_argument("--block-cache", default="device", choices=["device", "host"],
-                    help="with --residency host: block cache manager as a kernel (HIP graph replays) or the "
-                         "reference's worker threads (eager launches)")
-    ap.add_argument("--overlap", action="store_true",
-                    help="with --residency host: attend the cached rows while the missed blocks are staged")
-    ap.add_argument("--drift", default="0.5,0.75,1.0",
-                    help="with --residency host: noise levels of the drifting-query measurements (empty: none)")
-    ap.add_argument("--no-kmeans", action="store_true", help="skip the prefill clustering measurement")
-    ap.add_argument("--estimate-next", action="store_true",
-                    help="also measure the step with next-layer cluster estimation (zones of layer l+1 chosen "
-                         "at the end of layer l from a predicted query)")
-    ap.add_argument("--end-to-end", action="store_true",
-                    help="a whole decoded token of a random-weight model of the config's shape (all layers, one "
-                         "HIP graph per token) instead of the attention-only layer-step")
-    ap.add_argument("--repeats", type=int, default=21,
-                    help="repetitions of the timed region of --steps layer-steps; the median is reported")
-    ap.add_argument("--no-read-probe", action="store_true",
-                    help="skip the read-only streaming probe (the measured read ceiling of the part, reported as read_probe)")
-    ap.add_argument("--read-probe", action="store_true", help="kept for older command lines: the probe runs by default")
-    ap.add_argument("--copy-probe", action="store_true",
-                    help="also run 8 device copies of 256 MiB (a known-size kernel to scale rocprofv3 byte counters by)")
-    args = ap.parse_args()
-    if args.gpus != 1:
-        sys.exit("bench.py measures one GPU: the wave-index path has no cross-GPU exchange (run with --gpus 1)")
-    if not torch.cuda.is_available():
-        sys.exit("bench.py needs a GPU")
-    dev = torch.device("cuda:0")
-    torch.cuda.set_device(dev)
-    cfg = CONFIGS[args.config]
-    L = args.layers or cfg["L"]
+def compact(rec):
+    """What an entry of other_configs carries: the step time, both rooflines and the check against the oracle."""
+    out = {k: rec[k] for k in ("us_per_layer_step", "cold_us_per_layer_step", "value", "unit", "step_roofline", "roofline",
+                               "stages_us", "host_link", "drifting_queries") if k in rec}
+    out["workload"] = rec["config"]["workload"]
+    cpu = rec.get("cpu_baseline")
+    if cpu:
+        out["max_abs_vs_oracle"] = cpu["max_abs_vs_gpu"]
+        out["mean_abs_vs_oracle"] = cpu["mean_abs_vs_gpu"]
+        out["cpu_us_per_layer_step"] = cpu["us_per_layer_step"]
+        out["cpu_sample"] = cpu["sample"]
+    if "stages" in rec:
+        out["stages_us"] = {k: v.get("us_in_step", v["us"]) for k, v in rec["stages"].items()}
+    return out
+
+
+def bench_device(args, cfg, config_name, L, dev, extras=True):
+    """The layer-step over a device-resident store for one configuration; returns the record.  extras: the
+    read probe, the prefill clustering, next-layer estimation and the full CPU baseline (the headline
+    configuration); without them only one CPU layer-step is run, for the check against the oracle."""
     B, Hkv, gs = cfg["B"], cfg["Hkv"], cfg["gs"]
     BG = B * Hkv
-    if args.copy_probe:
-        a = torch.empty(256 << 20, dtype=torch.uint8, device=dev).fill_(1)
-        b = torch.empty_like(a)
-        for _ in range(8):
-            b.copy_(a)
-        torch.cuda.synchronize()
-        del a, b
-    if args.end_to_end:
-        return bench_end_to_end(args, cfg, dev)
-    est_next = args.residency == "device" and args.estimate_next and not args.no_graph and L >= 4
-    cache, queries, nprobe, es = build_cache(cfg, L, dev, args.residency, args.block_cache, est_next,
-                                             overlap_miss_staging=args.overlap)
+    est_next = extras and args.estimate_next and not args.no_graph and L >= 4
+    cache, queries, nprobe, es = build_cache(cfg, L, dev, "device", "device", est_next, overlap_miss_staging=False)
     static_len = cache.static_pattern_total  # 4 + 64 + the token being decoded (already counted)
-    if args.residency == "host":
-        return bench_host(args, cfg, cache, queries, L, nprobe, es, static_len)
 
     # every layer-step is "not the last layer" for timing purposes: same static_len everywhere
     def step(l):
@@ -680,14 +685,19 @@ def main():
 
     run_steps(0, max(args.warmup, CL))
     torch.cuda.synchronize()
-    # the timed region (exactly args.steps layer-steps between two synchronisations) is repeated and the
-    # median repetition reported: a short region is a single graph replay, one sample of which says little
+    # the timed region (args.steps layer-steps between two synchronisations) is repeated and the median
+    # repetition reported.  A region shorter than one graph of CL steps is a single graph replay of about a
+    # millisecond, of which the launch from the host and the synchronisation are a visible part (about 1 us per
+    # layer-step at 20 steps): such a region replays its graph `inner` times back to back, and the time is
+    # divided by all the layer-steps it ran
+    inner = max(1, 320 // args.steps) if (graphs is not None and args.steps < CL) else 1
     reps_t = []
     for _ in range(max(args.repeats, 1)):
         t0 = time.perf_counter()
-        run_steps(0, args.steps)
+        for _ in range(inner):
+            run_steps(0, args.steps)
         torch.cuda.synchronize()
-        reps_t.append((time.perf_counter() - t0) / args.steps)
+        reps_t.append((time.perf_counter() - t0) / (args.steps * inner))
     reps_t.sort()
     t_step = reps_t[len(reps_t) // 2]
 
@@ -762,9 +772,10 @@ def main():
         "value": tokens_per_s, "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": t_step * 1e3, "us_per_layer_step": t_step * 1e6, "higher_is_better": True,
         "timed_region": {"repeats": len(reps_t), "statistic": "median", "min_us_per_layer_step": reps_t[0] * 1e6,
-                         "max_us_per_layer_step": reps_t[-1] * 1e6},
+                         "max_us_per_layer_step": reps_t[-1] * 1e6, "layer_steps_per_region": args.steps * inner,
+                         "replays_of_the_steps_per_region": inner},
         "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
-        "config": {"workload": f"{args.config}: {cfg['desc']}; nprobe {nprobe}, estimation zone {es}, "
+        "config": {"workload": f"{config_name}: {cfg['desc']}; nprobe {nprobe}, estimation zone {es}, "
                                f"steady zone {static_len}, {L} layers with independent seeds (seeded Gaussian-mixture "
                                f"K/V drawn by torch's generator on the device), "
                                f"{'HIP graph replay (32 layer-steps per graph)' if graphs is not None else 'eager launches'}",
@@ -784,7 +795,7 @@ def main():
     # without it); an event pair around one eager launch also counts the dispatch of the launch
     # (eager_event_us; null_launch_us is what the same pair reads around an empty kernel).
     t_dom = t_attn_in_step if t_attn_in_step else t_attn
-    traffic, traffic_source = measured_traffic(args.config)
+    traffic, traffic_source = measured_traffic(config_name)
     result["roofline"] = {"bound": "hbm", "kernel": "attend_kernel (ri_wave_attention)",
                           "achieved": attn_bytes / t_dom / 1e9, "peak": HBM_PEAK / 1e9, "unit": "GB/s",
                           "frac": attn_bytes / t_dom / HBM_PEAK, "traffic": traffic, "traffic_source": traffic_source,
@@ -796,19 +807,113 @@ def main():
         result["stages"]["wave_attention"]["us_in_step"] = t_attn_in_step * 1e6
     if est_next:
         result["next_layer_estimation"] = bench_estimate_next(args, cache, queries, outs, L, static_len)
-    if not args.no_read_probe:
+    if extras and not args.no_read_probe:
         result["read_probe"] = read_probe(dev)
-    if not args.no_kmeans:
-        result["prefill_kmeans"] = bench_kmeans(cfg, dev)
     if not args.no_cpu_baseline:
-        t_cpu, n, ref = cpu_baseline(cache, cfg, queries, nprobe, es, static_len)
+        t_cpu, n, ref = cpu_baseline(cache, cfg, queries, nprobe, es, static_len, max_seconds=10.0 if extras else 0.0,
+                                     min_samples=3 if extras else 1)
         d = (outs[0].view(BG, gs, 128).cpu().float() - ref.float()).abs()
         result["cpu_baseline"] = {"value": B / (Lmodel * t_cpu), "unit": "tokens/s", "us_per_layer_step": t_cpu * 1e6,
                                   "cores": torch.get_num_threads(), "kind": "port",
-                                  "sample": f"median of {n} full-shape decode layer-steps of layer 0 (oracle/pipeline.py), about 10 s of CPU work",
+                                  "sample": f"median of {n} full-shape decode layer-steps of layer 0 (oracle/pipeline.py)" +
+                                            (", about 10 s of CPU work" if extras else ""),
                                   "note": "the checker's restatement, not a tuned CPU implementation: float64 matrix "
                                           "products and a Python loop over the groups",
                                   "max_abs_vs_gpu": float(d.max()), "mean_abs_vs_gpu": float(d.mean())}
+    return result
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=640)
+    ap.add_argument("--warmup", type=int, default=64)
+    ap.add_argument("--config", default="c2", choices=sorted(CONFIGS))
+    ap.add_argument("--layers", type=int, default=0, help="distinct layers (default: the config's)")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-graph", action="store_true", help="time eager launches instead of HIP graph replays")
+    ap.add_argument("--residency", default="device", choices=["device", "host"],
+                    help="host: clustered K/V in pinned host memory behind the block cache (staged operator path, "
+                         "eager launches; reports the cold first pass and the warm steady state)")
+    ap.add_argument("--block-cache", default="device", choices=["device", "host"],
+                    help="with --residency host: block cache manager as a kernel (HIP graph replays) or the "
+                         "reference's worker threads (eager launches)")
+    ap.add_argument("--overlap", action="store_true",
+                    help="with --residency host: attend the cached rows while the missed blocks are staged")
+    ap.add_argument("--drift", default="0.5,0.75,1.0",
+                    help="with --residency host: noise levels of the drifting-query measurements (empty: none)")
+    ap.add_argument("--no-kmeans", action="store_true", help="skip the prefill clustering measurement")
+    ap.add_argument("--estimate-next", action="store_true",
+                    help="also measure the step with next-layer cluster estimation (zones of layer l+1 chosen "
+                         "at the end of layer l from a predicted query)")
+    ap.add_argument("--end-to-end", action="store_true",
+                    help="a whole decoded token of a random-weight model of the config's shape (all layers, one "
+                         "HIP graph per token) instead of the attention-only layer-step")
+    ap.add_argument("--repeats", type=int, default=21,
+                    help="repetitions of the timed region of --steps layer-steps; the median is reported")
+    ap.add_argument("--no-read-probe", action="store_true",
+                    help="skip the read-only streaming probe (the measured read ceiling of the part, reported as read_probe)")
+    ap.add_argument("--read-probe", action="store_true", help="kept for older command lines: the probe runs by default")
+    ap.add_argument("--no-other-configs", action="store_true",
+                    help="with the default configuration: skip the short runs of c1, c5 and c4 (host-resident) that are "
+                         "reported as other_configs")
+    ap.add_argument("--copy-probe", action="store_true",
+                    help="also run 8 device copies of 256 MiB (a known-size kernel to scale rocprofv3 byte counters by)")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py measures one GPU: the wave-index path has no cross-GPU exchange (run with --gpus 1)")
+    if not torch.cuda.is_available():
+        sys.exit("bench.py needs a GPU")
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    cfg = CONFIGS[args.config]
+    L = args.layers or cfg["L"]
+    B, Hkv, gs = cfg["B"], cfg["Hkv"], cfg["gs"]
+    BG = B * Hkv
+    if args.copy_probe:
+        a = torch.empty(256 << 20, dtype=torch.uint8, device=dev).fill_(1)
+        b = torch.empty_like(a)
+        for _ in range(8):
+            b.copy_(a)
+        torch.cuda.synchronize()
+        del a, b
+    if args.end_to_end:
+        return bench_end_to_end(args, cfg, dev)
+    if args.residency == "host":
+        cache, queries, nprobe, es = build_cache(cfg, L, dev, "host", args.block_cache, False,
+                                                 overlap_miss_staging=args.overlap)
+        print(json.dumps(bench_host(args, cfg, cache, queries, L, nprobe, es, cache.static_pattern_total)))
+        return
+    result = bench_device(args, cfg, args.config, L, dev, extras=True)
+    torch.cuda.empty_cache()      # the cache and its graphs went with the function's locals
+    if not args.no_kmeans:
+        km = bench_kmeans(cfg, dev)
+        if not args.no_cpu_baseline:
+            km["cpu_baseline"] = kmeans_cpu_baseline(cfg)
+            km["cpu_baseline"]["cpu_over_gpu"] = km["cpu_baseline"]["ms_per_sequence"] / km["ms_per_sequence"]
+        result["prefill_kmeans"] = km
+        from retrievalattention_amd import kernels
+        kernels.release_cached_graphs(retired_workspaces=False)
+        torch.cuda.empty_cache()
+    if args.config == "c2" and not args.no_other_configs:
+        # the other named configurations, each on a short run of its own (the c2 cache is gone by now)
+        import copy
+        others = {}
+        sub = copy.copy(args)
+        sub.steps, sub.warmup, sub.repeats, sub.estimate_next = min(args.steps, 128), min(args.warmup, 32), 7, False
+        sub.drift, sub.no_graph = "0.75", False
+        for name, cname, Ls in (("c1", "c1", 8), ("c5", "c5", 2)):
+            log(f"[bench] other config {name}")
+            others[name] = compact(bench_device(sub, CONFIGS[cname], cname, Ls, dev, extras=False))
+            torch.cuda.empty_cache()
+        log("[bench] other config c4_host")
+        c4 = CONFIGS["c4"]
+        cache, queries, nprobe, es = build_cache(c4, 2, dev, "host", "device", False, overlap_miss_staging=False)
+        others["c4_host"] = compact(bench_host(sub, c4, cache, queries, 2, nprobe, es, cache.static_pattern_total,
+                                               config_name="c4", cpu_seconds=0.0))
+        del cache, queries
+        torch.cuda.empty_cache()
+        result["other_configs"] = others
     print(json.dumps(result))
 
 

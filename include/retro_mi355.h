@@ -137,6 +137,12 @@ int ri_score_logits(const void* q, const void* centroids, float* logits, int BG,
  *   every call leaves at zero again); calls sharing a workspace must not overlap in time.
  *   BG <= 4096. */
 size_t ri_flash_decoding_workspace_bytes(int BG, int gs);
+/* Clears the arrival counters at the head of an attention workspace (of ri_weighted_flash_decoding,
+ * ri_wave_attention, ri_wave_attention_part or ri_buffer_attention) with a small kernel on `stream`; no
+ * memset, so the call can be captured.  Every attention call leaves the counters at zero; this is for the
+ * case that a launch did not run to its end (device fault or reset): counters left non-zero would make
+ * every later call on that workspace write no output.  No counterpart in the reference. */
+int ri_attention_workspace_reset(void* workspace, size_t workspace_bytes, ri_stream_t stream);
 int ri_weighted_flash_decoding(const void* q, const void* k, const void* v, const void* weight,
                                const int32_t* cache_seqlens, const void* prev_out,
                                const float* prev_lse, void* out, float* lse_out, int BG,

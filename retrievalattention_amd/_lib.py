@@ -23,6 +23,7 @@ SIGNATURES = {
     "ri_score_select": (I, [P] * 13 + [I, P, I, I, I, I, I, I, I, F, P, SZ, P]),
     "ri_score_logits": (I, [P, P, P, I, I, I, F, P, SZ, P]),
     "ri_flash_decoding_workspace_bytes": (SZ, [I, I]),
+    "ri_attention_workspace_reset": (I, [P, SZ, P]),
     "ri_weighted_flash_decoding": (I, [P, P, P, P, P, P, P, P, P, I, I, I, I64, F, P, SZ, P]),
     "ri_wave_attention_workspace_bytes": (SZ, [I, I]),
     "ri_wave_attention": (I, [P, P, P, I64, I, P, P, P, I64, P, I, P, P, I, P, P, P, P, P, P, P, P, I, I, I, I, F, P, SZ, P]),

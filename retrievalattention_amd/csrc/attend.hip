@@ -713,6 +713,19 @@ static int wave_attention_impl(const void* q, const void* steady_k, const void* 
   return launch_attend(P, BG, gs, nw, stream);
 }
 
+// Clears the arrival counters at the head of an attention workspace with a small kernel on `stream` (no
+// memset: the call can be captured).  Every attention launch leaves its counters at zero, so this is only
+// needed after a launch that did not run to its end (a fault, a device reset): its groups' counters may be
+// left non-zero, and later launches on that workspace would then never see a last arrival and write nothing.
+extern "C" int ri_attention_workspace_reset(void* workspace, size_t workspace_bytes, ri_stream_t stream) {
+  if (!workspace || ri_misaligned16(workspace)) return RI_ERR_ARG;
+  if (workspace_bytes < RI_MAX_GROUPS * sizeof(int)) return RI_ERR_WORKSPACE;
+  attend_clear_counters_kernel<<<(RI_MAX_GROUPS + 255) / 256, 256, 0, (hipStream_t)stream>>>((int*)workspace,
+                                                                                             RI_MAX_GROUPS);
+  RI_HIP_CHECK_LAUNCH();
+  return RI_OK;
+}
+
 extern "C" int ri_wave_attention(const void* q, const void* steady_k, const void* steady_v,
                                  int64_t steady_stride, int static_len, const int32_t* static_len_dev,
                                  const void* store_k,

@@ -91,6 +91,15 @@ def _workspace(nbytes, device, tag):
     return w
 
 
+def reset_attention_workspaces():
+    """Clears the arrival counters of every attention scratch tensor (on the current stream of its device).
+    The attention launches leave them at zero; call this after a launch that did not run to its end."""
+    for (dev, tag), w in _workspaces.items():
+        if tag.startswith("attn"):
+            with torch.cuda.device(w.device):
+                check(lib().ri_attention_workspace_reset(_p(w), w.numel(), _stream()), "attention_workspace_reset")
+
+
 def release_cached_graphs(retired_workspaces=True):
     """Drops what the library keeps alive for replays: the captured clusterings of segment_k_means_csr (only the
     library replays those, so this is always safe) and, with retired_workspaces, the scratch tensors that were

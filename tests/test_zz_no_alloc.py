@@ -88,3 +88,82 @@ def test_static_scratch_rejects_shapes_beyond_its_array(dev):
     rc = lib.ri_wave_attention_static(p, p, p, 1, 1, None, p, p, 1, None, 0, p, p, 1, p, None, None, None, None, None, p,
                                       None, BG, gs, 32, 0, 1.0, None)
     assert rc == -3 and b"workspace" in lib.ri_status_string(rc)
+
+
+def _static_call(lib, d, out, vl, BG, gs, nc, nprobe, es, stream, static_len=71):
+    p = lambda t: None if t is None else C.c_void_p(t.data_ptr())
+    rc = lib.ri_wave_attention_static(
+        p(d["q"]), p(d["stk"]), p(d["stv"]), 80, static_len, None, p(d["sk"]), p(d["sv"]), d["rows"], None, 0, p(d["rto"]),
+        p(d["rst"]), nprobe, p(d["meta"]), p(d["est"]) if es else None, p(d["logits"]) if es else None, None, p(d["vsum"]),
+        p(d["csz"]), p(out), p(vl), BG, gs, nc, es, 1 / math.sqrt(128), C.c_void_p(stream))
+    assert rc == 0, lib.ri_status_string(rc)
+
+
+def test_static_scratch_calls_allocate_nothing_and_replay_from_a_graph(dev):
+    """What the entry point is for.  (1) After one warm-up call, further calls leave the device's free memory and
+    torch's allocator untouched: no hipMalloc behind the call.  (2) A call captured into a HIP graph (after the
+    scratch size was asked for, which resolves the array's address outside the capture) replays to the same
+    bits as the workspace entry point, several times, with eager calls on the same array in between."""
+    from retrievalattention_amd import _lib
+    lib = _lib.lib()
+    BG, gs, nc, N, nprobe, es = 8, 4, 512, 8192, 9, 118
+    d = _case(dev, BG, gs, nc, N, nprobe, es, seed=51)
+    ref, vl_ref = _attend(dev, d, BG, gs, nc, nprobe, es, static=False)
+    out = torch.zeros(BG, gs, 128, dtype=torch.bfloat16, device=dev)
+    vl = torch.zeros(BG, dtype=torch.int32, device=dev)
+    assert lib.ri_wave_attention_static_scratch_bytes() == 8 << 20
+    stream = torch.cuda.current_stream().cuda_stream
+    _static_call(lib, d, out, vl, BG, gs, nc, nprobe, es, stream)      # warm-up: code object loaded, address known
+    torch.cuda.synchronize()
+    free0, alloc0, reserved0 = torch.cuda.mem_get_info()[0], torch.cuda.memory_allocated(), torch.cuda.memory_reserved()
+    for _ in range(5):
+        _static_call(lib, d, out, vl, BG, gs, nc, nprobe, es, stream)
+    torch.cuda.synchronize()
+    assert torch.cuda.mem_get_info()[0] == free0
+    assert torch.cuda.memory_allocated() == alloc0 and torch.cuda.memory_reserved() == reserved0
+    assert torch.equal(out.cpu().view(torch.int16), ref.view(torch.int16))
+    # captured and replayed
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        _static_call(lib, d, out, vl, BG, gs, nc, nprobe, es, side.cuda_stream)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        _static_call(lib, d, out, vl, BG, gs, nc, nprobe, es, torch.cuda.current_stream().cuda_stream)
+    small = _case(dev, 3, 7, 256, 3000, 5, 0, seed=52)
+    for rep in range(4):
+        out.zero_(); vl.zero_()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out.cpu().view(torch.int16), ref.view(torch.int16)), f"replay {rep}"
+        assert torch.equal(vl.cpu(), vl_ref)
+        _attend(dev, small, 3, 7, 256, 5, 0, static=True)       # eager work on the same array between replays
+
+
+def test_workspace_reset_recovers_poisoned_counters(dev):
+    """Counters left non-zero (as by a launch that never finished) are cleared by ri_attention_workspace_reset;
+    the next call on that workspace is then correct again."""
+    from retrievalattention_amd import _lib
+    lib = _lib.lib()
+    BG, gs, nc, N, nprobe, es = 4, 4, 256, 4096, 6, 40
+    d = _case(dev, BG, gs, nc, N, nprobe, es, seed=53)
+    ref, _ = _attend(dev, d, BG, gs, nc, nprobe, es, static=False)
+    p = lambda t: None if t is None else C.c_void_p(t.data_ptr())
+    nb = lib.ri_wave_attention_workspace_bytes(BG, gs)
+    ws = torch.zeros(nb, dtype=torch.uint8, device=dev)
+    ws.view(torch.int32)[:BG] = 3                      # stale arrivals
+    stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    assert lib.ri_attention_workspace_reset(p(ws), nb, stream) == 0
+    out = torch.zeros(BG, gs, 128, dtype=torch.bfloat16, device=dev)
+    vl = torch.zeros(BG, dtype=torch.int32, device=dev)
+    rc = lib.ri_wave_attention(p(d["q"]), p(d["stk"]), p(d["stv"]), 80, 71, None, p(d["sk"]), p(d["sv"]), d["rows"], None, 0,
+                               p(d["rto"]), p(d["rst"]), nprobe, p(d["meta"]), p(d["est"]), p(d["logits"]), None,
+                               p(d["vsum"]), p(d["csz"]), p(out), p(vl), BG, gs, nc, es, 1 / math.sqrt(128), p(ws), nb,
+                               stream)
+    assert rc == 0
+    torch.cuda.synchronize()
+    assert torch.equal(out.cpu().view(torch.int16), ref.view(torch.int16))
+    assert bool((ws.view(torch.int32)[:BG] == 0).all())
+    assert lib.ri_attention_workspace_reset(p(ws), 64, stream) == -3
