@@ -40,7 +40,7 @@ class retroinfer_cache(KV_Cache):
                  n_centroids, n_segment, nprobe, max_compute_cluster_num, cache_unit_size, cache_cluster_num,
                  num_gpus, model_size, use_cluster_estimation=False, kv_residency="auto",
                  block_cache="device", device_positions=False, overlap_miss_staging=False, pin_workers=False,
-                 profiler_ranges=False):
+                 profiler_ranges=False, reference_stale_row=False):
         super().__init__(layer_num, batch_size, max_length, num_key_value_heads, num_heads, head_dim, dtype,
                          layer_mapping, num_gpus, model_size)
         if head_dim != 128 or dtype != torch.bfloat16:
@@ -88,6 +88,9 @@ class retroinfer_cache(KV_Cache):
         # the reference's NVTX ranges (retroinfer_cache.py:558-678) as roctx ranges of the same names
         self.profiler_ranges = bool(profiler_ranges)
         self.pin_workers = bool(pin_workers)
+        # worker-thread manager with next-layer estimation only: leave the layer's new token out of the
+        # pre-assembled execution buffer, as the reference does (its attention then reads the stale row there)
+        self.reference_stale_row = bool(reference_stale_row)
 
         self.input_length = self.max_length - max_new_length
         self.max_new_length = min(max_new_length - 1, THRESHOLD_LENGTH)  # one token comes out of prefill
@@ -743,11 +746,12 @@ class retroinfer_cache(KV_Cache):
             # against :541-542, whose attention then sees a stale row there): the token's row is brought in now,
             # so that every residency attends the same rows
             torch.cuda.current_stream().wait_stream(self.copystream)
-            BGd = (BG, -1, D)
-            self.execution_buffer_keys[buf][:, static_len - 1, 0] = \
-                self.steady_zone_keys[layer_idx].view(BGd)[:, static_len - 1]
-            self.execution_buffer_values[buf][:, static_len - 1, 0] = \
-                self.steady_zone_values[layer_idx].view(BGd)[:, static_len - 1]
+            if not self.reference_stale_row:
+                BGd = (BG, -1, D)
+                self.execution_buffer_keys[buf][:, static_len - 1, 0] = \
+                    self.steady_zone_keys[layer_idx].view(BGd)[:, static_len - 1]
+                self.execution_buffer_values[buf][:, static_len - 1, 0] = \
+                    self.steady_zone_values[layer_idx].view(BGd)[:, static_len - 1]
         if fuse_est:
             attn = torch.empty((BG, gs, D), dtype=self.dtype, device=queries.device)
             kernels.buffer_attention(

@@ -380,6 +380,59 @@ def test_next_layer_cluster_estimation(dev, residency):
 
 
 
+def test_reference_stale_row_switch(dev):
+    """reference_stale_row=True (worker-thread manager with next-layer estimation) reproduces the reference's
+    arithmetic: from the third layer on the execution buffer was assembled during the previous layer, before the
+    layer's new token was appended (retroinfer_cache.py:644-652 against :541-542), so the attention reads the
+    row as it was then (zeros for the first generated token) instead of the token's K/V.  Checked against the
+    oracle fed that stale row; without the switch the same layers match the oracle fed the real row."""
+    from retrievalattention_amd.cache_hub import retroinfer_cache
+    layers, B, Hkv, gs, ctx = 4, 1, 2, 4, 2048 + 68
+    nc, nprobe, es = 128, 6, 30
+    K, V = _gen(layers, B, Hkv, gs, ctx, 128, dev, 21)
+    BG = B * Hkv
+    outs = {}
+    for stale in (False, True):
+        cache = retroinfer_cache(
+            valid_start=[0] * B, layer_num=layers, batch_size=B, max_length=ctx + 8, num_key_value_heads=Hkv,
+            num_heads=Hkv * gs, head_dim=128, dtype=torch.bfloat16, layer_mapping={str(l): "cuda:0" for l in range(layers)},
+            max_new_length=8, static_pattern_start=4, static_pattern_end=64, core=4, n_centroids=nc, n_segment=1,
+            nprobe=nprobe, max_compute_cluster_num=nprobe + es, cache_unit_size=8, cache_cluster_num=3 * nprobe,
+            num_gpus=1, model_size=8, use_cluster_estimation=True, kv_residency="host", block_cache="host",
+            reference_stale_row=stale)
+        _prefill(cache, K, V, layers, B)
+        g = torch.Generator().manual_seed(22)
+        q = [torch.randn(B, 1, Hkv * gs, 128, generator=g).to(torch.bfloat16) for _ in range(layers)]
+        for l in range(layers):
+            kn = (4 * torch.randn(B, 1, Hkv, 128, generator=g)).to(torch.bfloat16)   # a key that matters
+            vn = (4 * torch.randn(B, 1, Hkv, 128, generator=g)).to(torch.bfloat16)
+            cache.decode_update_kv_cache(kn.to(dev), vn.to(dev), l)
+            out = cache.compute(q[l].to(dev), l, q[l + 1].to(dev) if l + 1 < layers else None)
+            torch.cuda.synchronize()
+            static_len = cache.static_pattern_total if l == layers - 1 else cache.static_pattern_total + 1
+            size_bf = cache.cluster_size[l].cpu()
+            size_i = size_bf.float().to(torch.int32)
+            rows = size_i.sum(1)
+            lk, lv = cache.list_keys[l].view(BG, -1, 128), cache.list_values[l].view(BG, -1, 128)
+            sk = [lk[gi, :int(rows[gi])].clone() for gi in range(BG)]
+            sv = [lv[gi, :int(rows[gi])].clone() for gi in range(BG)]
+            stk = cache.steady_zone_keys[l].view(BG, -1, 128).cpu().clone()
+            stv = cache.steady_zone_values[l].view(BG, -1, 128).cpu().clone()
+            if stale and l >= 2:
+                stk[:, static_len - 1] = 0
+                stv[:, static_len - 1] = 0
+            ref, _ = pipeline.decode_step(
+                q[l].view(BG, gs, 128), stk, stv, static_len, cache.centroids[l].cpu(), cache.value_sum[l].cpu(),
+                cache.centroids_mask[l].cpu(), size_i, size_bf, sk, sv, torch.cumsum(size_i.long(), 1) - size_i.long(),
+                nprobe, es, 8, cache.buffer_size)
+            _close(out.cpu().view(BG, gs, 128), ref)
+            outs[(stale, l)] = out.cpu().float()
+        del cache
+    # the switch changes something from the third layer on, and nothing before
+    assert torch.equal(outs[(False, 0)], outs[(True, 0)]) and torch.equal(outs[(False, 1)], outs[(True, 1)])
+    assert float((outs[(False, 2)] - outs[(True, 2)]).abs().max()) > 1e-2
+
+
 @pytest.mark.parametrize("residency", ["device", "host", "host-cpu", "device-pos"])
 def test_index_growth_after_1024_generated_tokens(dev, residency):
     """Decode-time index update (reference: retroinfer_cache.py:462-546): once the steady zone holds
