@@ -175,7 +175,13 @@ __global__ __launch_bounds__(64 * NW, GS_PAD == 16 ? 1 : 3) void attend_kernel(A
   __shared__ float sh_al[NW][16];
   __shared__ float sh_m[NW][GS_PAD];
   __shared__ float sh_l[NW][GS_PAD];
-  __shared__ float sh_acc[NW][GS_PAD][RI_DIM];
+  // the waves' numerators for the merge: up to eight heads they are laid over the wave's own value tile (dead
+  // once its rows are done), which keeps a four-wave workgroup under 40 KB of LDS (four per compute unit)
+  constexpr bool ACC_OVER_VT = GS_PAD * RI_DIM * sizeof(float) <= 16 * ATT_VT_STRIDE * sizeof(uint16_t);
+  __shared__ float sh_acc_own[ACC_OVER_VT ? 1 : NW][ACC_OVER_VT ? 1 : GS_PAD][RI_DIM];
+  auto acc_of = [&](int w) -> float* {
+    return ACC_OVER_VT ? reinterpret_cast<float*>(sh_vt[w]) : &sh_acc_own[ACC_OVER_VT ? 0 : w][0][0];
+  };
   __shared__ __attribute__((aligned(16))) uint16_t sh_q[GS_PAD][RI_DIM];
   __shared__ int sh_desc[NW][ATT_DESC_MAX];
   __shared__ float sh_w[NW][ATT_DESC_MAX];
@@ -442,7 +448,7 @@ __global__ __launch_bounds__(64 * NW, GS_PAD == 16 ? 1 : 3) void attend_kernel(A
     const int head = 4 * h + i;
     if (head < GS_PAD) {
 #pragma unroll
-      for (int dt = 0; dt < 8; ++dt) sh_acc[wave][head][16 * dt + n] = st.acc[dt][i];
+      for (int dt = 0; dt < 8; ++dt) acc_of(wave)[head * RI_DIM + 16 * dt + n] = st.acc[dt][i];
     }
   }
   __syncthreads();
@@ -458,7 +464,7 @@ __global__ __launch_bounds__(64 * NW, GS_PAD == 16 ? 1 : 3) void attend_kernel(A
 #pragma unroll
     for (int w = 0; w < NW; ++w) {
       const float f = (sh_m[w][j] == -INFINITY) ? 0.f : __expf(sh_m[w][j] - M);
-      a += sh_acc[w][j][d] * f;
+      a += acc_of(w)[j * RI_DIM + d] * f;
       l += sh_l[w][j] * f;
     }
     const size_t o = ((size_t)g * S + split) * GS_PAD + j;
