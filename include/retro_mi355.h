@@ -43,7 +43,7 @@ enum {
 const char* ri_status_string(int status);
 int ri_last_hip_error(void);
 /* ABI version: bumped when a signature changes. */
-int ri_abi_version(void);   /* 5 */
+int ri_abi_version(void);   /* 6 */
 /* Launches an empty kernel on `stream`: lets a caller measure the per-dispatch overhead that
  * event timings of back-to-back launches include.  No counterpart in the reference. */
 int ri_null_launch(ri_stream_t stream);
@@ -331,7 +331,8 @@ int ri_kmeans_value_sum(const void* values, const int32_t* counts, const int32_t
  *   sizes, starts [BG, meta_stride] int32: tokens and first host-store row of every cluster
  *   blk_off [BG, blk_off_stride] int32: exclusive prefix of ceil(size / block), ncl + 1 entries
  * State, all device memory owned by the caller and only touched by this call:
- *   stamp [BG, stamp_stride] int32 (zero-initialised: nothing resident), blk_ids
+ *   stamp [BG, stamp_stride] int32 (zero-initialised: nothing resident; else the step that last touched the
+ *   cluster), order [BG, stamp_stride] int32 (the cluster's position inside that step, any initial content), blk_ids
  *   [BG, blk_ids_stride] int32 (cache block ids of resident clusters at blk_off),
  *   free_list [BG, capacity] int32 (initialised 0..capacity-1), free_count [BG] (= capacity),
  *   epoch [BG] (= 0).
@@ -340,8 +341,11 @@ int ri_kmeans_value_sum(const void* values, const int32_t* counts, const int32_t
  * size, token offset), update (execution-buffer token offset, size, cache block id).
  * Policy: the walk over the ranks stops at the first cluster whose blocks do not fit
  * buffer_size; the longest prefix of the misses that fits `capacity` is admitted; victims are
- * whole clusters, least recently touched step first, ascending id inside a step, never one
- * touched in this call.  np <= 4096, ncl <= 65536.  capacity may be 0 (no block cache, as
+ * whole clusters from the least recently used end of the reference's list until the admission is covered
+ * (wave_buffer_cpu.cpp:140-142).  The list is kept as (step, order inside the step) per cluster: the hits of a
+ * call are touched in reverse rank order and the admitted misses pushed in rank order behind them
+ * (:106-114, :170-176), so the hit / miss / admission lists and the evictions are those of the reference's
+ * manager; block id values are the manager's own (the reference's come from an unordered_set).  np <= 4096, ncl <= 65536.  capacity may be 0 (no block cache, as
  * throughput_eval/test.py:77 runs the reference): every kept cluster is then a miss at every call and
  * nothing is admitted (wave_buffer_cpu.cpp:119-130 with a capacity of 0); free_list may then be NULL.
  * With row_src [BG, row_src_stride] and meta [BG, 4] (both or neither): for attention in place over
@@ -351,7 +355,7 @@ int ri_kmeans_value_sum(const void* values, const int32_t* counts, const int32_t
  * ri_score_select writes it, and the hit count is reported as 0 (nothing to copy). */
 int ri_lru_access_update(const int32_t* ret_ids, const int32_t* sizes, const int32_t* starts,
                          int meta_stride, const int32_t* blk_off, int blk_off_stride, int32_t* stamp,
-                         int stamp_stride, int32_t* blk_ids, int blk_ids_stride, int32_t* free_list,
+                         int32_t* order, int stamp_stride, int32_t* blk_ids, int blk_ids_stride, int32_t* free_list,
                          int32_t* free_count, int32_t* epoch, int32_t* hit_ids, int32_t* hit_sizes,
                          int32_t* hit_cumsum, int32_t* hit_num, int32_t* miss_ids,
                          int32_t* miss_sizes, int32_t* miss_cumsum, int32_t* miss_num,

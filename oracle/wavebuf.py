@@ -6,7 +6,7 @@ update); the copy functions are the loop oracles of
 library/retroinfer/test/test_gather_copy.py (:110-127, :190-194, :233-237).
 Block ids: the reference takes them from an unordered_set (iteration order unspecified,
 :153-156); this model hands out the lowest free id last released first, like the library.
-DeviceLruModel restates the policy of the device-side manager, which is this build's own.
+DeviceLruModel restates the device-side manager: the same policy, kept as (step, order in step) pairs.
 """
 import torch
 
@@ -86,13 +86,16 @@ class LruModel:
 
 
 class DeviceLruModel:
-    """The block cache policy of the device-side manager (csrc/lru.hip), one group, plain Python.
-    Same access walk and admission prefix as LruModel; recency is the number of the last step that
-    touched a cluster; victims are whole clusters, oldest step first (ages of 255 steps and more
-    count alike), ascending id inside the boundary age, never one touched in the current step, and
-    an admission the victims cannot cover is cut short.  Freed ids are appended to the free list
-    in ascending cluster id; admitted clusters take ids off the end of the list in rank order."""
-    AGES = 256
+    """The device-side manager (csrc/lru.hip), one group, plain Python: the reference's policy (LruModel) with
+    the manager's own bookkeeping.  Recency is a pair per resident cluster instead of a linked list: the number
+    of the last step that touched it and its order inside that step, which reproduces the list of
+    wave_buffer_cpu.cpp:106-114 and :170-176 (hits are moved to the front in reverse rank order, then the
+    admitted misses are pushed in rank order): inside a step the admitted misses are more recent than the hits,
+    later-ranked misses more recent than earlier ones, earlier-ranked hits more recent than later ones.
+    Victims are taken from the least recent end until the request is covered, hits of the current step included
+    (:140-142).  Freed block ids are appended to the free list in ascending cluster id; admitted clusters take
+    ids off the end of the list in rank order (block id VALUES are the manager's own: the reference takes them
+    from an unordered_set)."""
 
     def __init__(self, sizes, block, capacity, buffer_size, stage_row0=None):
         self.block, self.capacity, self.buffer_size = block, capacity, buffer_size
@@ -104,7 +107,8 @@ class DeviceLruModel:
             self.start.append(row)
             row += s_
         self.nblk = [(s_ + block - 1) // block for s_ in self.sizes]
-        self.stamp = [0] * len(self.sizes)
+        self.stamp = [0] * len(self.sizes)     # 0: not resident, else the step of the last touch
+        self.sub = [0] * len(self.sizes)       # order inside that step (larger = more recent)
         self.blocks = {}                       # resident cluster -> block ids
         self.free = list(range(capacity))
         self.epoch = 0
@@ -140,8 +144,9 @@ class DeviceLruModel:
                 row = self.start[c]
                 for sz in self._blocks(c):
                     miss.append((row, sz, ms)); ms += sz; row += self.block
-        for c in hits:
+        for i, c in enumerate(hits):
             self.stamp[c] = E
+            self.sub[c] = len(hits) - 1 - i
         admit, need = [], 0
         for c, off in misses:
             if need + self.nblk[c] > self.capacity:
@@ -149,36 +154,24 @@ class DeviceLruModel:
             need += self.nblk[c]; admit.append((c, off))
         to_free = need - len(self.free)
         if to_free > 0:
-            age = lambda c: min(E - self.stamp[c], self.AGES - 1)
-            cand = [c for c in range(len(self.sizes)) if self.stamp[c] not in (0, E)]
-            hist = [0] * self.AGES
-            for c in cand:
-                hist[age(c)] += self.nblk[c]
-            acc, cut = 0, -1
-            for a in range(self.AGES - 1, 0, -1):
-                if acc + hist[a] >= to_free:
-                    cut = a
+            order = sorted(self.blocks, key=lambda c: (self.stamp[c], self.sub[c]))   # least recent first
+            victims, got = [], 0
+            for c in order:
+                if got >= to_free:
                     break
-                acc += hist[a]
-            rem, run = to_free - acc, 0
-            for c in cand:                      # ascending id
-                out = cut < 0 or age(c) > cut
-                if age(c) == cut:
-                    out = run < rem
-                    run += self.nblk[c]
-                if out:
-                    self.free.extend(self.blocks.pop(c))
-                    self.stamp[c] = 0
+                victims.append(c); got += self.nblk[c]
+            for c in sorted(victims):
+                self.free.extend(self.blocks.pop(c))
+                self.stamp[c] = 0
         F = len(self.free)
         upd, taken = [], 0
-        for c, off in admit:
-            if taken + self.nblk[c] > F:
-                break
-            ids_c = [self.free[F - 1 - (taken + j)] for j in range(self.nblk[c])]
-            for j, (b, sz) in enumerate(zip(ids_c, self._blocks(c))):
-                upd.append((b, sz, off + j * self.block))
+        for j, (c, off) in enumerate(admit):
+            ids_c = [self.free[F - 1 - (taken + k)] for k in range(self.nblk[c])]
+            for k, (b, sz) in enumerate(zip(ids_c, self._blocks(c))):
+                upd.append((b, sz, off + k * self.block))
             self.blocks[c] = ids_c
             self.stamp[c] = E
+            self.sub[c] = len(hits) + j
             taken += self.nblk[c]
         del self.free[F - taken:]
         self.epoch = E

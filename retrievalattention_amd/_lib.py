@@ -31,7 +31,7 @@ SIGNATURES = {
     "ri_wave_attention_static_scratch_bytes": (SZ, []),
     "ri_wave_attention_static": (I, [P, P, P, I64, I, P, P, P, I64, P, I, P, P, I, P, P, P, P, P, P, P, P, I, I, I, I, F, P]),
     "ri_buffer_attention": (I, [P, P, P, I64, P, I, P, P, P, P, P, I, I, I, I, F, P, SZ, P]),
-    "ri_lru_access_update": (I, [P, P, P, I, P, I, P, I, P, I, P, P, P] + [P] * 12 + [P, I, I, P] + [I] * 6 + [P]),
+    "ri_lru_access_update": (I, [P, P, P, I, P, I, P, P, I, P, I, P, P, P] + [P] * 12 + [P, I, I, P] + [I] * 6 + [P]),
     "ri_gather_copy_vectors": (I, [P, P, P, P, P, P, P, I, I, I, I, I, I, P]),
     "ri_gather_copy_and_concat": (I, [P] * 17 + [I] * 7 + [P]),
     "ri_gather_copy_and_scatter": (I, [P] * 8 + [I] * 5 + [P]),

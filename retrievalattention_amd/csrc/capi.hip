@@ -7,7 +7,7 @@ void ri_set_last_hip_error(int e) { g_last_hip_error = e; }
 
 extern "C" int ri_last_hip_error(void) { return g_last_hip_error; }
 
-extern "C" int ri_abi_version(void) { return 5; }
+extern "C" int ri_abi_version(void) { return 6; }
 
 // An empty launch: what a dependent kernel dispatch costs on this stream, for callers that want to
 // separate dispatch overhead from kernel time in event measurements.

@@ -11,17 +11,20 @@
 //     admission list for the scatter kernel.
 // The lists have the layout the copy kernels of gather.hip read.
 //
-// Recency is kept per cluster as the number of the last step that touched it.  Eviction takes
-// whole clusters, oldest step first and ascending cluster id inside the boundary step, until the
-// request is covered; clusters touched in the current step are never evicted, so an admission
-// that cannot be covered is cut short instead.  (The reference keeps a linked list in touch
-// order; which of several equally old clusters goes first is the only observable difference,
-// and nothing downstream depends on it: hits and misses deliver the same bytes.)
+// Recency is kept per resident cluster as a pair: the number of the last step that touched it and its order
+// inside that step.  That reproduces the reference's list (wave_buffer_cpu.cpp:106-114: the hits are moved to
+// the front in reverse rank order; :170-176: then the admitted misses are pushed in rank order): inside a
+// step the admitted misses are the most recent, later-ranked ones first, then the hits, earlier-ranked ones
+// first.  Eviction takes whole clusters from the least recent end until the request is covered, hits of the
+// current step included (:140-142; their blocks have been listed for this step's attention, which runs
+// before the admission copy overwrites them).  The victims are found without sorting: a radix selection over
+// the step ages (four 8-bit digits) gives the boundary step, and inside that step the clusters are ranked by
+// their order through an LDS table indexed by it.
 #include "ri_common.h"
 
 #define LRU_THREADS 1024
 #define LRU_WAVES (LRU_THREADS / 64)
-#define LRU_AGES 256
+#define LRU_DIGIT 256
 
 struct LruParams {
   const int32_t* ret_ids;   // [BG, np] cluster ids in rank order
@@ -29,6 +32,7 @@ struct LruParams {
   const int32_t* starts;    // [BG, meta_stride] first row of the cluster in the host store
   const int32_t* blk_off;   // [BG, blk_off_stride] exclusive prefix of ceil(size / block)
   int32_t* stamp;           // [BG, stamp_stride] 0 = not resident, else last step that touched it
+  int32_t* order;           // [BG, stamp_stride] order inside that step (larger = more recent)
   int32_t* blk_ids;         // [BG, blk_ids_stride] cache block ids of resident clusters, at blk_off
   int32_t* free_list;       // [BG, capacity] free block ids, the first free_count are valid
   int32_t* free_count;      // [BG]
@@ -72,10 +76,14 @@ __device__ __forceinline__ void lru_scan(const int (&v)[N], int (&pre)[N], int (
 template <int R>
 __global__ __launch_bounds__(LRU_THREADS) void lru_kernel(LruParams P) {
   constexpr int NPMAX = LRU_THREADS * R;
-  __shared__ int sh_scan[5 * LRU_WAVES];
-  __shared__ int sh_hist[LRU_AGES];
-  __shared__ int sh_cut[2];  // boundary age, blocks freed by strictly older clusters
-  __shared__ int sh_off[NPMAX], sh_src[NPMAX];
+  __shared__ int sh_scan[6 * LRU_WAVES];
+  __shared__ int sh_hist[LRU_DIGIT];
+  __shared__ int sh_cut[2];  // selected digit, blocks freed by clusters with a larger one
+  // token offsets and sources of the ranks for the row table; later the blocks of the boundary step's
+  // clusters by their order inside the step (2 * NPMAX entries: hits below, admitted misses above)
+  __shared__ int sh_tab[2 * NPMAX];
+  int* const sh_off = sh_tab;
+  int* const sh_src = sh_tab + NPMAX;
   const int g = blockIdx.x;
   const int tid = threadIdx.x;
   const int block = P.block;
@@ -83,6 +91,7 @@ __global__ __launch_bounds__(LRU_THREADS) void lru_kernel(LruParams P) {
   const int32_t* starts = P.starts + (size_t)g * P.meta_stride;
   const int32_t* boff = P.blk_off + (size_t)g * P.blk_off_stride;
   int32_t* stamp = P.stamp + (size_t)g * P.stamp_stride;
+  int32_t* order = P.order + (size_t)g * P.stamp_stride;
   int32_t* bids = P.blk_ids + (size_t)g * P.blk_ids_stride;
   int32_t* flist = P.free_list + (size_t)g * P.capacity;
   const size_t lo = (size_t)g * P.buffer_size;
@@ -116,7 +125,7 @@ __global__ __launch_bounds__(LRU_THREADS) void lru_kernel(LruParams P) {
   lru_scan<1>(v1, p1, t1, sh_scan);
   // the walk stops at the first cluster whose blocks no longer fit: everything after it is dropped
   bool keep[R], hit[R], miss[R];
-  int v5[5] = {0, 0, 0, 0, 0}, p5[5], t5[5];
+  int v5[6] = {0, 0, 0, 0, 0, 0}, p5[6], t5[6];
   {
     int run = p1[0];
 #pragma unroll
@@ -130,22 +139,25 @@ __global__ __launch_bounds__(LRU_THREADS) void lru_kernel(LruParams P) {
       v5[2] += miss[i] ? nb[i] : 0;
       v5[3] += miss[i] ? sz[i] : 0;
       v5[4] += keep[i] ? 1 : 0;
+      v5[5] += hit[i] ? 1 : 0;
     }
   }
-  lru_scan<5>(v5, p5, t5, sh_scan);
-  // per rank: hit blocks, kept tokens, miss blocks, miss tokens of the lower ranks
-  int hb_pre[R], tok_pre[R], mb_pre[R], mt_pre[R];
+  lru_scan<6>(v5, p5, t5, sh_scan);
+  // per rank: hit blocks, kept tokens, miss blocks, miss tokens, hits of the lower ranks
+  int hb_pre[R], tok_pre[R], mb_pre[R], mt_pre[R], hit_idx[R];
   {
-    int a = p5[0], b = p5[1], cc = p5[2], d = p5[3];
+    int a = p5[0], b = p5[1], cc = p5[2], d = p5[3], h = p5[5];
 #pragma unroll
     for (int i = 0; i < R; ++i) {
-      hb_pre[i] = a; tok_pre[i] = b; mb_pre[i] = cc; mt_pre[i] = d;
+      hb_pre[i] = a; tok_pre[i] = b; mb_pre[i] = cc; mt_pre[i] = d; hit_idx[i] = h;
       a += hit[i] ? nb[i] : 0;
       b += keep[i] ? sz[i] : 0;
       cc += miss[i] ? nb[i] : 0;
       d += miss[i] ? sz[i] : 0;
+      h += hit[i] ? 1 : 0;
     }
   }
+  const int nhits = t5[5];
   // tok_pre: tokens of kept clusters of lower rank (position in the row table); the hit list's own
   // token offsets are only needed without a row table
   int hit_tok[R];
@@ -211,6 +223,7 @@ __global__ __launch_bounds__(LRU_THREADS) void lru_kernel(LruParams P) {
         }
       }
       stamp[c[i]] = E;
+      order[c[i]] = nhits - 1 - hit_idx[i];   // hits are moved to the front in reverse rank order
     }
     if (miss[i]) {
       const int row = start_c[i];
@@ -231,55 +244,83 @@ __global__ __launch_bounds__(LRU_THREADS) void lru_kernel(LruParams P) {
       P.meta[g * 4 + 3] = 0;
     }
   }
-  if (tid < LRU_AGES) sh_hist[tid] = 0;
-  __syncthreads();  // the hits carry this step's stamp before anybody looks for victims
+  __syncthreads();  // the hits carry this step's stamp and order before anybody looks for victims
 
-  // ---- eviction: free (need - F0) blocks from the oldest clusters ----
+  // ---- eviction: free (need - F0) blocks from the least recently used clusters ----
   const int to_free = need - F0;  // uniform
   int F = F0;
   if (to_free > 0) {
-    // thread t owns the ids [t*K, t*K + K): id order inside the boundary age comes out of a prefix sum
+    // thread t owns the ids [t*K, t*K + K)
     const int K = (P.ncl + LRU_THREADS - 1) / LRU_THREADS;
     const int c0 = tid * K, c1 = min(P.ncl, c0 + K);
-    for (int cc = c0; cc < c1; ++cc) {
-      const int st = stamp[cc];
-      if (st != 0 && st != E) atomicAdd(&sh_hist[min(E - st, LRU_AGES - 1)], boff[cc + 1] - boff[cc]);
-    }
-    __syncthreads();
-    if (tid == 0) {
-      int acc = 0, cut = -1;
-      for (int a = LRU_AGES - 1; a >= 1; --a) {
-        if (acc + sh_hist[a] >= to_free) { cut = a; break; }
-        acc += sh_hist[a];
+    // boundary step: the age A such that every resident cluster older than A goes and the clusters of age A
+    // cover the remaining `rem` blocks; radix selection over the four bytes of the age, oldest first
+    uint32_t sel_mask = 0, sel_val = 0;
+    int rem = to_free;
+    for (int b = 3; b >= 0; --b) {
+      if (tid < LRU_DIGIT) sh_hist[tid] = 0;
+      if (tid == 0) { sh_cut[0] = 0; sh_cut[1] = 0; }
+      __syncthreads();
+      for (int cc = c0; cc < c1; ++cc) {
+        const int st = stamp[cc];
+        if (st == 0) continue;
+        const uint32_t age = (uint32_t)(E - st);
+        if ((age & sel_mask) == sel_val) atomicAdd(&sh_hist[(age >> (8 * b)) & 255u], boff[cc + 1] - boff[cc]);
       }
-      sh_cut[0] = cut;  // -1: even every untouched cluster does not cover the request
-      sh_cut[1] = acc;
+      __syncthreads();
+      if (tid < 64) {
+        // lane l holds the digits 255 - 4l .. 252 - 4l (oldest first); the lane whose running total crosses
+        // rem holds the boundary digit
+        int h[4], sum = 0;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) { h[i] = sh_hist[255 - (4 * tid + i)]; sum += h[i]; }
+        const int incl = (int)ri_wave_incl_scan((uint32_t)sum);
+        int acc = incl - sum;
+        if (acc < rem && rem <= incl) {
+          int sel = 0;
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            if (acc < rem && rem <= acc + h[i]) { sel = 255 - (4 * tid + i); sh_cut[1] = acc; }
+            acc += h[i];
+          }
+          sh_cut[0] = sel;
+        }
+      }
+      __syncthreads();
+      sel_val |= (uint32_t)sh_cut[0] << (8 * b);
+      sel_mask |= 255u << (8 * b);
+      rem -= sh_cut[1];
     }
+    const uint32_t cut = sel_val;   // boundary age; rem blocks are still wanted from the clusters of that age
+    // the clusters of the boundary step, least recent first = ascending order inside the step
+    for (int i = tid; i < 2 * NPMAX; i += LRU_THREADS) sh_tab[i] = 0;
     __syncthreads();
-    const int cut = sh_cut[0];
-    const int rem = to_free - sh_cut[1];  // blocks still wanted from the boundary age
-    int tie = 0;
     for (int cc = c0; cc < c1; ++cc) {
       const int st = stamp[cc];
-      if (st != 0 && st != E && min(E - st, LRU_AGES - 1) == cut) tie += boff[cc + 1] - boff[cc];
+      if (st != 0 && (uint32_t)(E - st) == cut) sh_tab[min(max(order[cc], 0), 2 * NPMAX - 1)] = boff[cc + 1] - boff[cc];
     }
-    int vt[1] = {tie}, pt[1], tt[1];
-    lru_scan<1>(vt, pt, tt, sh_scan);
-    int run = pt[0], ev = 0;
+    __syncthreads();
+    {
+      // exclusive prefix of the table in place: thread t owns the entries [t * 2R, t * 2R + 2R)
+      int own[2 * R], vt[1] = {0}, pt[1], tt[1];
+#pragma unroll
+      for (int i = 0; i < 2 * R; ++i) { own[i] = sh_tab[tid * 2 * R + i]; vt[0] += own[i]; }
+      lru_scan<1>(vt, pt, tt, sh_scan);
+      int run = pt[0];
+#pragma unroll
+      for (int i = 0; i < 2 * R; ++i) { sh_tab[tid * 2 * R + i] = run; run += own[i]; }
+    }
+    __syncthreads();
+    int ev = 0;
     uint64_t ev_bits = 0;  // K <= 64 ids per thread
     for (int cc = c0; cc < c1; ++cc) {
       const int st = stamp[cc];
-      if (st == 0 || st == E) continue;
-      const int age = min(E - st, LRU_AGES - 1);
-      const int nbc = boff[cc + 1] - boff[cc];
-      bool out = cut < 0 || age > cut;
-      if (age == cut) {
-        out = run < rem;
-        run += nbc;
-      }
+      if (st == 0) continue;
+      const uint32_t age = (uint32_t)(E - st);
+      const bool out = age > cut || (age == cut && sh_tab[min(max(order[cc], 0), 2 * NPMAX - 1)] < rem);
       if (out) {
         ev_bits |= 1ull << (cc - c0);
-        ev += nbc;
+        ev += boff[cc + 1] - boff[cc];
       }
     }
     int ve[1] = {ev}, pe[1], te[1];
@@ -296,16 +337,19 @@ __global__ __launch_bounds__(LRU_THREADS) void lru_kernel(LruParams P) {
   }
 
   // ---- admission: block ids come off the end of the free list in rank order ----
-  int vb[1] = {0}, pb[1], tb[1];
+  int vb[2] = {0, 0}, pb[2], tb[2];
 #pragma unroll
   for (int i = 0; i < R; ++i) {
-    adm[i] = adm[i] && adm_pre[i] + nb[i] <= F;  // cut short if the untouched clusters did not cover the request
+    adm[i] = adm[i] && adm_pre[i] + nb[i] <= F;  // (always true: everything resident can be evicted)
     vb[0] += adm[i] ? nb[i] : 0;
+    vb[1] += adm[i] ? 1 : 0;
   }
-  lru_scan<1>(vb, pb, tb, sh_scan);
+  lru_scan<2>(vb, pb, tb, sh_scan);
+  int adm_idx = pb[1];
 #pragma unroll
   for (int i = 0; i < R; ++i) {
     if (adm[i]) {
+      order[c[i]] = nhits + adm_idx++;   // pushed to the front in rank order, after the hits
       int32_t* ids = bids + boff_c[i];
       for (int j = 0; j < nb[i]; ++j) {
         const int id = flist[F - 1 - (adm_pre[i] + j)];
@@ -326,7 +370,7 @@ __global__ __launch_bounds__(LRU_THREADS) void lru_kernel(LruParams P) {
 
 extern "C" int ri_lru_access_update(const int32_t* ret_ids, const int32_t* sizes, const int32_t* starts,
                                     int meta_stride, const int32_t* blk_off, int blk_off_stride, int32_t* stamp,
-                                    int stamp_stride, int32_t* blk_ids, int blk_ids_stride, int32_t* free_list,
+                                    int32_t* order, int stamp_stride, int32_t* blk_ids, int blk_ids_stride, int32_t* free_list,
                                     int32_t* free_count, int32_t* epoch, int32_t* hit_ids, int32_t* hit_sizes,
                                     int32_t* hit_cumsum, int32_t* hit_num, int32_t* miss_ids, int32_t* miss_sizes,
                                     int32_t* miss_cumsum, int32_t* miss_num, int32_t* upd_buf, int32_t* upd_sizes,
@@ -334,7 +378,7 @@ extern "C" int ri_lru_access_update(const int32_t* ret_ids, const int32_t* sizes
                                     int stage_row0, int32_t* meta, int BG, int np, int ncl, int buffer_size,
                                     int capacity, int block, ri_stream_t stream) {
   // (a cache without blocks has an empty free list: its pointer may be null)
-  if (!ret_ids || !sizes || !starts || !blk_off || !stamp || !blk_ids || (!free_list && capacity > 0) || !free_count ||
+  if (!ret_ids || !sizes || !starts || !blk_off || !stamp || !order || !blk_ids || (!free_list && capacity > 0) || !free_count ||
       !epoch ||
       !hit_ids || !hit_sizes || !hit_cumsum || !hit_num || !miss_ids || !miss_sizes || !miss_cumsum || !miss_num ||
       !upd_buf || !upd_sizes || !upd_cache || !upd_num)
@@ -344,7 +388,7 @@ extern "C" int ri_lru_access_update(const int32_t* ret_ids, const int32_t* sizes
     return RI_ERR_ARG;
   if (meta_stride < ncl || blk_off_stride < ncl + 1 || stamp_stride < ncl || blk_ids_stride <= 0) return RI_ERR_ARG;
   if (row_src && (!meta || row_src_stride < buffer_size * block || stage_row0 < capacity * block)) return RI_ERR_ARG;
-  LruParams P = {ret_ids, sizes, starts, blk_off, stamp, blk_ids, free_list, free_count, epoch,
+  LruParams P = {ret_ids, sizes, starts, blk_off, stamp, order, blk_ids, free_list, free_count, epoch,
                  hit_ids, hit_sizes, hit_cumsum, hit_num, miss_ids, miss_sizes, miss_cumsum, miss_num,
                  upd_buf, upd_sizes, upd_cache, upd_num, row_src, meta, row_src_stride, stage_row0,
                  np, ncl, meta_stride, blk_off_stride, stamp_stride, blk_ids_stride, buffer_size, capacity, block};

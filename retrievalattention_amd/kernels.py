@@ -421,7 +421,8 @@ class DeviceLru:
     def __init__(self, BG, max_clusters, max_blocks, capacity, buffer_size, block, device):
         i32 = lambda *s: torch.zeros(s, dtype=torch.int32, device=device)
         self.BG, self.capacity, self.buffer_size, self.block = BG, capacity, buffer_size, block
-        self.stamp = i32(BG, max_clusters)
+        self.stamp = i32(BG, max_clusters)     # step that last touched a resident cluster (0: not resident)
+        self.order = i32(BG, max_clusters)     # ... and the cluster's position inside that step
         self.blk_off = i32(BG, max_clusters + 1)
         self.blk_ids = i32(BG, max_blocks)
         self.free_list = torch.arange(capacity, dtype=torch.int32, device=device).repeat(BG, 1).contiguous()
@@ -443,7 +444,7 @@ class DeviceLru:
         ncl = sizes.shape[1]
         check(lib().ri_lru_access_update(
             _p(ret_ids), _p(sizes), _p(starts), sizes.stride(0), _p(self.blk_off), self.blk_off.shape[1],
-            _p(self.stamp), self.stamp.shape[1], _p(self.blk_ids), self.blk_ids.shape[1], _p(self.free_list),
+            _p(self.stamp), _p(self.order), self.stamp.shape[1], _p(self.blk_ids), self.blk_ids.shape[1], _p(self.free_list),
             _p(self.free_count), _p(self.epoch), *[_p(t) for t in lists], _p(row_src),
             0 if row_src is None else row_src.shape[1], stage_row0, _p(meta), BG, np_, ncl, self.buffer_size,
             self.capacity, self.block, _stream()), "lru_access_update")

@@ -60,17 +60,21 @@ def test_lists_match_the_model_step_by_step(dev, ncl, nprobe, capacity, buffer_s
             assert lru.free_list[g, :len(models[g].free)].tolist() == models[g].free
             stamp = lru.stamp[g, :ncl].cpu()
             assert [int(x) for x in stamp] == models[g].stamp
+            order = lru.order[g, :ncl].cpu()
+            assert all(int(order[c]) == models[g].sub[c] for c in models[g].blocks)
     assert capacity == 0 or any(len(m.blocks) > 0 for m in models)
 
 
-@pytest.mark.parametrize("ncl,capacity,steps,seed", [(40, 24, 250, 0), (300, 64, 250, 1), (12, 10, 200, 2)])
-def test_one_probe_per_step_equals_the_reference_policy(dev, ncl, capacity, steps, seed):
-    """With one retrieved cluster per step every recency stamp is unique, and with fewer than 255 steps no age
-    saturates: step-granular recency is then the reference's touch order, so the kernel's hit / miss / admission
-    lists and its evictions must equal those of the reference's manager (LruModel, itself checked against the
-    reference's own BufferManager build), block id values aside (an id map is kept and must stay a bijection)."""
+@pytest.mark.parametrize("ncl,nprobe,capacity,steps,seed", [(40, 1, 24, 250, 0), (300, 1, 64, 250, 1), (200, 12, 60, 80, 2),
+                                                           (60, 8, 10, 120, 3), (3000, 150, 900, 40, 4)])
+def test_lists_equal_the_reference_policy(dev, ncl, nprobe, capacity, steps, seed):
+    """The kernel's hit / miss / admission lists and its evictions equal those of the reference's manager
+    (LruModel, itself checked against the reference's own BufferManager build) over random probe traces: one
+    probe per step, several probes with eviction pressure, a cache smaller than one step's hits (hits of the
+    current step are evicted), a config-4-like size.  Block id values aside: an id map is kept and must stay
+    a bijection."""
     from retrievalattention_amd import kernels
-    BG, block, buffer_size = 2, 8, 16
+    BG, block, buffer_size = 2, 8, max(16, 4 * nprobe)
     rnd = random.Random(seed)
     sizes = [[rnd.randint(0, 30) for _ in range(ncl)] for _ in range(BG)]
     refs = [LruModel(s, block, capacity, buffer_size) for s in sizes]
@@ -81,10 +85,10 @@ def test_one_probe_per_step_equals_the_reference_policy(dev, ncl, capacity, step
     lru.set_sizes(sz)
     lists = [torch.full((BG, buffer_size), -7, dtype=torch.int32, device=dev) if i % 4 != 3
              else torch.zeros(BG, dtype=torch.int32, device=dev) for i in range(12)]
-    hot = [rnd.sample(range(ncl), max(2, ncl // 3)) for _ in range(BG)]
+    hot = [rnd.sample(range(ncl), max(2, min(ncl, 3 * nprobe), ncl // 3 if nprobe == 1 else 0)) for _ in range(BG)]
     evictions = 0
     for step in range(steps):
-        ids = [[rnd.choice(hot[g]) if rnd.random() < 0.6 else rnd.randrange(ncl)] for g in range(BG)]
+        ids = [rnd.sample(hot[g] if rnd.random() < 0.6 else range(ncl), nprobe) for g in range(BG)]
         lru.access_update(torch.tensor(ids, dtype=torch.int32, device=dev), sz, st, lists)
         torch.cuda.synchronize()
         host = [x.cpu() for x in lists]
@@ -93,21 +97,20 @@ def test_one_probe_per_step_equals_the_reference_policy(dev, ncl, capacity, step
             hit, miss = refs[g].access(ids[g])
             upd = refs[g].update()
             evictions += len(before - set(refs[g].resident))
-            # blocks of clusters evicted in this step go back to the free list and may be handed out again at once
-            maps[g].retain({b for ids_c in refs[g].resident.values() for b in ids_c} - {b for b, _, _ in upd})
+            lists_g = []
             for k, ref in enumerate((hit, miss, upd)):
                 a, b, c, n = host[4 * k:4 * k + 4]
                 assert int(n[g]) == len(ref), (step, g, k)
                 got = list(zip(a[g, :len(ref)].tolist(), b[g, :len(ref)].tolist(), c[g, :len(ref)].tolist()))
-                if k == 2:
-                    got = [(z, y, x) for x, y, z in got]
-                if k == 1:                      # misses: host rows, no block ids involved
-                    assert got == ref, (step, g, k)
-                else:
-                    if k == 2:                  # admission hands out ids: the map learns them
-                        for (bg, _, _), (br, _, _) in zip(got, ref):
-                            maps[g].bind(bg, br)
-                    assert [(maps[g].to_ref(x), y, z) for x, y, z in got] == ref, (step, g, k)
+                lists_g.append([(z, y, x) for x, y, z in got] if k == 2 else got)
+            # hits: block ids through the map (a hit of this step may be evicted by the same step's admission)
+            assert [(maps[g].to_ref(x), y, z) for x, y, z in lists_g[0]] == hit, (step, g, 0)
+            assert lists_g[1] == miss, (step, g, 1)      # misses: host rows, no block ids involved
+            # blocks of clusters evicted in this step go back to the free list and may be handed out again at once
+            maps[g].retain({b for ids_c in refs[g].resident.values() for b in ids_c} - {b for b, _, _ in upd})
+            for (bg, _, _), (br, _, _) in zip(lists_g[2], upd):     # admission hands out ids: the map learns them
+                maps[g].bind(bg, br)
+            assert [(maps[g].to_ref(x), y, z) for x, y, z in lists_g[2]] == upd, (step, g, 2)
             # the same clusters are resident: evictions happened in the same order
             resident = set(torch.nonzero(lru.stamp[g, :ncl]).flatten().tolist())
             assert resident == set(refs[g].resident), (step, g)
@@ -153,6 +156,6 @@ def test_bad_arguments(dev):
     z = torch.zeros(64, dtype=torch.int32, device=dev)
     p = z.data_ptr()
     ptrs = [p] * 12
-    assert l.ri_lru_access_update(p, p, p, 8, p, 9, p, 8, p, 8, p, p, p, *ptrs, None, 0, 0, None, 1, 4097, 8, 4, 4, 8, None) == -1   # np too large
-    assert l.ri_lru_access_update(p, p, p, 4, p, 9, p, 8, p, 8, p, p, p, *ptrs, None, 0, 0, None, 1, 2, 8, 4, 4, 8, None) == -1      # stride < ncl
-    assert l.ri_lru_access_update(None, p, p, 8, p, 9, p, 8, p, 8, p, p, p, *ptrs, None, 0, 0, None, 1, 2, 8, 4, 4, 8, None) == -1
+    assert l.ri_lru_access_update(p, p, p, 8, p, 9, p, p, 8, p, 8, p, p, p, *ptrs, None, 0, 0, None, 1, 4097, 8, 4, 4, 8, None) == -1   # np too large
+    assert l.ri_lru_access_update(p, p, p, 4, p, 9, p, p, 8, p, 8, p, p, p, *ptrs, None, 0, 0, None, 1, 2, 8, 4, 4, 8, None) == -1      # stride < ncl
+    assert l.ri_lru_access_update(None, p, p, 8, p, 9, p, p, 8, p, 8, p, p, p, *ptrs, None, 0, 0, None, 1, 2, 8, 4, 4, 8, None) == -1

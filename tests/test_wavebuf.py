@@ -177,78 +177,48 @@ def test_pinned_workers():
     del wb, pool
 
 
-def test_device_lru_model_invariants():
-    """The policy the device-side manager implements, on its Python restatement: every requested
-    cluster is a hit or a miss exactly once (until the buffer cut-off), hit <=> resident, block ids
-    unique, resident blocks + free blocks = capacity, victims are the least recently touched."""
-    import random
-    from oracle.wavebuf import DeviceLruModel
-    rnd = random.Random(3)
-    sizes = [rnd.randint(0, 40) for _ in range(200)]
-    m = DeviceLruModel(sizes, 8, 60, 48)
-    last_touch = {}
-    for step in range(1, 60):
-        ids = rnd.sample(range(200), 12)
-        resident_before = set(m.blocks)
-        hit, miss, upd = m.step(ids)
-        pages, seen = 0, []
-        for c in ids:
-            pages += m.nblk[c]
-            if pages > 48:
-                break
-            if m.nblk[c]:
-                seen.append(c)
-        assert len(hit) + len(miss) == sum(m.nblk[c] for c in seen)
-        assert sum(sz for _, sz, _ in hit) + sum(sz for _, sz, _ in miss) == sum(sizes[c] for c in seen)
-        hits = [c for c in seen if c in resident_before]
-        assert len(hit) == sum(m.nblk[c] for c in hits)
-        for c in seen:
-            if c in m.blocks:
-                last_touch[c] = step
-        used = [b for ids_c in m.blocks.values() for b in ids_c]
-        assert len(set(used)) == len(used) and not set(used) & set(m.free)
-        assert len(used) + len(m.free) == 60
-        evicted = resident_before - set(m.blocks)
-        if evicted:   # nothing older than a victim stays resident, except within the boundary step
-            newest_victim = max(last_touch[c] for c in evicted)
-            for c in m.blocks:
-                if c not in seen:
-                    assert last_touch[c] >= newest_victim or last_touch[c] == newest_victim
-            oldest_kept = min((last_touch[c] for c in m.blocks if c not in seen), default=step)
-            assert max(last_touch[c] for c in evicted) <= oldest_kept
-        for c in evicted:
-            last_touch.pop(c, None)
-
-
-@pytest.mark.parametrize("ncl,capacity,steps,seed", [(40, 24, 250, 0), (300, 64, 250, 1), (12, 10, 200, 2), (30, 0, 50, 3)])
-def test_device_policy_equals_the_reference_policy_with_one_probe_per_step(ncl, capacity, steps, seed):
-    """Where the two block cache policies must coincide they do: with one retrieved cluster per step the
-    step-granular recency of DeviceLruModel is a total order (every stamp unique) and, below 255 steps, no age
-    saturates, so it is the touch order of the reference's list (LruModel, pinned by the reference's own
-    BufferManager build).  Hit, miss and admission lists and the set of resident clusters after every step are
-    identical, block id values aside (the two hand out free ids in different orders; the map must stay a
-    bijection)."""
+@pytest.mark.parametrize("ncl,nprobe,capacity,buffer_size,steps,seed", [
+    (200, 12, 60, 48, 80, 0),        # constant eviction pressure, several probes per step
+    (60, 8, 10, 64, 120, 1),         # a cache smaller than one step's hits: hits of the current step are evicted
+    (300, 20, 40, 30, 60, 2),        # buffer cut-off and admission prefix
+    (40, 1, 24, 16, 250, 3),         # one probe per step
+    (500, 30, 4000, 400, 30, 4),     # no eviction at all
+    (30, 6, 0, 64, 20, 5),           # no cache
+])
+def test_device_manager_model_follows_the_reference_policy(ncl, nprobe, capacity, buffer_size, steps, seed):
+    """DeviceLruModel (what the device-side manager is compared with, list by list) keeps the reference's
+    policy: over random probe traces its hit, miss and admission lists and the set of resident clusters after
+    every step equal those of LruModel, which is pinned by the reference's own BufferManager build; only the
+    block id values differ (the two hand out free ids in different orders; the map must stay a bijection)."""
     import random
     from oracle.wavebuf import DeviceLruModel
     from tests.parity import BlockIdMap
     rnd = random.Random(seed)
-    sizes = [rnd.randint(0, 30) for _ in range(ncl)]
-    dev_m, ref_m, ids_map = DeviceLruModel(sizes, 8, capacity, 16), LruModel(sizes, 8, capacity, 16), BlockIdMap()
-    hot = rnd.sample(range(ncl), max(2, ncl // 3))
-    evictions = 0
+    sizes = [rnd.choice([0, 1, 7, 8, 9, 16, 23]) if rnd.random() < 0.3 else rnd.randint(1, 30) for _ in range(ncl)]
+    dev_m, ref_m, ids_map = DeviceLruModel(sizes, 8, capacity, buffer_size), LruModel(sizes, 8, capacity, buffer_size), BlockIdMap()
+    hot = rnd.sample(range(ncl), min(ncl, 3 * nprobe))
+    evictions = evicted_hits = 0
     for step in range(steps):
-        ids = [rnd.choice(hot) if rnd.random() < 0.6 else rnd.randrange(ncl)]
+        ids = rnd.sample(hot if rnd.random() < 0.7 else range(ncl), nprobe)
         before = set(ref_m.resident)
         hit_r, miss_r = ref_m.access(ids)
+        hit_keys = list(ref_m.hit_keys)
         upd_r = ref_m.update()
-        evictions += len(before - set(ref_m.resident))
+        gone = before - set(ref_m.resident)
+        evictions += len(gone)
+        evicted_hits += len(gone & set(hit_keys))
         hit_d, miss_d, upd_d = dev_m.step(ids)
         assert miss_d == miss_r
+        assert [(ids_map.to_ref(b), s, o) for b, s, o in hit_d] == hit_r
         ids_map.retain({b for v in ref_m.resident.values() for b in v} - {b for b, _, _ in upd_r})
         assert len(upd_d) == len(upd_r)
         for (bd, _, _), (br, _, _) in zip(upd_d, upd_r):
             ids_map.bind(bd, br)
-        assert [(ids_map.to_ref(b), s, o) for b, s, o in hit_d] == hit_r
         assert [(ids_map.to_ref(b), s, o) for b, s, o in upd_d] == upd_r
         assert set(dev_m.blocks) == set(ref_m.resident)
-    assert evictions > 0 or capacity == 0
+        used = [b for v in dev_m.blocks.values() for b in v]
+        assert len(set(used)) == len(used) and not set(used) & set(dev_m.free) and len(used) + len(dev_m.free) == capacity
+    if seed in (0, 1, 3):
+        assert evictions > 0
+    if seed == 1:
+        assert evicted_hits > 0
