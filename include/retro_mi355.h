@@ -10,7 +10,9 @@
  *    host arrays registered with set_indices/set_kv, so the caller keeps them alive.
  *  - `stream` is a hipStream_t passed as void* (NULL = the default stream).  Kernels
  *    are only enqueued; nothing synchronises unless stated.
- *  - Element type of K/V/centroid/query data is bfloat16 (uint16 bit patterns).
+ *  - Element type of K/V/centroid/query data is bfloat16 (uint16 bit patterns); every entry point whose
+ *    arithmetic depends on the element type has a twin with the suffix _f16 for IEEE half (the copy and
+ *    permutation entry points move 16-bit elements of either type).
  *    head_dim must be 128 (the reference hard-codes it: gather_copy.cu:196-199).
  *  - Return value: RI_OK (0) or a negative RI_ERR_* code; ri_status_string() names it
  *    and ri_last_hip_error() returns the HIP error behind RI_ERR_LAUNCH.
@@ -108,6 +110,16 @@ int ri_score_select(const void* q, const void* centroids, const uint8_t* mask,
                     int row_src_stride, int32_t* meta, int BG, int gs, int nc, int np, int es,
                     int page, int max_pages, float scale, void* workspace,
                     size_t workspace_bytes, ri_stream_t stream);
+/* ri_score_select on IEEE half instead of bfloat16 (every 16-bit tensor of the call; fp32 and integer
+ * arguments as above; the reference's operators and cache take either type: batch_gemm_softmax.cu:185-197,
+ * gather_copy.cu:63-67, and its harnesses default to fp16: simple_test.py:29). */
+int ri_score_select_f16(const void* q, const void* centroids, const uint8_t* mask,
+                        const int32_t* cluster_size_i32, const int32_t* cluster_start,
+                        float* logits, void* dist, int64_t* cI, int32_t* ret_ids,
+                        int32_t* est_ids, int32_t* ret_tok_off, int32_t* ret_start, int32_t* row_src,
+                        int row_src_stride, int32_t* meta, int BG, int gs, int nc, int np, int es,
+                        int page, int max_pages, float scale, void* workspace,
+                        size_t workspace_bytes, ri_stream_t stream);
 
 /* Scores only: logits[g, j, c] = scale * <q[g,j,:], centroids[g,c,:]> in fp32, no selection.
  * Used when the zones of a layer were chosen ahead of time from a predicted query
@@ -117,6 +129,11 @@ int ri_score_select(const void* q, const void* centroids, const uint8_t* mask,
  * workspace: ri_score_select_workspace_bytes(BG, gs, nc). */
 int ri_score_logits(const void* q, const void* centroids, float* logits, int BG, int gs, int nc,
                     float scale, void* workspace, size_t workspace_bytes, ri_stream_t stream);
+/* ri_score_logits on IEEE half instead of bfloat16 (every 16-bit tensor of the call; fp32 and integer
+ * arguments as above; the reference's operators and cache take either type: batch_gemm_softmax.cu:185-197,
+ * gather_copy.cu:63-67, and its harnesses default to fp16: simple_test.py:29). */
+int ri_score_logits_f16(const void* q, const void* centroids, float* logits, int BG, int gs, int nc,
+                        float scale, void* workspace, size_t workspace_bytes, ri_stream_t stream);
 
 /* ------------------------------------------------------------------------------------
  * (4) Weighted flash decoding
@@ -148,6 +165,14 @@ int ri_weighted_flash_decoding(const void* q, const void* k, const void* v, cons
                                const float* prev_lse, void* out, float* lse_out, int BG,
                                int gs, int S, int64_t kv_stride, float scale, void* workspace,
                                size_t workspace_bytes, ri_stream_t stream);
+/* ri_weighted_flash_decoding on IEEE half instead of bfloat16 (every 16-bit tensor of the call; fp32 and integer
+ * arguments as above; the reference's operators and cache take either type: batch_gemm_softmax.cu:185-197,
+ * gather_copy.cu:63-67, and its harnesses default to fp16: simple_test.py:29). */
+int ri_weighted_flash_decoding_f16(const void* q, const void* k, const void* v, const void* weight,
+                                   const int32_t* cache_seqlens, const void* prev_out,
+                                   const float* prev_lse, void* out, float* lse_out, int BG,
+                                   int gs, int S, int64_t kv_stride, float scale, void* workspace,
+                                   size_t workspace_bytes, ri_stream_t stream);
 
 /* Fused wave-index attention over a device-resident cluster store: replaces steps 4-8 of
  * retroinfer_cache.compute (gather_copy_vectors → weighted_flash_decoding →
@@ -183,6 +208,19 @@ int ri_wave_attention(const void* q, const void* steady_k, const void* steady_v,
                       const void* cluster_size_bf16, void* out, int32_t* valid_lengths,
                       int BG, int gs, int nc, int es, float scale, void* workspace,
                       size_t workspace_bytes, ri_stream_t stream);
+/* ri_wave_attention on IEEE half instead of bfloat16 (every 16-bit tensor of the call; fp32 and integer
+ * arguments as above; the reference's operators and cache take either type: batch_gemm_softmax.cu:185-197,
+ * gather_copy.cu:63-67, and its harnesses default to fp16: simple_test.py:29). */
+int ri_wave_attention_f16(const void* q, const void* steady_k, const void* steady_v,
+                          int64_t steady_stride, int static_len, const int32_t* static_len_dev,
+                          const void* store_k,
+                          const void* store_v, int64_t store_stride, const int32_t* row_src,
+                          int row_src_stride, const int32_t* ret_tok_off, const int32_t* ret_start, int np,
+                          const int32_t* meta, const int32_t* est_ids,
+                          const float* logits, const void* est_centroids, const void* value_sum,
+                          const void* cluster_size_bf16, void* out, int32_t* valid_lengths,
+                          int BG, int gs, int nc, int es, float scale, void* workspace,
+                          size_t workspace_bytes, ri_stream_t stream);
 
 /* One part of a wave attention over a row table (host-resident store, block cache managed on the device;
  * cache_hub/retroinfer_cache.py:629-674, where the reference overlaps the transfer of missed blocks with
@@ -206,6 +244,18 @@ int ri_wave_attention_part(const void* q, const void* steady_k, const void* stea
                            const float* prev_lse, void* out, float* lse_out, int32_t* valid_lengths,
                            int BG, int gs, int nc, int es, float scale, void* workspace,
                            size_t workspace_bytes, ri_stream_t stream);
+/* ri_wave_attention_part on IEEE half instead of bfloat16 (every 16-bit tensor of the call; fp32 and integer
+ * arguments as above; the reference's operators and cache take either type: batch_gemm_softmax.cu:185-197,
+ * gather_copy.cu:63-67, and its harnesses default to fp16: simple_test.py:29). */
+int ri_wave_attention_part_f16(const void* q, const void* steady_k, const void* steady_v,
+                               int64_t steady_stride, int static_len, const int32_t* static_len_dev,
+                               const void* store_k, const void* store_v, int64_t store_stride,
+                               const int32_t* row_src, int row_src_stride, int src_row_lo, int src_row_hi,
+                               const int32_t* meta, const int32_t* est_ids, const float* logits,
+                               const void* value_sum, const void* cluster_size_bf16, const void* prev_out,
+                               const float* prev_lse, void* out, float* lse_out, int32_t* valid_lengths,
+                               int BG, int gs, int nc, int es, float scale, void* workspace,
+                               size_t workspace_bytes, ri_stream_t stream);
 
 /* ri_wave_attention for callers that cannot allocate device memory: code running under HIP stream
  * capture, tight serving loops, harnesses that forbid hipMalloc.  No counterpart in the reference.
@@ -228,6 +278,17 @@ int ri_wave_attention_static(const void* q, const void* steady_k, const void* st
                              const float* logits, const void* est_centroids, const void* value_sum,
                              const void* cluster_size_bf16, void* out, int32_t* valid_lengths, int BG,
                              int gs, int nc, int es, float scale, ri_stream_t stream);
+/* ri_wave_attention_static on IEEE half instead of bfloat16 (every 16-bit tensor of the call; fp32 and integer
+ * arguments as above; the reference's operators and cache take either type: batch_gemm_softmax.cu:185-197,
+ * gather_copy.cu:63-67, and its harnesses default to fp16: simple_test.py:29). */
+int ri_wave_attention_static_f16(const void* q, const void* steady_k, const void* steady_v,
+                                 int64_t steady_stride, int static_len, const int32_t* static_len_dev,
+                                 const void* store_k, const void* store_v, int64_t store_stride,
+                                 const int32_t* row_src, int row_src_stride, const int32_t* ret_tok_off,
+                                 const int32_t* ret_start, int np, const int32_t* meta, const int32_t* est_ids,
+                                 const float* logits, const void* est_centroids, const void* value_sum,
+                                 const void* cluster_size_bf16, void* out, int32_t* valid_lengths, int BG,
+                                 int gs, int nc, int es, float scale, ri_stream_t stream);
 
 /* Attention over an execution buffer with the estimation zone fused in: replaces
  * gather_copy_vectors → weighted_flash_decoding (estimation) and the final
@@ -243,6 +304,14 @@ int ri_buffer_attention(const void* q, const void* buf_k, const void* buf_v, int
                         const float* logits, const void* value_sum, const void* cluster_size_bf16,
                         void* out, int BG, int gs, int nc, int es, float scale, void* workspace,
                         size_t workspace_bytes, ri_stream_t stream);
+/* ri_buffer_attention on IEEE half instead of bfloat16 (every 16-bit tensor of the call; fp32 and integer
+ * arguments as above; the reference's operators and cache take either type: batch_gemm_softmax.cu:185-197,
+ * gather_copy.cu:63-67, and its harnesses default to fp16: simple_test.py:29). */
+int ri_buffer_attention_f16(const void* q, const void* buf_k, const void* buf_v, int64_t buf_stride,
+                            const int32_t* cache_seqlens, int max_len, const int32_t* est_ids,
+                            const float* logits, const void* value_sum, const void* cluster_size_bf16,
+                            void* out, int BG, int gs, int nc, int es, float scale, void* workspace,
+                            size_t workspace_bytes, ri_stream_t stream);
 
 /* ------------------------------------------------------------------------------------
  * (3) Wave-buffer copies
@@ -294,6 +363,11 @@ int ri_gather_copy_and_scatter(const void* ksrc, void* kcache, const void* vsrc,
  * effects are produced by ri_kmeans_update instead, in a fixed summation order.) */
 int ri_kmeans_assign(const void* data, const void* centroids, int32_t* assign, int P, int N,
                      int nc, int seg, int64_t head_rows, ri_stream_t stream);
+/* ri_kmeans_assign on IEEE half instead of bfloat16 (every 16-bit tensor of the call; fp32 and integer
+ * arguments as above; the reference's operators and cache take either type: batch_gemm_softmax.cu:185-197,
+ * gather_copy.cu:63-67, and its harnesses default to fp16: simple_test.py:29). */
+int ri_kmeans_assign_f16(const void* data, const void* centroids, int32_t* assign, int P, int N,
+                         int nc, int seg, int64_t head_rows, ri_stream_t stream);
 
 /* Inverted lists: replaces triton_reverse_index (cache_hub/kmeans.py:128-173) in CSR form.
  * counts [P, nc] int32, offsets [P, nc+1] int32 (exclusive prefix), members [P, N] int32 =
@@ -317,12 +391,25 @@ int ri_kmeans_update(const void* data, const int32_t* counts, const int32_t* off
                      const int32_t* members, void* centroids, int P, int N, int nc, int seg,
                      int64_t head_rows, int normalize, void* workspace, size_t workspace_bytes,
                      ri_stream_t stream);
+/* ri_kmeans_update on IEEE half instead of bfloat16 (every 16-bit tensor of the call; fp32 and integer
+ * arguments as above; the reference's operators and cache take either type: batch_gemm_softmax.cu:185-197,
+ * gather_copy.cu:63-67, and its harnesses default to fp16: simple_test.py:29). */
+int ri_kmeans_update_f16(const void* data, const int32_t* counts, const int32_t* offsets,
+                         const int32_t* members, void* centroids, int P, int N, int nc, int seg,
+                         int64_t head_rows, int normalize, void* workspace, size_t workspace_bytes,
+                         ri_stream_t stream);
 
 /* Per-cluster value sums: replaces triton_index_add (cache_hub/kmeans.py:176-221).
  * value_sum[p,c,:] = bf16(Σ member value rows), Σ in the same fixed order as above. */
 int ri_kmeans_value_sum(const void* values, const int32_t* counts, const int32_t* offsets,
                         const int32_t* members, void* value_sum, int P, int N, int nc,
                         void* workspace, size_t workspace_bytes, ri_stream_t stream);
+/* ri_kmeans_value_sum on IEEE half instead of bfloat16 (every 16-bit tensor of the call; fp32 and integer
+ * arguments as above; the reference's operators and cache take either type: batch_gemm_softmax.cu:185-197,
+ * gather_copy.cu:63-67, and its harnesses default to fp16: simple_test.py:29). */
+int ri_kmeans_value_sum_f16(const void* values, const int32_t* counts, const int32_t* offsets,
+                            const int32_t* members, void* value_sum, int P, int N, int nc,
+                            void* workspace, size_t workspace_bytes, ri_stream_t stream);
 
 /* Device-side block cache manager: BufferManager::batch_access followed by
  * BufferManager::batch_update (wave_buffer_cpu.cpp:190-257 and :102-188) in one launch, one

@@ -7,7 +7,7 @@ arithmetic below is the one its call sites imply
     out = (e^{lse_prev} * out_prev + sum_r e^{s_r} v_r) / (e^{lse_prev} + sum_r w_r e^{s_r})
     lse = log(denominator),  s_r = scale * q.k_r
 
-Computed in fp64 from the bf16 inputs; outputs rounded to bf16 like the kernel's.
+Computed in fp64 from the 16-bit inputs; outputs rounded to their element type like the kernel's.
 """
 import math
 import torch
@@ -21,7 +21,7 @@ def weighted_flash_decoding(q, k, v, weight=None, previous_out=None, previous_ls
     S = k.shape[1]
     if scale is None:
         scale = 1.0 / math.sqrt(D)
-    out = torch.empty(BG, gs, D, dtype=torch.bfloat16)
+    out = torch.empty(BG, gs, D, dtype=q.dtype if q.dtype in (torch.bfloat16, torch.float16) else torch.bfloat16)
     lse = torch.empty(BG, gs, dtype=torch.float32)
     for g in range(BG):
         n = S if cache_seqlens is None else int(cache_seqlens[g])
@@ -37,7 +37,7 @@ def weighted_flash_decoding(q, k, v, weight=None, previous_out=None, previous_ls
             f = torch.exp(previous_lse[g].double() - m)
             num = num + f[:, None] * previous_out[g].double()
             den = den + f
-        out[g] = (num / den[:, None]).to(torch.bfloat16)
+        out[g] = (num / den[:, None]).to(out.dtype)
         lse[g] = (m + torch.log(den)).to(torch.float32)
     return out, lse
 

@@ -14,8 +14,9 @@ def _f32(t: torch.Tensor) -> np.ndarray:
     return t.to(torch.float32).numpy()
 
 
-def _to_bf16(a: np.ndarray) -> torch.Tensor:
-    return torch.from_numpy(np.ascontiguousarray(a, dtype=np.float32)).to(torch.bfloat16)
+def _to_bf16(a: np.ndarray, dtype=torch.bfloat16) -> torch.Tensor:
+    """fp32 array -> tensor of the 16-bit element type (round to nearest even)."""
+    return torch.from_numpy(np.ascontiguousarray(a, dtype=np.float32)).to(dtype)
 
 
 def init_indices(num_tokens: int, num_centroids: int) -> torch.Tensor:
@@ -88,7 +89,7 @@ def update(cent: torch.Tensor, s: np.ndarray, cnt: np.ndarray, normalize: bool) 
         if normalize:
             nrm = np.sqrt(_lane_butterfly_sumsq(x)).astype(np.float32)
             x = (x / nrm[:, None]).astype(np.float32)
-        out[torch.from_numpy(nz)] = _to_bf16(x)
+        out[torch.from_numpy(nz)] = _to_bf16(x, cent.dtype)
     return out
 
 
@@ -102,7 +103,7 @@ def train_step(data, cent, normalize):
 def value_sum(value: torch.Tensor, a: np.ndarray, nc: int) -> torch.Tensor:
     """kmeans.py:205-221: fp32 sums cast to the value dtype."""
     s, _ = cluster_sums(value, a, nc)
-    return _to_bf16(s)
+    return _to_bf16(s, value.dtype)
 
 
 def reverse_index(a: np.ndarray, nc: int):
@@ -137,7 +138,7 @@ def segment_k_means(key, value, num_centroids, num_iters=10, num_segments=1):
                 c, _, _ = train_step(d, c, True)
             cent[g, s * ncs:(s + 1) * ncs] = c
     assigns = np.zeros((G, N), dtype=np.int64)
-    vsum = torch.zeros(G, nc, D, dtype=torch.bfloat16)
+    vsum = torch.zeros(G, nc, D, dtype=value.dtype)
     lists, sizes = [], []
     for g in range(G):
         c, a, cnt = train_step(key[g], cent[g], False)

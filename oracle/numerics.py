@@ -20,3 +20,13 @@ def bf16_ulp(x: torch.Tensor) -> torch.Tensor:
     a = x.abs().to(torch.float32).clamp_min(2.0 ** -126)
     e = torch.floor(torch.log2(a))
     return torch.exp2(e - 7)
+
+
+def ulp16(x: torch.Tensor, dtype=torch.bfloat16) -> torch.Tensor:
+    """spacing of the numbers of a 16-bit float type at |x|: bfloat16 (8 significant bits) or float16
+    (11 significant bits, subnormal below 2^-14)."""
+    if dtype == torch.bfloat16:
+        return bf16_ulp(x)
+    a = x.abs().to(torch.float32).clamp_min(2.0 ** -14)
+    e = torch.floor(torch.log2(a))
+    return torch.exp2(e - 10)

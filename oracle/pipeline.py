@@ -37,11 +37,11 @@ def decode_step(q, steady_k, steady_v, static_len, centroids, value_sum, mask, s
     BG, gs, D = q.shape
     scale = 1.0 / math.sqrt(D)
     x = scoring.logits_fp32(q, centroids, scale) if logits is None else logits
-    _, _, _, soft = scoring.softmax_from_logits(x if zone_logits is None else zone_logits)
+    _, _, _, soft = scoring.softmax_from_logits(x if zone_logits is None else zone_logits, q.dtype)
     dist = scoring.dist_from_softmax(soft, mask)
     ret, est = scoring.select(dist, nprobe, es)
     kept, offs = scoring.retrieval_layout(ret, size_i32, page, max_pages)
-    out = torch.empty(BG, gs, D, dtype=torch.bfloat16)
+    out = torch.empty(BG, gs, D, dtype=q.dtype)
     for g in range(BG):
         ks, vs = [steady_k[g, :static_len]], [steady_v[g, :static_len]]
         for c in ret[g, :int(kept[g])]:
@@ -50,7 +50,7 @@ def decode_step(q, steady_k, steady_v, static_len, centroids, value_sum, mask, s
         po = pl = None
         if es > 0:
             eo, el = attention.estimation(x[g:g + 1], est[g:g + 1], value_sum[g:g + 1], size_bf16[g:g + 1])
-            po, pl = eo.to(torch.bfloat16), el.float()
+            po, pl = eo.to(q.dtype), el.float()
         out[g] = attention.weighted_flash_decoding(q[g:g + 1], torch.cat(ks)[None], torch.cat(vs)[None], None,
                                                    po, pl)[0][0]
     return out, dict(dist=dist, ret=ret, est=est, kept=kept, offs=offs, logits=x)

@@ -18,13 +18,14 @@ def logits_fp32(q: torch.Tensor, cent: torch.Tensor, scale: float) -> torch.Tens
     return acc * torch.tensor(scale, dtype=torch.float32)
 
 
-def softmax_from_logits(x: torch.Tensor):
-    """(D bf16, row max, 1/row sum, Softmax bf16) from fp32 logits x [BG, gs, nc]."""
-    D = x.to(torch.bfloat16)
+def softmax_from_logits(x: torch.Tensor, dtype=torch.bfloat16):
+    """(D, row max, 1/row sum, Softmax) from fp32 logits x [BG, gs, nc]; D and Softmax in the 16-bit element
+    type of the operator's tensors (bfloat16 or float16: batch_gemm_softmax.cu:185-197)."""
+    D = x.to(dtype)
     m = x.max(dim=-1, keepdim=True).values
     z = torch.exp(x - m).sum(dim=-1, keepdim=True)
     inv = 1.0 / z
-    soft = (torch.exp(D.float() - m) * inv).to(torch.bfloat16)
+    soft = (torch.exp(D.float() - m) * inv).to(dtype)
     return D, m.squeeze(-1), inv.squeeze(-1), soft
 
 
@@ -32,15 +33,15 @@ def batch_gemm_softmax(q, cent, scale=None):
     """Reference semantics of batch_gemm_softmax: returns (D, norm, inv_sum, softmax)."""
     if scale is None:
         scale = 1.0 / math.sqrt(q.shape[-1])
-    return softmax_from_logits(logits_fp32(q, cent, scale))
+    return softmax_from_logits(logits_fp32(q, cent, scale), q.dtype)
 
 
 def dist_from_softmax(soft: torch.Tensor, mask: torch.Tensor = None) -> torch.Tensor:
-    """dist = bf16(sum_j float(P_j)), masked clusters -> finfo(bf16).min
+    """dist = dtype(sum_j float(P_j)) in the element type of the softmax, masked clusters -> finfo(dtype).min
     (cache_hub/retroinfer_cache.py:572-573)."""
-    d = soft.float().sum(dim=1).to(torch.bfloat16)
+    d = soft.float().sum(dim=1).to(soft.dtype)
     if mask is not None:
-        d = d.masked_fill(mask.bool(), BF16_MIN)
+        d = d.masked_fill(mask.bool(), torch.finfo(soft.dtype).min)
     return d
 
 

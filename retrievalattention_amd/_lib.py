@@ -21,26 +21,36 @@ SIGNATURES = {
     "ri_batch_gemm_softmax_f16": (I, [P, P, P, P, P, P, I, I, I, I, F, F, P]),
     "ri_score_select_workspace_bytes": (SZ, [I, I, I]),
     "ri_score_select": (I, [P] * 13 + [I, P, I, I, I, I, I, I, I, F, P, SZ, P]),
+    "ri_score_select_f16": (I, [P] * 13 + [I, P, I, I, I, I, I, I, I, F, P, SZ, P]),
     "ri_score_logits": (I, [P, P, P, I, I, I, F, P, SZ, P]),
+    "ri_score_logits_f16": (I, [P, P, P, I, I, I, F, P, SZ, P]),
     "ri_flash_decoding_workspace_bytes": (SZ, [I, I]),
     "ri_attention_workspace_reset": (I, [P, SZ, P]),
     "ri_weighted_flash_decoding": (I, [P, P, P, P, P, P, P, P, P, I, I, I, I64, F, P, SZ, P]),
+    "ri_weighted_flash_decoding_f16": (I, [P, P, P, P, P, P, P, P, P, I, I, I, I64, F, P, SZ, P]),
     "ri_wave_attention_workspace_bytes": (SZ, [I, I]),
     "ri_wave_attention": (I, [P, P, P, I64, I, P, P, P, I64, P, I, P, P, I, P, P, P, P, P, P, P, P, I, I, I, I, F, P, SZ, P]),
+    "ri_wave_attention_f16": (I, [P, P, P, I64, I, P, P, P, I64, P, I, P, P, I, P, P, P, P, P, P, P, P, I, I, I, I, F, P, SZ, P]),
     "ri_wave_attention_part": (I, [P, P, P, I64, I, P, P, P, I64, P, I, I, I, P, P, P, P, P, P, P, P, P, P, I, I, I, I, F, P, SZ, P]),
+    "ri_wave_attention_part_f16": (I, [P, P, P, I64, I, P, P, P, I64, P, I, I, I, P, P, P, P, P, P, P, P, P, P, I, I, I, I, F, P, SZ, P]),
     "ri_wave_attention_static_scratch_bytes": (SZ, []),
     "ri_wave_attention_static": (I, [P, P, P, I64, I, P, P, P, I64, P, I, P, P, I, P, P, P, P, P, P, P, P, I, I, I, I, F, P]),
+    "ri_wave_attention_static_f16": (I, [P, P, P, I64, I, P, P, P, I64, P, I, P, P, I, P, P, P, P, P, P, P, P, I, I, I, I, F, P]),
     "ri_buffer_attention": (I, [P, P, P, I64, P, I, P, P, P, P, P, I, I, I, I, F, P, SZ, P]),
+    "ri_buffer_attention_f16": (I, [P, P, P, I64, P, I, P, P, P, P, P, I, I, I, I, F, P, SZ, P]),
     "ri_lru_access_update": (I, [P, P, P, I, P, I, P, P, I, P, I, P, P, P] + [P] * 12 + [P, I, I, P] + [I] * 6 + [P]),
     "ri_gather_copy_vectors": (I, [P, P, P, P, P, P, P, I, I, I, I, I, I, P]),
     "ri_gather_copy_and_concat": (I, [P] * 17 + [I] * 7 + [P]),
     "ri_gather_copy_and_scatter": (I, [P] * 8 + [I] * 5 + [P]),
     "ri_kmeans_assign": (I, [P, P, P, I, I, I, I, I64, P]),
+    "ri_kmeans_assign_f16": (I, [P, P, P, I, I, I, I, I64, P]),
     "ri_kmeans_workspace_bytes": (SZ, [I, I, I]),
     "ri_kmeans_build_lists": (I, [P, P, P, P, I, I, I, P, SZ, P]),
     "ri_kmeans_reduce_workspace_bytes": (SZ, [I, I, I]),
     "ri_kmeans_update": (I, [P, P, P, P, P, I, I, I, I, I64, I, P, SZ, P]),
+    "ri_kmeans_update_f16": (I, [P, P, P, P, P, I, I, I, I, I64, I, P, SZ, P]),
     "ri_kmeans_value_sum": (I, [P, P, P, P, P, I, I, I, P, SZ, P]),
+    "ri_kmeans_value_sum_f16": (I, [P, P, P, P, P, I, I, I, P, SZ, P]),
     "ri_permute_rows": (I, [P, P, P, I, I, I64, I64, P]),
     "ri_threadpool_create": (P, [I]),
     "ri_threadpool_create_pinned": (P, [I, I]),

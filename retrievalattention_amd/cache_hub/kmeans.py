@@ -69,7 +69,7 @@ _MAX_GRAPHS = 4
 def segment_k_means_csr(key, value, num_centroids, num_iters=10, num_segments=1, init_indices=None,
                         reuse_graph=False):
     """Runs the clustering and returns a KMeansResult (no dense cluster lists, no host copy).
-    key/value [G, N, 128] bf16 contiguous device tensors.
+    key/value [G, N, 128] bfloat16 or float16 contiguous device tensors.
 
     reuse_graph (off unless asked for): the second call with keys at the same address and the same
     shape and parameters captures the launches into a HIP graph, and later such calls replay it.
@@ -78,8 +78,10 @@ def segment_k_means_csr(key, value, num_centroids, num_iters=10, num_segments=1,
     turn this on (prefill_update_kv_cache does: it copies everything into the cache's tensors at once;
     value sums are always fresh)."""
     G, N, D = key.shape
-    if D != 128 or key.dtype != torch.bfloat16 or not key.is_contiguous():
-        raise ValueError("segment_k_means: expected contiguous bf16 [G, N, 128] keys")
+    if D != 128 or key.dtype not in (torch.bfloat16, torch.float16) or not key.is_contiguous():
+        raise ValueError("segment_k_means: expected contiguous bfloat16 or float16 [G, N, 128] keys")
+    if value.dtype != key.dtype:
+        raise ValueError("segment_k_means: keys and values must have the same element type")
     if num_centroids % num_segments != 0:
         raise AssertionError("num_centroids must be divisible by num_segments")
     nc, S = num_centroids, num_segments

@@ -43,8 +43,8 @@ class retroinfer_cache(KV_Cache):
                  profiler_ranges=False, reference_stale_row=False):
         super().__init__(layer_num, batch_size, max_length, num_key_value_heads, num_heads, head_dim, dtype,
                          layer_mapping, num_gpus, model_size)
-        if head_dim != 128 or dtype != torch.bfloat16:
-            raise ValueError("the gfx950 kernels are built for head_dim 128 and bfloat16")
+        if head_dim != 128 or dtype not in (torch.bfloat16, torch.float16):
+            raise ValueError("the gfx950 kernels are built for head_dim 128 and bfloat16 or float16")
         if cache_unit_size != 8:
             raise ValueError("cache_unit_size must be 8 (block size of the copy kernels)")
         # limits of the kernels, checked here so that they surface at construction and not at the first decode step

@@ -93,7 +93,7 @@ __device__ __forceinline__ void wave_rows(int total, int nwaves, int wid, int* r
 // Merges the S split partials of group g (and the optional previous result) and writes the
 // output: wave w of the calling workgroup takes heads w, w+NW, ...; lanes first cover the splits
 // (statistics), then two dims each.
-template <int GS_PAD, int NW>
+template <int GS_PAD, int NW, bool HALF>
 __device__ __forceinline__ void combine_group(const AttendParams& P, int g, int S, int lenA, int lenB) {
   const int gs = P.gs;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -122,9 +122,11 @@ __device__ __forceinline__ void combine_group(const AttendParams& P, int g, int 
     float A0 = 0.f, A1 = 0.f;
     if (P.prev_lse && pl != -INFINITY) {  // an empty earlier part carries no weight, whatever its output holds
       const float fp = __expf(pl - M);
+      float p0, p1;
+      ri_unpack2<HALF>(po, p0, p1);
       L += fp;
-      A0 = fp * __uint_as_float(po << 16);
-      A1 = fp * __uint_as_float(po & 0xffff0000u);
+      A0 = fp * p0;
+      A1 = fp * p1;
     }
 #pragma unroll
     for (int u = 0; u < CB_PRE; ++u) {
@@ -147,7 +149,8 @@ __device__ __forceinline__ void combine_group(const AttendParams& P, int g, int 
     }
     // nothing attended at all (an empty part): zeros and a log-sum-exp of -inf, not 0/0
     const bool any = L > 0.f;
-    const uint32_t o = (uint32_t)ri_f32_to_bf16(any ? A0 / L : 0.f) | ((uint32_t)ri_f32_to_bf16(any ? A1 / L : 0.f) << 16);
+    const uint32_t o = (uint32_t)ri_f32_to_e16<HALF>(any ? A0 / L : 0.f) |
+                       ((uint32_t)ri_f32_to_e16<HALF>(any ? A1 / L : 0.f) << 16);
     *reinterpret_cast<uint32_t*>(P.out + ((size_t)g * gs + j) * RI_DIM + 2 * lane) = o;
     if (lane == 0 && P.lse_out) P.lse_out[(size_t)g * gs + j] = M + __logf(L);
   }
@@ -166,7 +169,8 @@ __device__ __forceinline__ void combine_group(const AttendParams& P, int g, int 
 // arrivals) of a launch with the same number of waves per compute unit.
 // The rank tables of the retrieval zone (np + 1 token offsets, np first rows) live in dynamic LDS, sized by
 // the launch, so that any number of probes the selection accepts can be attended.
-template <int GS_PAD, int NW, int PF>
+// HALF: q, K, V, value sums, cluster sizes, weights and outputs are IEEE half instead of bfloat16.
+template <int GS_PAD, int NW, int PF, bool HALF>
 __global__ __launch_bounds__(64 * NW, GS_PAD == 16 ? 1 : 3) void attend_kernel(AttendParams P) {
   constexpr int NH = GS_PAD / 4;
   constexpr int NT = 64 * NW;
@@ -306,8 +310,8 @@ __global__ __launch_bounds__(64 * NW, GS_PAD == 16 ? 1 : 3) void attend_kernel(A
               d = rs ? rs[rb] : rb;
               if (!est_split && P.row_src && (d < P.src_lo || d >= P.src_hi)) d = -1;
             }
-            if (wB) w = ri_bf16_to_f32(wB[rb]);
-            if (wsrc) w = ri_bf16_to_f32(wsrc[d]);
+            if (wB) w = ri_e16_to_f32<HALF>(wB[rb]);
+            if (wsrc) w = ri_e16_to_f32<HALF>(wsrc[d]);
           }
         }
         dsc[i] = d;
@@ -335,9 +339,12 @@ __global__ __launch_bounds__(64 * NW, GS_PAD == 16 ? 1 : 3) void attend_kernel(A
       auto compute = [&](const uint4* bks, const uint4* vs_, int j) {
         f32x4_t acc = (f32x4_t){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-        for (int kk = 0; kk < 4; ++kk)
-          acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
-              ri_as_bf16x8(*reinterpret_cast<const uint4*>(qrow + kk * 32)), ri_as_bf16x8(bks[kk]), acc, 0, 0, 0);
+        for (int kk = 0; kk < 4; ++kk) {
+          const uint4 qv = *reinterpret_cast<const uint4*>(qrow + kk * 32);
+          acc = HALF ? __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8_t, qv),
+                                                              __builtin_bit_cast(f16x8_t, bks[kk]), acc, 0, 0, 0)
+                     : __builtin_amdgcn_mfma_f32_16x16x32_bf16(ri_as_bf16x8(qv), ri_as_bf16x8(bks[kk]), acc, 0, 0, 0);
+        }
         float sv[NH];
 #pragma unroll
         for (int i = 0; i < NH; ++i) {
@@ -352,7 +359,7 @@ __global__ __launch_bounds__(64 * NW, GS_PAD == 16 ? 1 : 3) void attend_kernel(A
         }
         const bool valid = dsc[j * 16 + n] >= 0;
         const float w = wsh[j * 16 + n];
-        chunk_update<GS_PAD>(st, sv, valid, w, vs_, vt, pb, al_sh, lane);
+        chunk_update<GS_PAD, HALF>(st, sv, valid, w, vs_, vt, pb, al_sh, lane);
       };
 #pragma unroll
       for (int s = 0; s < PF; ++s)
@@ -387,7 +394,7 @@ __global__ __launch_bounds__(64 * NW, GS_PAD == 16 ? 1 : 3) void attend_kernel(A
         float w = 0.f;
         if (row < s1) {
           d = ids[row];
-          w = ri_bf16_to_f32(cs[d]);
+          w = ri_e16_to_f32<HALF>(cs[d]);
         }
         dsc[i] = d;
         wsh[i] = w;
@@ -421,7 +428,7 @@ __global__ __launch_bounds__(64 * NW, GS_PAD == 16 ? 1 : 3) void attend_kernel(A
           if (j < nch) {
             const bool valid = dsc[j * 16 + n] >= 0;
             const float w = wsh[j * 16 + n];
-            chunk_update<GS_PAD>(st, sc[s], valid, w, v[s], vt, pb, al_sh, lane);
+            chunk_update<GS_PAD, HALF>(st, sc[s], valid, w, v[s], vt, pb, al_sh, lane);
             if (j + PF < nch) issue(sc[s], v[s], j + PF);
           }
         }
@@ -502,7 +509,7 @@ __global__ __launch_bounds__(64 * NW, GS_PAD == 16 ? 1 : 3) void attend_kernel(A
     sh_last = (__hip_atomic_fetch_add(&P.counters[g], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == S - 1);
   __syncthreads();
   if (!sh_last) return;
-  combine_group<GS_PAD, NW>(P, g, S, lenA_all, lenB);
+  combine_group<GS_PAD, NW, HALF>(P, g, S, lenA_all, lenB);
   // ready for the next launch (every arrival of this launch has been counted; launches that share the
   // workspace do not overlap)
   if (threadIdx.x == 0) __hip_atomic_store(&P.counters[g], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -539,16 +546,21 @@ static void carve_workspace(AttendParams& P, void* workspace, int BG, int gp) {
   P.part_acc = P.part_ml + (size_t)BG * S * gp * 2;
 }
 
-static int launch_attend(AttendParams& P, int BG, int gs, int nw, hipStream_t s) {
+template <bool HALF>
+static void launch_attend_t(const AttendParams& P, dim3 grid, int gp, int nw, size_t tab_bytes, hipStream_t s) {
+  if (nw == 8 && gp == 4) attend_kernel<4, 8, 1, HALF><<<grid, 512, tab_bytes, s>>>(P);
+  else if (nw == 8 && gp == 8) attend_kernel<8, 8, 1, HALF><<<grid, 512, tab_bytes, s>>>(P);
+  else if (gp == 4) attend_kernel<4, 4, 1, HALF><<<grid, 256, tab_bytes, s>>>(P);
+  else if (gp == 8) attend_kernel<8, 4, 1, HALF><<<grid, 256, tab_bytes, s>>>(P);
+  else attend_kernel<16, 4, 1, HALF><<<grid, 256, tab_bytes, s>>>(P);
+}
+
+static int launch_attend(AttendParams& P, int BG, int gs, int nw, bool half, hipStream_t s) {
   const int S = P.S_kv + P.S_es;
   const dim3 grid(S, BG);
   const size_t tab_bytes = P.ret_off ? (size_t)(2 * P.np + 1) * sizeof(int) : 0;
-  const int gp = gs_pad_of(gs);
-  if (nw == 8 && gp == 4) attend_kernel<4, 8, 1><<<grid, 512, tab_bytes, s>>>(P);
-  else if (nw == 8 && gp == 8) attend_kernel<8, 8, 1><<<grid, 512, tab_bytes, s>>>(P);
-  else if (gp == 4) attend_kernel<4, 4, 1><<<grid, 256, tab_bytes, s>>>(P);
-  else if (gp == 8) attend_kernel<8, 4, 1><<<grid, 256, tab_bytes, s>>>(P);
-  else attend_kernel<16, 4, 1><<<grid, 256, tab_bytes, s>>>(P);
+  if (half) launch_attend_t<true>(P, grid, gs_pad_of(gs), nw, tab_bytes, s);
+  else launch_attend_t<false>(P, grid, gs_pad_of(gs), nw, tab_bytes, s);
   RI_HIP_CHECK_LAUNCH();
   return RI_OK;
 }
@@ -607,11 +619,10 @@ static void plan_splits(int64_t kv_rows, int64_t es_rows, int es_row_bytes, int 
   *S_es = per_group - kv;
 }
 
-extern "C" int ri_weighted_flash_decoding(const void* q, const void* k, const void* v, const void* weight,
-                                          const int32_t* cache_seqlens, const void* prev_out,
-                                          const float* prev_lse, void* out, float* lse_out, int BG, int gs,
-                                          int S, int64_t kv_stride, float scale, void* workspace,
-                                          size_t workspace_bytes, ri_stream_t stream) {
+static int flash_decoding_impl(const void* q, const void* k, const void* v, const void* weight,
+                               const int32_t* cache_seqlens, const void* prev_out, const float* prev_lse, void* out,
+                               float* lse_out, int BG, int gs, int S, int64_t kv_stride, float scale, void* workspace,
+                               size_t workspace_bytes, bool half, ri_stream_t stream) {
   if (!q || !k || !v || !out || !workspace) return RI_ERR_ARG;
   if (ri_any_misaligned16(q, k, v, weight, prev_out, out, workspace)) return RI_ERR_ARG;
   if (BG <= 0 || BG > RI_MAX_GROUPS || gs <= 0 || gs > 16 || S < 0 || kv_stride < S) return RI_ERR_ARG;
@@ -638,7 +649,25 @@ extern "C" int ri_weighted_flash_decoding(const void* q, const void* k, const vo
   P.out = (uint16_t*)out;
   P.lse_out = lse_out;
   carve_workspace(P, workspace, BG, gp);
-  return launch_attend(P, BG, gs, nw, (hipStream_t)stream);
+  return launch_attend(P, BG, gs, nw, half, (hipStream_t)stream);
+}
+
+extern "C" int ri_weighted_flash_decoding(const void* q, const void* k, const void* v, const void* weight,
+                                          const int32_t* cache_seqlens, const void* prev_out,
+                                          const float* prev_lse, void* out, float* lse_out, int BG, int gs,
+                                          int S, int64_t kv_stride, float scale, void* workspace,
+                                          size_t workspace_bytes, ri_stream_t stream) {
+  return flash_decoding_impl(q, k, v, weight, cache_seqlens, prev_out, prev_lse, out, lse_out, BG, gs, S, kv_stride,
+                             scale, workspace, workspace_bytes, false, stream);
+}
+
+extern "C" int ri_weighted_flash_decoding_f16(const void* q, const void* k, const void* v, const void* weight,
+                                              const int32_t* cache_seqlens, const void* prev_out,
+                                              const float* prev_lse, void* out, float* lse_out, int BG, int gs,
+                                              int S, int64_t kv_stride, float scale, void* workspace,
+                                              size_t workspace_bytes, ri_stream_t stream) {
+  return flash_decoding_impl(q, k, v, weight, cache_seqlens, prev_out, prev_lse, out, lse_out, BG, gs, S, kv_stride,
+                             scale, workspace, workspace_bytes, true, stream);
 }
 
 // Shared body of ri_wave_attention and ri_wave_attention_static.  `scratch` holds the arrival
@@ -656,7 +685,7 @@ static int wave_attention_impl(const void* q, const void* steady_k, const void* 
                                const int32_t* meta, const int32_t* est_ids, const float* logits,
                                const void* est_centroids, const void* value_sum, const void* cluster_size_bf16,
                                void* out, int32_t* valid_lengths, int BG, int gs, int nc, int es, float scale,
-                               void* scratch, size_t scratch_bytes, bool clear_counters, hipStream_t stream,
+                               void* scratch, size_t scratch_bytes, bool clear_counters, bool half, hipStream_t stream,
                                int src_lo = INT32_MIN, int src_hi = INT32_MAX, const void* prev_out = nullptr,
                                const float* prev_lse = nullptr, float* lse_out = nullptr) {
   if (!q || !steady_k || !steady_v || !store_k || !store_v || !meta || !out || !scratch) return RI_ERR_ARG;
@@ -716,7 +745,7 @@ static int wave_attention_impl(const void* q, const void* steady_k, const void* 
     attend_clear_counters_kernel<<<(BG + 255) / 256, 256, 0, stream>>>(P.counters, BG);
     RI_HIP_CHECK_LAUNCH();
   }
-  return launch_attend(P, BG, gs, nw, stream);
+  return launch_attend(P, BG, gs, nw, half, stream);
 }
 
 // Clears the arrival counters at the head of an attention workspace with a small kernel on `stream` (no
@@ -732,6 +761,23 @@ extern "C" int ri_attention_workspace_reset(void* workspace, size_t workspace_by
   return RI_OK;
 }
 
+static int ri_wave_attention_any(const void* q, const void* steady_k, const void* steady_v,
+                                 int64_t steady_stride, int static_len, const int32_t* static_len_dev,
+                                 const void* store_k,
+                                 const void* store_v, int64_t store_stride, const int32_t* row_src,
+                                 int row_src_stride, const int32_t* ret_tok_off, const int32_t* ret_start, int np,
+                                 const int32_t* meta, const int32_t* est_ids,
+                                 const float* logits, const void* est_centroids, const void* value_sum,
+                                 const void* cluster_size_bf16, void* out, int32_t* valid_lengths, int BG, int gs,
+                                 int nc, int es, float scale, void* workspace, size_t workspace_bytes,
+                                 ri_stream_t stream, bool half) {
+  if (workspace && workspace_bytes < attn_workspace_bytes(BG, gs)) return RI_ERR_WORKSPACE;
+  return wave_attention_impl(q, steady_k, steady_v, steady_stride, static_len, static_len_dev, store_k, store_v,
+                             store_stride, row_src, row_src_stride, ret_tok_off, ret_start, np, meta, est_ids, logits,
+                             est_centroids, value_sum, cluster_size_bf16, out, valid_lengths, BG, gs, nc, es, scale,
+                             workspace, workspace_bytes, false, half, (hipStream_t)stream);
+}
+
 extern "C" int ri_wave_attention(const void* q, const void* steady_k, const void* steady_v,
                                  int64_t steady_stride, int static_len, const int32_t* static_len_dev,
                                  const void* store_k,
@@ -742,11 +788,20 @@ extern "C" int ri_wave_attention(const void* q, const void* steady_k, const void
                                  const void* cluster_size_bf16, void* out, int32_t* valid_lengths, int BG, int gs,
                                  int nc, int es, float scale, void* workspace, size_t workspace_bytes,
                                  ri_stream_t stream) {
-  if (workspace && workspace_bytes < attn_workspace_bytes(BG, gs)) return RI_ERR_WORKSPACE;
-  return wave_attention_impl(q, steady_k, steady_v, steady_stride, static_len, static_len_dev, store_k, store_v,
-                             store_stride, row_src, row_src_stride, ret_tok_off, ret_start, np, meta, est_ids, logits,
-                             est_centroids, value_sum, cluster_size_bf16, out, valid_lengths, BG, gs, nc, es, scale,
-                             workspace, workspace_bytes, false, (hipStream_t)stream);
+  return ri_wave_attention_any(q, steady_k, steady_v, steady_stride, static_len, static_len_dev, store_k, store_v, store_stride, row_src, row_src_stride, ret_tok_off, ret_start, np, meta, est_ids, logits, est_centroids, value_sum, cluster_size_bf16, out, valid_lengths, BG, gs, nc, es, scale, workspace, workspace_bytes, stream, false);
+}
+
+extern "C" int ri_wave_attention_f16(const void* q, const void* steady_k, const void* steady_v,
+                                 int64_t steady_stride, int static_len, const int32_t* static_len_dev,
+                                 const void* store_k,
+                                 const void* store_v, int64_t store_stride, const int32_t* row_src,
+                                 int row_src_stride, const int32_t* ret_tok_off, const int32_t* ret_start, int np,
+                                 const int32_t* meta, const int32_t* est_ids,
+                                 const float* logits, const void* est_centroids, const void* value_sum,
+                                 const void* cluster_size_bf16, void* out, int32_t* valid_lengths, int BG, int gs,
+                                 int nc, int es, float scale, void* workspace, size_t workspace_bytes,
+                                 ri_stream_t stream) {
+  return ri_wave_attention_any(q, steady_k, steady_v, steady_stride, static_len, static_len_dev, store_k, store_v, store_stride, row_src, row_src_stride, ret_tok_off, ret_start, np, meta, est_ids, logits, est_centroids, value_sum, cluster_size_bf16, out, valid_lengths, BG, gs, nc, es, scale, workspace, workspace_bytes, stream, true);
 }
 
 // Part of a wave attention: the steady zone and estimation zone as asked for, and of the rows of the row
@@ -754,6 +809,26 @@ extern "C" int ri_wave_attention(const void* q, const void* steady_k, const void
 // as (prev_out, prev_lse) and this part's log-sum-exp goes out, so that two launches over disjoint row
 // windows give the attention over all rows.  Used with a host-resident store: the rows already in the
 // block cache are attended while the missed blocks are still being staged, and the staged rows follow.
+static int ri_wave_attention_part_any(const void* q, const void* steady_k, const void* steady_v,
+                                      int64_t steady_stride, int static_len, const int32_t* static_len_dev,
+                                      const void* store_k, const void* store_v, int64_t store_stride,
+                                      const int32_t* row_src, int row_src_stride, int src_row_lo, int src_row_hi,
+                                      const int32_t* meta, const int32_t* est_ids, const float* logits,
+                                      const void* value_sum, const void* cluster_size_bf16, const void* prev_out,
+                                      const float* prev_lse, void* out, float* lse_out, int32_t* valid_lengths,
+                                      int BG, int gs, int nc, int es, float scale, void* workspace,
+                                      size_t workspace_bytes, ri_stream_t stream, bool half) {
+  if (!row_src || src_row_lo >= src_row_hi) return RI_ERR_ARG;
+  if (workspace && workspace_bytes < attn_workspace_bytes(BG, gs)) return RI_ERR_WORKSPACE;
+  // a part that leaves the steady zone out must not pick its length up from the device either
+  if (static_len == 0) static_len_dev = nullptr;
+  return wave_attention_impl(q, steady_k, steady_v, steady_stride, static_len, static_len_dev, store_k, store_v,
+                             store_stride, row_src, row_src_stride, nullptr, nullptr, 0, meta, est_ids, logits, nullptr,
+                             value_sum, cluster_size_bf16, out, valid_lengths, BG, gs, nc, es, scale, workspace,
+                             workspace_bytes, false, half, (hipStream_t)stream, src_row_lo, src_row_hi, prev_out, prev_lse,
+                             lse_out);
+}
+
 extern "C" int ri_wave_attention_part(const void* q, const void* steady_k, const void* steady_v,
                                       int64_t steady_stride, int static_len, const int32_t* static_len_dev,
                                       const void* store_k, const void* store_v, int64_t store_stride,
@@ -763,15 +838,19 @@ extern "C" int ri_wave_attention_part(const void* q, const void* steady_k, const
                                       const float* prev_lse, void* out, float* lse_out, int32_t* valid_lengths,
                                       int BG, int gs, int nc, int es, float scale, void* workspace,
                                       size_t workspace_bytes, ri_stream_t stream) {
-  if (!row_src || src_row_lo >= src_row_hi) return RI_ERR_ARG;
-  if (workspace && workspace_bytes < attn_workspace_bytes(BG, gs)) return RI_ERR_WORKSPACE;
-  // a part that leaves the steady zone out must not pick its length up from the device either
-  if (static_len == 0) static_len_dev = nullptr;
-  return wave_attention_impl(q, steady_k, steady_v, steady_stride, static_len, static_len_dev, store_k, store_v,
-                             store_stride, row_src, row_src_stride, nullptr, nullptr, 0, meta, est_ids, logits, nullptr,
-                             value_sum, cluster_size_bf16, out, valid_lengths, BG, gs, nc, es, scale, workspace,
-                             workspace_bytes, false, (hipStream_t)stream, src_row_lo, src_row_hi, prev_out, prev_lse,
-                             lse_out);
+  return ri_wave_attention_part_any(q, steady_k, steady_v, steady_stride, static_len, static_len_dev, store_k, store_v, store_stride, row_src, row_src_stride, src_row_lo, src_row_hi, meta, est_ids, logits, value_sum, cluster_size_bf16, prev_out, prev_lse, out, lse_out, valid_lengths, BG, gs, nc, es, scale, workspace, workspace_bytes, stream, false);
+}
+
+extern "C" int ri_wave_attention_part_f16(const void* q, const void* steady_k, const void* steady_v,
+                                      int64_t steady_stride, int static_len, const int32_t* static_len_dev,
+                                      const void* store_k, const void* store_v, int64_t store_stride,
+                                      const int32_t* row_src, int row_src_stride, int src_row_lo, int src_row_hi,
+                                      const int32_t* meta, const int32_t* est_ids, const float* logits,
+                                      const void* value_sum, const void* cluster_size_bf16, const void* prev_out,
+                                      const float* prev_lse, void* out, float* lse_out, int32_t* valid_lengths,
+                                      int BG, int gs, int nc, int es, float scale, void* workspace,
+                                      size_t workspace_bytes, ri_stream_t stream) {
+  return ri_wave_attention_part_any(q, steady_k, steady_v, steady_stride, static_len, static_len_dev, store_k, store_v, store_stride, row_src, row_src_stride, src_row_lo, src_row_hi, meta, est_ids, logits, value_sum, cluster_size_bf16, prev_out, prev_lse, out, lse_out, valid_lengths, BG, gs, nc, es, scale, workspace, workspace_bytes, stream, true);
 }
 
 // ------------------------------------------------------------------------------------
@@ -811,6 +890,26 @@ extern "C" size_t ri_wave_attention_static_scratch_bytes(void) {
   return RI_STATIC_SCRATCH_BYTES;
 }
 
+static int ri_wave_attention_static_any(const void* q, const void* steady_k, const void* steady_v,
+                                        int64_t steady_stride, int static_len, const int32_t* static_len_dev,
+                                        const void* store_k, const void* store_v, int64_t store_stride,
+                                        const int32_t* row_src, int row_src_stride, const int32_t* ret_tok_off,
+                                        const int32_t* ret_start, int np, const int32_t* meta,
+                                        const int32_t* est_ids, const float* logits, const void* est_centroids,
+                                        const void* value_sum, const void* cluster_size_bf16, void* out,
+                                        int32_t* valid_lengths, int BG, int gs, int nc, int es, float scale,
+                                        ri_stream_t stream, bool half) {
+  void* ptr = nullptr;
+  const int rc = static_scratch_ptr(&ptr);
+  if (rc) return rc;
+  // the array keeps what the previous call left: the counters are cleared by a kernel on the caller's
+  // stream (a fill kernel, not a memset, so that the call can be captured into a graph)
+  return wave_attention_impl(q, steady_k, steady_v, steady_stride, static_len, static_len_dev, store_k, store_v,
+                             store_stride, row_src, row_src_stride, ret_tok_off, ret_start, np, meta, est_ids, logits,
+                             est_centroids, value_sum, cluster_size_bf16, out, valid_lengths, BG, gs, nc, es, scale, ptr,
+                             RI_STATIC_SCRATCH_BYTES, true, half, (hipStream_t)stream);
+}
+
 extern "C" int ri_wave_attention_static(const void* q, const void* steady_k, const void* steady_v,
                                         int64_t steady_stride, int static_len, const int32_t* static_len_dev,
                                         const void* store_k, const void* store_v, int64_t store_stride,
@@ -820,22 +919,26 @@ extern "C" int ri_wave_attention_static(const void* q, const void* steady_k, con
                                         const void* value_sum, const void* cluster_size_bf16, void* out,
                                         int32_t* valid_lengths, int BG, int gs, int nc, int es, float scale,
                                         ri_stream_t stream) {
-  void* ptr = nullptr;
-  const int rc = static_scratch_ptr(&ptr);
-  if (rc) return rc;
-  // the array keeps what the previous call left: the counters are cleared by a kernel on the caller's
-  // stream (a fill kernel, not a memset, so that the call can be captured into a graph)
-  return wave_attention_impl(q, steady_k, steady_v, steady_stride, static_len, static_len_dev, store_k, store_v,
-                             store_stride, row_src, row_src_stride, ret_tok_off, ret_start, np, meta, est_ids, logits,
-                             est_centroids, value_sum, cluster_size_bf16, out, valid_lengths, BG, gs, nc, es, scale, ptr,
-                             RI_STATIC_SCRATCH_BYTES, true, (hipStream_t)stream);
+  return ri_wave_attention_static_any(q, steady_k, steady_v, steady_stride, static_len, static_len_dev, store_k, store_v, store_stride, row_src, row_src_stride, ret_tok_off, ret_start, np, meta, est_ids, logits, est_centroids, value_sum, cluster_size_bf16, out, valid_lengths, BG, gs, nc, es, scale, stream, false);
 }
 
-extern "C" int ri_buffer_attention(const void* q, const void* buf_k, const void* buf_v, int64_t buf_stride,
+extern "C" int ri_wave_attention_static_f16(const void* q, const void* steady_k, const void* steady_v,
+                                        int64_t steady_stride, int static_len, const int32_t* static_len_dev,
+                                        const void* store_k, const void* store_v, int64_t store_stride,
+                                        const int32_t* row_src, int row_src_stride, const int32_t* ret_tok_off,
+                                        const int32_t* ret_start, int np, const int32_t* meta,
+                                        const int32_t* est_ids, const float* logits, const void* est_centroids,
+                                        const void* value_sum, const void* cluster_size_bf16, void* out,
+                                        int32_t* valid_lengths, int BG, int gs, int nc, int es, float scale,
+                                        ri_stream_t stream) {
+  return ri_wave_attention_static_any(q, steady_k, steady_v, steady_stride, static_len, static_len_dev, store_k, store_v, store_stride, row_src, row_src_stride, ret_tok_off, ret_start, np, meta, est_ids, logits, est_centroids, value_sum, cluster_size_bf16, out, valid_lengths, BG, gs, nc, es, scale, stream, true);
+}
+
+static int ri_buffer_attention_any(const void* q, const void* buf_k, const void* buf_v, int64_t buf_stride,
                                    const int32_t* cache_seqlens, int max_len, const int32_t* est_ids,
                                    const float* logits, const void* value_sum, const void* cluster_size_bf16,
                                    void* out, int BG, int gs, int nc, int es, float scale, void* workspace,
-                                   size_t workspace_bytes, ri_stream_t stream) {
+                                   size_t workspace_bytes, ri_stream_t stream, bool half) {
   if (!q || !buf_k || !buf_v || !cache_seqlens || !out || !workspace) return RI_ERR_ARG;
   if (ri_any_misaligned16(q, buf_k, buf_v, value_sum, out, workspace)) return RI_ERR_ARG;
   if (BG <= 0 || BG > RI_MAX_GROUPS || gs <= 0 || gs > 16 || max_len <= 0 || max_len > buf_stride || es < 0 ||
@@ -866,6 +969,22 @@ extern "C" int ri_buffer_attention(const void* q, const void* buf_k, const void*
   const int nw = attend_waves(gs);
   plan_splits(max_len / 4 + 64, es, est_row_bytes(gs, false), BG, nw, &P.S_kv, &P.S_es);
   carve_workspace(P, workspace, BG, gp);
-  return launch_attend(P, BG, gs, nw, (hipStream_t)stream);
+  return launch_attend(P, BG, gs, nw, half, (hipStream_t)stream);
+}
+
+extern "C" int ri_buffer_attention(const void* q, const void* buf_k, const void* buf_v, int64_t buf_stride,
+                                   const int32_t* cache_seqlens, int max_len, const int32_t* est_ids,
+                                   const float* logits, const void* value_sum, const void* cluster_size_bf16,
+                                   void* out, int BG, int gs, int nc, int es, float scale, void* workspace,
+                                   size_t workspace_bytes, ri_stream_t stream) {
+  return ri_buffer_attention_any(q, buf_k, buf_v, buf_stride, cache_seqlens, max_len, est_ids, logits, value_sum, cluster_size_bf16, out, BG, gs, nc, es, scale, workspace, workspace_bytes, stream, false);
+}
+
+extern "C" int ri_buffer_attention_f16(const void* q, const void* buf_k, const void* buf_v, int64_t buf_stride,
+                                   const int32_t* cache_seqlens, int max_len, const int32_t* est_ids,
+                                   const float* logits, const void* value_sum, const void* cluster_size_bf16,
+                                   void* out, int BG, int gs, int nc, int es, float scale, void* workspace,
+                                   size_t workspace_bytes, ri_stream_t stream) {
+  return ri_buffer_attention_any(q, buf_k, buf_v, buf_stride, cache_seqlens, max_len, est_ids, logits, value_sum, cluster_size_bf16, out, BG, gs, nc, es, scale, workspace, workspace_bytes, stream, true);
 }
 

@@ -29,7 +29,10 @@ struct WaveState {
   f32x4_t acc[8];
 };
 
-__device__ __forceinline__ uint16_t ri_to_bf16_hw(float x) {
+// probability -> the 16-bit element type of the P.V operands (hardware conversion, round to nearest even)
+template <bool HALF>
+__device__ __forceinline__ uint16_t ri_p_to_e16(float x) {
+  if (HALF) return __builtin_bit_cast(uint16_t, (_Float16)x);
   const __bf16 b = (__bf16)x;
   return __builtin_bit_cast(uint16_t, b);
 }
@@ -41,7 +44,7 @@ __device__ __forceinline__ uint16_t ri_to_bf16_hw(float x) {
 // row-major; P·V = 8 MFMA 16x16x16 whose B operands come from LDS transpose reads
 // (ds_read_b64_tr_b16: lane l of a 16-lane group receives element l%4 of the 8-byte pieces
 // addressed by lanes l/4, l/4+4, l/4+8, l/4+12 — four consecutive rows of one column).
-template <int GS_PAD>
+template <int GS_PAD, bool HALF>
 __device__ __forceinline__ void chunk_update(WaveState<GS_PAD>& st, const float* sv, bool valid, float w,
                                              const uint4 v[4], uint16_t* vt, uint16_t* pb, float* al_sh,
                                              int lane) {
@@ -72,7 +75,7 @@ __device__ __forceinline__ void chunk_update(WaveState<GS_PAD>& st, const float*
     rescale |= (al[i] != 1.f);
     st.l[i] = st.l[i] * al[i] + w * p;
     st.m[i] = mn;
-    pb[ri_head_of<GS_PAD>(h, i) * 16 + n] = ri_to_bf16_hw(p);
+    pb[ri_head_of<GS_PAD>(h, i) * 16 + n] = ri_p_to_e16<HALF>(p);
   }
   // the running maximum rarely moves after the first chunks: rescale only when some head's did
   const bool any_rescale = __any(rescale);
@@ -97,7 +100,11 @@ __device__ __forceinline__ void chunk_update(WaveState<GS_PAD>& st, const float*
   for (int dt = 0; dt < 8; ++dt) {
     const bf16x4s_t vb = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
         (bf16x4s_t __attribute__((address_space(3)))*)(vsrc + 16 * dt));
-    st.acc[dt] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(pa, vb, st.acc[dt], 0, 0, 0);
+    if (HALF)
+      st.acc[dt] = __builtin_amdgcn_mfma_f32_16x16x16f16(__builtin_bit_cast(f16x4_t, pa), __builtin_bit_cast(f16x4_t, vb),
+                                                         st.acc[dt], 0, 0, 0);
+    else
+      st.acc[dt] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(pa, vb, st.acc[dt], 0, 0, 0);
   }
   __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
   __builtin_amdgcn_wave_barrier();  // the tile and P are rewritten by the next chunk

@@ -45,7 +45,8 @@ __device__ __forceinline__ size_t km_row0(int p, int seg, int64_t head_rows, int
 // row (i/4)*8 + (l/32)*4 + i%4, column l%32.  nc is a multiple of 32; the last tile may hold
 // fewer sub-tiles.
 // ------------------------------------------------------------------------------------
-template <int KM_TT, int KM_CT>
+// HALF: keys and centroids are IEEE half instead of bfloat16.
+template <int KM_TT, int KM_CT, bool HALF>
 __global__ __launch_bounds__(KM_WAVES * 64) void km_assign_kernel(const uint16_t* __restrict__ data,
                                                                   const uint16_t* __restrict__ cent,
                                                                   int32_t* __restrict__ assign, int N, int nc,
@@ -119,8 +120,10 @@ __global__ __launch_bounds__(KM_WAVES * 64) void km_assign_kernel(const uint16_t
           const uint4 a = *reinterpret_cast<const uint4*>(&sh_c[buf][half * 32 + r][((kk * 2 + hh) ^ (r & 15)) * 8]);
 #pragma unroll
           for (int tt = 0; tt < KM_TT; ++tt)
-            acc[tt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ri_as_bf16x8(a), ri_as_bf16x8(b[tt][kk]), acc[tt], 0, 0,
-                                                              0);
+            acc[tt] = HALF ? __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8_t, a),
+                                                                    __builtin_bit_cast(f16x8_t, b[tt][kk]), acc[tt], 0, 0, 0)
+                           : __builtin_amdgcn_mfma_f32_32x32x16_bf16(ri_as_bf16x8(a), ri_as_bf16x8(b[tt][kk]), acc[tt], 0,
+                                                                     0, 0);
         }
         // argmax epilogue: the lane's 16 scores are in ascending row order, so the first score
         // equal to their maximum is the lowest row; the index search only runs when some lane
@@ -452,6 +455,7 @@ __global__ __launch_bounds__(256) void km_counts_kernel(const int32_t* __restric
 // member ids with one load, the ids are broadcast from the lanes, and the sixteen row loads are all
 // in flight before the first add; a short last round adds +0 for its missing rows, which changes no
 // sum.  (Two dependent round trips per sixteen rows instead of two per row for a list's tail.)
+template <bool HALF>
 __device__ __forceinline__ void km_sum_rows(const uint32_t* __restrict__ rp, const int32_t* __restrict__ mem, int k0,
                                             int k1, float& s0, float& s1) {
   const int lane = threadIdx.x & 63;
@@ -466,13 +470,15 @@ __device__ __forceinline__ void km_sum_rows(const uint32_t* __restrict__ rp, con
     }
 #pragma unroll
     for (int j = 0; j < 16; ++j) {
-      s0 += __uint_as_float(v[j] << 16);
-      s1 += __uint_as_float(v[j] & 0xffff0000u);
+      float x0, x1;
+      ri_unpack2<HALF>(v[j], x0, x1);   // a missing row reads as the word 0 = (+0, +0) in either type
+      s0 += x0;
+      s1 += x1;
     }
   }
 }
 
-template <bool MEAN>
+template <bool MEAN, bool HALF>
 __device__ __forceinline__ void km_finish(float s0, float s1, int count, int normalize, uint32_t* op) {
   if (MEAN) {
     const float cnt = (float)count;
@@ -487,7 +493,7 @@ __device__ __forceinline__ void km_finish(float s0, float s1, int count, int nor
       s1 = s1 / nrm;
     }
   }
-  *op = (uint32_t)ri_f32_to_bf16(s0) | ((uint32_t)ri_f32_to_bf16(s1) << 16);
+  *op = (uint32_t)ri_f32_to_e16<HALF>(s0) | ((uint32_t)ri_f32_to_e16<HALF>(s1) << 16);
 }
 
 // slots of one problem: the last list starts below N and a slot index is at most 2 (N / KM_BLK) + 1
@@ -521,7 +527,7 @@ __device__ __forceinline__ int km_slot_owner(const int32_t* __restrict__ off, in
 // grid (item workgroups + ceil(nc / 4), P), four waves each.  The first item_wgs workgroups take
 // one slot per wave (blocks of long lists, their fp32 sums go to partial[p][slot]); the others one
 // cluster per wave.
-template <bool MEAN>
+template <bool MEAN, bool HALF>
 __global__ __launch_bounds__(256) void km_reduce_kernel(const uint16_t* __restrict__ rows,
                                                         const int32_t* __restrict__ counts,
                                                         const int32_t* __restrict__ offsets,
@@ -539,7 +545,7 @@ __global__ __launch_bounds__(256) void km_reduce_kernel(const uint16_t* __restri
     int s, o, j;
     if (km_slot_owner(off, nc, slot, s, o, j) < 0) return;
     float s0 = 0.f, s1 = 0.f;
-    km_sum_rows(rp, members + (size_t)p * N + o, j * KM_BLK, min(s, (j + 1) * KM_BLK), s0, s1);
+    km_sum_rows<HALF>(rp, members + (size_t)p * N + o, j * KM_BLK, min(s, (j + 1) * KM_BLK), s0, s1);
     partial[((size_t)p * cap + slot) * 64 + lane] = make_float2(s0, s1);
     return;
   }
@@ -553,13 +559,13 @@ __global__ __launch_bounds__(256) void km_reduce_kernel(const uint16_t* __restri
   }
   if (s > KM_BLK) return;  // summed by the slot waves, finished by km_reduce_fold_kernel
   float s0 = 0.f, s1 = 0.f;
-  km_sum_rows(rp, members + (size_t)p * N + off[c], 0, s, s0, s1);
-  km_finish<MEAN>(s0, s1, s, normalize, op);
+  km_sum_rows<HALF>(rp, members + (size_t)p * N + off[c], 0, s, s0, s1);
+  km_finish<MEAN, HALF>(s0, s1, s, normalize, op);
 }
 
 // grid (item workgroups, P): the wave of a long list's first slot adds the block sums in block
 // order and finishes the cluster
-template <bool MEAN>
+template <bool MEAN, bool HALF>
 __global__ __launch_bounds__(256) void km_reduce_fold_kernel(const int32_t* __restrict__ offsets,
                                                              const float2* __restrict__ partial,
                                                              uint16_t* __restrict__ out, int cap, int nc,
@@ -591,7 +597,7 @@ __global__ __launch_bounds__(256) void km_reduce_fold_kernel(const int32_t* __re
     t.y += v.y;
   }
   uint32_t* op = reinterpret_cast<uint32_t*>(out + ((size_t)p * nc + c) * RI_DIM) + lane;
-  km_finish<MEAN>(t.x, t.y, s, normalize, op);
+  km_finish<MEAN, HALF>(t.x, t.y, s, normalize, op);
 }
 
 // out[p, i, :] = in[p, members[p, i], :]; 16 lanes per row
@@ -635,21 +641,32 @@ static int km_assign_args(const void* data, const void* centroids, const int32_t
   return RI_OK;
 }
 
-extern "C" int ri_kmeans_assign(const void* data, const void* centroids, int32_t* assign, int P, int N,
-                                int nc, int seg, int64_t head_rows, ri_stream_t stream) {
+template <bool HALF>
+static int km_assign(const void* data, const void* centroids, int32_t* assign, int P, int N, int nc, int seg,
+                     int64_t head_rows, ri_stream_t stream) {
   int rc = km_assign_args(data, centroids, assign, P, N, nc, seg);
   if (rc) return rc;
   if (nc > KM_WIDE_MIN_NC) {
     constexpr int wg_tokens = KM_WAVES * 32 * 4;
-    km_assign_kernel<4, 128><<<dim3((N + wg_tokens - 1) / wg_tokens, P), KM_WAVES * 64, 0, (hipStream_t)stream>>>(
+    km_assign_kernel<4, 128, HALF><<<dim3((N + wg_tokens - 1) / wg_tokens, P), KM_WAVES * 64, 0, (hipStream_t)stream>>>(
         (const uint16_t*)data, (const uint16_t*)centroids, assign, N, nc, seg, head_rows);
   } else {
     constexpr int wg_tokens = KM_WAVES * 32 * 2;
-    km_assign_kernel<2, 32><<<dim3((N + wg_tokens - 1) / wg_tokens, P), KM_WAVES * 64, 0, (hipStream_t)stream>>>(
+    km_assign_kernel<2, 32, HALF><<<dim3((N + wg_tokens - 1) / wg_tokens, P), KM_WAVES * 64, 0, (hipStream_t)stream>>>(
         (const uint16_t*)data, (const uint16_t*)centroids, assign, N, nc, seg, head_rows);
   }
   RI_HIP_CHECK_LAUNCH();
   return RI_OK;
+}
+
+extern "C" int ri_kmeans_assign(const void* data, const void* centroids, int32_t* assign, int P, int N,
+                                int nc, int seg, int64_t head_rows, ri_stream_t stream) {
+  return km_assign<false>(data, centroids, assign, P, N, nc, seg, head_rows, stream);
+}
+
+extern "C" int ri_kmeans_assign_f16(const void* data, const void* centroids, int32_t* assign, int P, int N,
+                                    int nc, int seg, int64_t head_rows, ri_stream_t stream) {
+  return km_assign<true>(data, centroids, assign, P, N, nc, seg, head_rows, stream);
 }
 
 extern "C" size_t ri_kmeans_workspace_bytes(int P, int N, int nc) {
@@ -725,7 +742,7 @@ extern "C" size_t ri_kmeans_reduce_workspace_bytes(int P, int N, int nc) {
   return (size_t)P * (size_t)km_item_cap(N) * RI_DIM * sizeof(float) + 256;
 }
 
-template <bool MEAN>
+template <bool MEAN, bool HALF>
 static int km_reduce(const void* rows, const int32_t* counts, const int32_t* offsets, const int32_t* members,
                      void* out, int P, int N, int nc, int seg, int64_t head_rows, int normalize, void* workspace,
                      size_t workspace_bytes, hipStream_t s) {
@@ -734,37 +751,67 @@ static int km_reduce(const void* rows, const int32_t* counts, const int32_t* off
   float2* partial = (float2*)(((uintptr_t)workspace + 255) & ~(uintptr_t)255);
   const int item_wgs = (cap + 3) / 4;
   if ((long long)item_wgs + (nc + 3) / 4 > 0x7fffffffLL) return RI_ERR_ARG;
-  km_reduce_kernel<MEAN><<<dim3(item_wgs + (nc + 3) / 4, P), 256, 0, s>>>(
+  km_reduce_kernel<MEAN, HALF><<<dim3(item_wgs + (nc + 3) / 4, P), 256, 0, s>>>(
       (const uint16_t*)rows, counts, offsets, members, (uint16_t*)out, partial, item_wgs, cap, N, nc, seg, head_rows,
       normalize);
   RI_HIP_CHECK_LAUNCH();
-  km_reduce_fold_kernel<MEAN><<<dim3(item_wgs, P), 256, 0, s>>>(offsets, partial, (uint16_t*)out, cap, nc, normalize);
+  km_reduce_fold_kernel<MEAN, HALF><<<dim3(item_wgs, P), 256, 0, s>>>(offsets, partial, (uint16_t*)out, cap, nc,
+                                                                      normalize);
   RI_HIP_CHECK_LAUNCH();
   return RI_OK;
+}
+
+template <bool HALF>
+static int km_update(const void* data, const int32_t* counts, const int32_t* offsets, const int32_t* members,
+                     void* centroids, int P, int N, int nc, int seg, int64_t head_rows, int normalize, void* workspace,
+                     size_t workspace_bytes, ri_stream_t stream) {
+  if (!data || !counts || !offsets || !members || !centroids || !workspace) return RI_ERR_ARG;
+  if (ri_any_misaligned16(data, centroids, workspace)) return RI_ERR_ARG;
+  int rc = km_check(P, N, nc);
+  if (rc) return rc;
+  if (seg <= 0 || P % seg != 0) return RI_ERR_ARG;
+  return km_reduce<true, HALF>(data, counts, offsets, members, centroids, P, N, nc, seg, head_rows, normalize,
+                               workspace, workspace_bytes, (hipStream_t)stream);
 }
 
 extern "C" int ri_kmeans_update(const void* data, const int32_t* counts, const int32_t* offsets,
                                 const int32_t* members, void* centroids, int P, int N, int nc, int seg,
                                 int64_t head_rows, int normalize, void* workspace, size_t workspace_bytes,
                                 ri_stream_t stream) {
-  if (!data || !counts || !offsets || !members || !centroids || !workspace) return RI_ERR_ARG;
-  if (ri_any_misaligned16(data, centroids, workspace)) return RI_ERR_ARG;
+  return km_update<false>(data, counts, offsets, members, centroids, P, N, nc, seg, head_rows, normalize, workspace,
+                          workspace_bytes, stream);
+}
+
+extern "C" int ri_kmeans_update_f16(const void* data, const int32_t* counts, const int32_t* offsets,
+                                    const int32_t* members, void* centroids, int P, int N, int nc, int seg,
+                                    int64_t head_rows, int normalize, void* workspace, size_t workspace_bytes,
+                                    ri_stream_t stream) {
+  return km_update<true>(data, counts, offsets, members, centroids, P, N, nc, seg, head_rows, normalize, workspace,
+                         workspace_bytes, stream);
+}
+
+template <bool HALF>
+static int km_value_sum(const void* values, const int32_t* counts, const int32_t* offsets, const int32_t* members,
+                        void* value_sum, int P, int N, int nc, void* workspace, size_t workspace_bytes,
+                        ri_stream_t stream) {
+  if (!values || !counts || !offsets || !members || !value_sum || !workspace) return RI_ERR_ARG;
+  if (ri_any_misaligned16(values, value_sum, workspace)) return RI_ERR_ARG;
   int rc = km_check(P, N, nc);
   if (rc) return rc;
-  if (seg <= 0 || P % seg != 0) return RI_ERR_ARG;
-  return km_reduce<true>(data, counts, offsets, members, centroids, P, N, nc, seg, head_rows, normalize, workspace,
-                         workspace_bytes, (hipStream_t)stream);
+  return km_reduce<false, HALF>(values, counts, offsets, members, value_sum, P, N, nc, 1, (int64_t)N, 0, workspace,
+                                workspace_bytes, (hipStream_t)stream);
 }
 
 extern "C" int ri_kmeans_value_sum(const void* values, const int32_t* counts, const int32_t* offsets,
                                    const int32_t* members, void* value_sum, int P, int N, int nc, void* workspace,
                                    size_t workspace_bytes, ri_stream_t stream) {
-  if (!values || !counts || !offsets || !members || !value_sum || !workspace) return RI_ERR_ARG;
-  if (ri_any_misaligned16(values, value_sum, workspace)) return RI_ERR_ARG;
-  int rc = km_check(P, N, nc);
-  if (rc) return rc;
-  return km_reduce<false>(values, counts, offsets, members, value_sum, P, N, nc, 1, (int64_t)N, 0, workspace,
-                          workspace_bytes, (hipStream_t)stream);
+  return km_value_sum<false>(values, counts, offsets, members, value_sum, P, N, nc, workspace, workspace_bytes, stream);
+}
+
+extern "C" int ri_kmeans_value_sum_f16(const void* values, const int32_t* counts, const int32_t* offsets,
+                                       const int32_t* members, void* value_sum, int P, int N, int nc, void* workspace,
+                                       size_t workspace_bytes, ri_stream_t stream) {
+  return km_value_sum<true>(values, counts, offsets, members, value_sum, P, N, nc, workspace, workspace_bytes, stream);
 }
 
 extern "C" int ri_permute_rows(const void* in, const int32_t* members, void* out, int P, int N,

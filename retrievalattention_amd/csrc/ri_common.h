@@ -28,6 +28,59 @@ __host__ __device__ __forceinline__ float ri_round_bf16(float f) {
   return ri_bf16_to_f32(ri_f32_to_bf16(f));
 }
 
+// ---- the two 16-bit element types: bfloat16 (HALF = false) and IEEE half (HALF = true) ----
+// The fused decode path, the k-means and the operators take either (the reference's operators and cache are
+// generic over Half and BFloat16: batch_gemm_softmax.cu:185-197, gather_copy.cu:63-67); a kernel is
+// instantiated per type and the entry points come in pairs (name, name_f16).
+typedef _Float16 f16x8_t __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x4_t __attribute__((ext_vector_type(4)));
+
+template <bool HALF>
+__host__ __device__ __forceinline__ float ri_e16_to_f32(uint16_t v) {
+  if (HALF) {
+#if defined(__HIP_DEVICE_COMPILE__)
+    return (float)__builtin_bit_cast(_Float16, v);
+#else
+    // host side: plain bit arithmetic (normal, subnormal, inf/nan)
+    const uint32_t s = (uint32_t)(v & 0x8000u) << 16, e = (v >> 10) & 31u, m = v & 0x3ffu;
+    union { uint32_t u; float f; } x;
+    if (e == 0) {
+      x.f = (float)m * 5.9604644775390625e-08f;   // m * 2^-24
+      x.u |= s;
+    } else {
+      x.u = s | (e == 31 ? 0x7f800000u : (e + 112u) << 23) | (m << 13);
+    }
+    return x.f;
+#endif
+  }
+  return ri_bf16_to_f32(v);
+}
+// round to nearest even
+template <bool HALF>
+__device__ __forceinline__ uint16_t ri_f32_to_e16(float f) {
+  if (HALF) return __builtin_bit_cast(uint16_t, (_Float16)f);
+  return ri_f32_to_bf16(f);
+}
+// fp32 value of the 16-bit rounding of f
+template <bool HALF>
+__device__ __forceinline__ float ri_round_e16(float f) {
+  return ri_e16_to_f32<HALF>(ri_f32_to_e16<HALF>(f));
+}
+// the two elements packed in a 32-bit word, as fp32
+template <bool HALF>
+__device__ __forceinline__ void ri_unpack2(uint32_t w, float& lo, float& hi) {
+  if (HALF) {
+    lo = (float)__builtin_bit_cast(_Float16, (uint16_t)(w & 0xffffu));
+    hi = (float)__builtin_bit_cast(_Float16, (uint16_t)(w >> 16));
+  } else {
+    lo = __uint_as_float(w << 16);
+    hi = __uint_as_float(w & 0xffff0000u);
+  }
+}
+// finfo(type).min as a bit pattern: the score of a masked (empty) cluster
+template <bool HALF>
+__host__ __device__ __forceinline__ uint16_t ri_e16_lowest() { return HALF ? 0xfbff : 0xff7f; }
+
 __device__ __forceinline__ bf16x8_t ri_as_bf16x8(uint4 v) {
   return __builtin_bit_cast(bf16x8_t, v);
 }
@@ -71,7 +124,7 @@ void ri_set_last_hip_error(int e);
 // ---- shared between score.hip and select.hip ----
 #define RI_SCORE_TILE 256          // centroids per softmax partial
 int ri_launch_score(const void* q, const void* centroids, float* logits, float* tile_max, float* tile_sum,
-                    int BG, int gs, int nc, float scale, hipStream_t s);
+                    int BG, int gs, int nc, float scale, bool half, hipStream_t s);
 
 // Row statistics from the per-256-column partials [ntiles, gs]: one wave per row, lanes over
 // tiles, xor-butterfly reductions (fixed order, so the result is reproducible).

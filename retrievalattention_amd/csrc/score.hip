@@ -17,18 +17,10 @@
 // ------------------------------------------------------------------------------------
 // HALF: the 16-bit element type of q, cent and the 16-bit logits is IEEE half instead of bfloat16
 // (batch_gemm_softmax.cu:185-197 dispatches on Half and BFloat16).
-typedef _Float16 f16x8_t __attribute__((ext_vector_type(8)));
-
 template <bool HALF>
-__device__ __forceinline__ uint16_t score_f32_to_16(float f) {
-  if (HALF) return __builtin_bit_cast(uint16_t, (_Float16)f);   // round to nearest even
-  return ri_f32_to_bf16(f);
-}
+__device__ __forceinline__ uint16_t score_f32_to_16(float f) { return ri_f32_to_e16<HALF>(f); }
 template <bool HALF>
-__device__ __forceinline__ float score_16_to_f32(uint16_t v) {
-  if (HALF) return (float)__builtin_bit_cast(_Float16, v);
-  return ri_bf16_to_f32(v);
-}
+__device__ __forceinline__ float score_16_to_f32(uint16_t v) { return ri_e16_to_f32<HALF>(v); }
 
 // TPW = 16-row centroid tiles per wave: a workgroup covers SCORE_TILE = 256 centroids with 16 / TPW waves.
 // Launched with 4 (four waves, sixteen loads in flight per lane); eight waves with eight loads and sixteen with
@@ -147,18 +139,12 @@ __device__ __forceinline__ void score_body(
   }
 }
 
-template <int TPW>
+template <bool HALF, int TPW>
 __global__ __launch_bounds__(1024 / TPW) void score_kernel(
     const uint16_t* __restrict__ q, const uint16_t* __restrict__ cent, float* __restrict__ logits,
-    uint16_t* __restrict__ logits_bf16, float* __restrict__ tile_max, float* __restrict__ tile_sum,
+    uint16_t* __restrict__ logits16, float* __restrict__ tile_max, float* __restrict__ tile_sum,
     int gs, int nc, int ntiles, float scale) {
-  score_body<false, TPW>(q, cent, logits, logits_bf16, tile_max, tile_sum, gs, nc, ntiles, scale);
-}
-
-__global__ __launch_bounds__(256) void score_kernel_f16(
-    const uint16_t* __restrict__ q, const uint16_t* __restrict__ cent, uint16_t* __restrict__ logits_f16,
-    float* __restrict__ tile_max, float* __restrict__ tile_sum, int gs, int nc, int ntiles, float scale) {
-  score_body<true, 4>(q, cent, nullptr, logits_f16, tile_max, tile_sum, gs, nc, ntiles, scale);
+  score_body<HALF, TPW>(q, cent, logits, logits16, tile_max, tile_sum, gs, nc, ntiles, scale);
 }
 
 // batch_gemm_softmax tail: finals into slot 0 of Norm/Sum, then the bf16 softmax.
@@ -220,12 +206,8 @@ static int batch_gemm_softmax_impl(const void* A, const void* B, void* D, float*
   const int ntiles = (n + SCORE_TILE - 1) / SCORE_TILE;
   // fp32 logits are not part of this interface: the partial statistics come from the fp32
   // accumulators inside the kernel, the softmax from the 16-bit D, as in the reference.
-  if (HALF)
-    score_kernel_f16<<<dim3(ntiles, batch_count), 256, 0, s>>>((const uint16_t*)A, (const uint16_t*)B,
-                                                               (uint16_t*)D, Norm, Sum, m, n, ntiles, alpha);
-  else
-    score_kernel<4><<<dim3(ntiles, batch_count), 256, 0, s>>>((const uint16_t*)A, (const uint16_t*)B, nullptr,
-                                                              (uint16_t*)D, Norm, Sum, m, n, ntiles, alpha);
+  score_kernel<HALF, 4><<<dim3(ntiles, batch_count), 256, 0, s>>>((const uint16_t*)A, (const uint16_t*)B, nullptr,
+                                                                  (uint16_t*)D, Norm, Sum, m, n, ntiles, alpha);
   RI_HIP_CHECK_LAUNCH();
   softmax_reduce_kernel<<<batch_count, 64 * m, 0, s>>>(Norm, Sum, ntiles, m);
   RI_HIP_CHECK_LAUNCH();
@@ -252,10 +234,15 @@ extern "C" int ri_batch_gemm_softmax_f16(const void* A, const void* B, void* D, 
 
 // scoring pass used by the fused selection (select.hip)
 int ri_launch_score(const void* q, const void* centroids, float* logits, float* tile_max, float* tile_sum,
-                    int BG, int gs, int nc, float scale, hipStream_t s) {
+                    int BG, int gs, int nc, float scale, bool half, hipStream_t s) {
   const int ntiles = (nc + SCORE_TILE - 1) / SCORE_TILE;
-  score_kernel<4><<<dim3(ntiles, BG), 256, 0, s>>>((const uint16_t*)q, (const uint16_t*)centroids, logits, nullptr,
-                                                   tile_max, tile_sum, gs, nc, ntiles, scale);
+  const uint16_t *qq = (const uint16_t*)q, *cc = (const uint16_t*)centroids;
+  if (half)
+    score_kernel<true, 4><<<dim3(ntiles, BG), 256, 0, s>>>(qq, cc, logits, nullptr, tile_max, tile_sum, gs, nc,
+                                                           ntiles, scale);
+  else
+    score_kernel<false, 4><<<dim3(ntiles, BG), 256, 0, s>>>(qq, cc, logits, nullptr, tile_max, tile_sum, gs, nc,
+                                                            ntiles, scale);
   RI_HIP_CHECK_LAUNCH();
   return RI_OK;
 }

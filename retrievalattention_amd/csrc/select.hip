@@ -39,7 +39,9 @@ __device__ __forceinline__ void hist_add(uint32_t* hist, uint32_t bin, bool acti
 // ------------------------------------------------------------------------------------
 // dist_kernel: grid (ceil(nc / 1024), BG), 256 threads, 4 consecutive ids per thread.
 // ------------------------------------------------------------------------------------
-template <int GSM>
+// HALF: scores are rounded to IEEE half instead of bfloat16 wherever the reference's tensors are (the D and
+// Softmax outputs of batch_gemm_softmax and the score sum carry the cache's element type).
+template <int GSM, bool HALF>
 __global__ __launch_bounds__(256) void dist_kernel(const float* __restrict__ logits,
                                                    const float* __restrict__ tile_max,
                                                    const float* __restrict__ tile_sum,
@@ -73,14 +75,14 @@ __global__ __launch_bounds__(256) void dist_kernel(const float* __restrict__ log
       const float x[4] = {x4[j].x, x4[j].y, x4[j].z, x4[j].w};
       const float m = sh_m[j], iz = sh_iz[j];
 #pragma unroll
-      for (int i = 0; i < 4; ++i) d[i] += ri_round_bf16(__expf(ri_round_bf16(x[i]) - m) * iz);
+      for (int i = 0; i < 4; ++i) d[i] += ri_round_e16<HALF>(__expf(ri_round_e16<HALF>(x[i]) - m) * iz);
     }
   }
   uint16_t bits[4], key[4];
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
-    bits[i] = ri_f32_to_bf16(d[i]);
-    if ((mk >> (8 * i)) & 0xffu) bits[i] = 0xff7f;  // finfo(bfloat16).min
+    bits[i] = ri_f32_to_e16<HALF>(d[i]);
+    if ((mk >> (8 * i)) & 0xffu) bits[i] = ri_e16_lowest<HALF>();  // finfo(type).min
     key[i] = (uint16_t)ri_bf16_sort_key(bits[i]);
   }
   if (in) {
@@ -130,12 +132,15 @@ __device__ __forceinline__ void block_excl_scan(const uint32_t (&v)[N], uint32_t
 // Scores are sums of at most 16 probabilities, so their keys span a small range: key 0x8000
 // (score +0) .. 0xC180 (score 16), plus the masked value far below.  One histogram bin per
 // distinct key makes the rank search exact in a single pass.
+// (IEEE half: 0x8000 .. 0xCC00, so 17 bins per thread cover bfloat16 scores and 20 cover half scores.)
 #define SEL_KEY_LO 0x8000u
-#define SEL_BPT 17                          // bins per thread
-#define SEL_BINS (SEL_THREADS * SEL_BPT)    // 17408 >= 0x4181 + 1
+#define SEL_BPT_BF16 17                     // bins per thread: 17 * 1024 = 17408 >= 0x4181 + 1
+#define SEL_BPT_F16 20                      //                  20 * 1024 = 20480 >= 0x4C01 + 1
+template <int BPT>
 __device__ __forceinline__ uint32_t sel_bin(uint32_t key) {
+  constexpr uint32_t BINS = SEL_THREADS * BPT;
   const uint32_t b = key >= SEL_KEY_LO ? key - SEL_KEY_LO + 1u : 0u;
-  return b < SEL_BINS ? b : SEL_BINS - 1;
+  return b < BINS ? b : BINS - 1;
 }
 
 // ------------------------------------------------------------------------------------
@@ -150,12 +155,15 @@ __device__ __forceinline__ uint32_t sel_bin(uint32_t key) {
 // loops over the owned keys are unrolled E8 times, so the common sizes do not carry (and fetch) the code of
 // sixty-four keys per thread.
 // R: ranks of the retrieval zone a thread owns in the token-layout phase (1 up to 1023 probes, 4 up to 4096).
-template <int E8, int R>
+// BPT: histogram bins per thread (SEL_BPT_BF16 or SEL_BPT_F16).
+template <int E8, int R, int BPT>
 __global__ __launch_bounds__(SEL_THREADS) void select_kernel(
     const uint16_t* __restrict__ keys, const int32_t* __restrict__ cluster_size,
     const int32_t* __restrict__ cluster_start, int64_t* __restrict__ cI, int32_t* __restrict__ ret_ids,
     int32_t* __restrict__ est_ids, int32_t* __restrict__ ret_tok_off, int32_t* __restrict__ ret_start,
     int32_t* __restrict__ row_src, int row_src_stride, int32_t* __restrict__ meta, int nc, int np, int es, int page, int max_pages) {
+  constexpr int SEL_BPT = BPT;
+  constexpr int SEL_BINS = SEL_THREADS * BPT;
   __shared__ uint32_t hist[SEL_BINS];
   __shared__ uint32_t sh_scan[2][3 * SEL_WAVES];  // two buffers, used alternately
   __shared__ uint32_t sh_sel[4];  // bin of T1, entries above it, bin of T2, entries above it
@@ -202,7 +210,7 @@ __global__ __launch_bounds__(SEL_THREADS) void select_kernel(
       }
     }
   };
-  for_each_key([&](int, uint32_t key) { hist_add(hist, sel_bin(key), true); });
+  for_each_key([&](int, uint32_t key) { hist_add(hist, sel_bin<BPT>(key), true); });
   __syncthreads();
 
   // ---- rank thresholds: T1 = key of descending rank np-1, T2 = key of rank k2-1 ----
@@ -239,7 +247,7 @@ __global__ __launch_bounds__(SEL_THREADS) void select_kernel(
   typedef typename std::conditional<(E8 <= 4), uint32_t, uint64_t>::type mask_t;
   mask_t m_gt1 = 0, m_eq1 = 0, m_gt2 = 0, m_eq2 = 0;
   for_each_key([&](int c, uint32_t key) {
-    const uint32_t bin = sel_bin(key);
+    const uint32_t bin = sel_bin<BPT>(key);
     const int i = c - cbeg;
     m_gt1 |= (mask_t)(bin > B1) << i;
     m_eq1 |= (mask_t)(bin == B1) << i;
@@ -276,7 +284,7 @@ __global__ __launch_bounds__(SEL_THREADS) void select_kernel(
   for (mask_t m = m_gt1; m; m &= m - 1) {  // above T1: the ranks of a bin start at hist[bin] = keys above it
     const int i = lowest(m);
     const uint32_t key = key_at(i);
-    const uint32_t slot = atomicAdd(&hist[sel_bin(key)], 1u);
+    const uint32_t slot = atomicAdd(&hist[sel_bin<BPT>(key)], 1u);
     sh_ret[slot] = (key << 16) | (0xffffu - (uint32_t)(cbeg + i));
   }
   {
@@ -424,13 +432,12 @@ extern "C" size_t ri_score_select_workspace_bytes(int BG, int gs, int nc) {
   return 2 * align256((size_t)BG * ntiles * gs * sizeof(float)) + align256((size_t)BG * nc * sizeof(uint16_t));
 }
 
-extern "C" int ri_score_select(const void* q, const void* centroids, const uint8_t* mask,
-                               const int32_t* cluster_size_i32, const int32_t* cluster_start,
-                               float* logits, void* dist, int64_t* cI, int32_t* ret_ids,
-                               int32_t* est_ids, int32_t* ret_tok_off, int32_t* ret_start,
-                               int32_t* row_src, int row_src_stride, int32_t* meta, int BG, int gs, int nc, int np,
-                               int es, int page, int max_pages, float scale, void* workspace,
-                               size_t workspace_bytes, ri_stream_t stream) {
+static int score_select_impl(const void* q, const void* centroids, const uint8_t* mask,
+                             const int32_t* cluster_size_i32, const int32_t* cluster_start, float* logits, void* dist,
+                             int64_t* cI, int32_t* ret_ids, int32_t* est_ids, int32_t* ret_tok_off, int32_t* ret_start,
+                             int32_t* row_src, int row_src_stride, int32_t* meta, int BG, int gs, int nc, int np, int es,
+                             int page, int max_pages, float scale, void* workspace, size_t workspace_bytes, bool half,
+                             ri_stream_t stream) {
   if (!q || !centroids || !logits || !ret_ids || !workspace) return RI_ERR_ARG;
   if (ri_any_misaligned16(q, centroids, logits, workspace)) return RI_ERR_ARG;
   if (BG <= 0 || gs <= 0 || gs > 16 || nc <= 0 || (nc % 8) != 0) return RI_ERR_ARG;
@@ -446,21 +453,31 @@ extern "C" int ri_score_select(const void* q, const void* centroids, const uint8
   float* tsum = (float*)w;
   w += align256((size_t)BG * ntiles * gs * sizeof(float));
   uint16_t* keys = (uint16_t*)w;
-  int rc = ri_launch_score(q, centroids, logits, tmax, tsum, BG, gs, nc, scale, s);
+  int rc = ri_launch_score(q, centroids, logits, tmax, tsum, BG, gs, nc, scale, half, s);
   if (rc) return rc;
   const dim3 dgrid((nc + DIST_IDS - 1) / DIST_IDS, BG);
-  if (gs <= 4)
-    dist_kernel<4><<<dgrid, 256, 0, s>>>(logits, tmax, tsum, mask, keys, (uint16_t*)dist, gs, nc, ntiles);
-  else if (gs <= 8)
-    dist_kernel<8><<<dgrid, 256, 0, s>>>(logits, tmax, tsum, mask, keys, (uint16_t*)dist, gs, nc, ntiles);
-  else
-    dist_kernel<16><<<dgrid, 256, 0, s>>>(logits, tmax, tsum, mask, keys, (uint16_t*)dist, gs, nc, ntiles);
+#define RI_DIST_LAUNCH(GSM)                                                                                       \
+  do {                                                                                                            \
+    if (half)                                                                                                     \
+      dist_kernel<GSM, true><<<dgrid, 256, 0, s>>>(logits, tmax, tsum, mask, keys, (uint16_t*)dist, gs, nc, ntiles); \
+    else                                                                                                          \
+      dist_kernel<GSM, false><<<dgrid, 256, 0, s>>>(logits, tmax, tsum, mask, keys, (uint16_t*)dist, gs, nc, ntiles); \
+  } while (0)
+  if (gs <= 4) RI_DIST_LAUNCH(4);
+  else if (gs <= 8) RI_DIST_LAUNCH(8);
+  else RI_DIST_LAUNCH(16);
+#undef RI_DIST_LAUNCH
   RI_HIP_CHECK_LAUNCH();
   const int per_thread = (nc + SEL_THREADS - 1) / SEL_THREADS;
-#define RI_SELECT_LAUNCH(E8, R)                                                                                       \
-  select_kernel<E8, R><<<BG, SEL_THREADS, 0, s>>>(keys, cluster_size_i32, cluster_start, cI, ret_ids, est_ids,       \
-                                                  ret_tok_off, ret_start, row_src, row_src_stride, meta, nc, np, es, \
-                                                  page, max_pages)
+#define RI_SELECT_LAUNCH_T(E8, R, BPT)                                                                               \
+  select_kernel<E8, R, BPT><<<BG, SEL_THREADS, 0, s>>>(keys, cluster_size_i32, cluster_start, cI, ret_ids, est_ids,  \
+                                                       ret_tok_off, ret_start, row_src, row_src_stride, meta, nc, np, \
+                                                       es, page, max_pages)
+#define RI_SELECT_LAUNCH(E8, R)                             \
+  do {                                                      \
+    if (half) RI_SELECT_LAUNCH_T(E8, R, SEL_BPT_F16);       \
+    else RI_SELECT_LAUNCH_T(E8, R, SEL_BPT_BF16);           \
+  } while (0)
   if (np < SEL_THREADS) {
     if (per_thread <= 8) RI_SELECT_LAUNCH(1, 1);
     else if (per_thread <= 16) RI_SELECT_LAUNCH(2, 1);
@@ -472,12 +489,37 @@ extern "C" int ri_score_select(const void* q, const void* centroids, const uint8
     else RI_SELECT_LAUNCH(8, 4);
   }
 #undef RI_SELECT_LAUNCH
+#undef RI_SELECT_LAUNCH_T
   RI_HIP_CHECK_LAUNCH();
   return RI_OK;
 }
 
-extern "C" int ri_score_logits(const void* q, const void* centroids, float* logits, int BG, int gs, int nc,
-                               float scale, void* workspace, size_t workspace_bytes, ri_stream_t stream) {
+extern "C" int ri_score_select(const void* q, const void* centroids, const uint8_t* mask,
+                               const int32_t* cluster_size_i32, const int32_t* cluster_start,
+                               float* logits, void* dist, int64_t* cI, int32_t* ret_ids,
+                               int32_t* est_ids, int32_t* ret_tok_off, int32_t* ret_start,
+                               int32_t* row_src, int row_src_stride, int32_t* meta, int BG, int gs, int nc, int np,
+                               int es, int page, int max_pages, float scale, void* workspace,
+                               size_t workspace_bytes, ri_stream_t stream) {
+  return score_select_impl(q, centroids, mask, cluster_size_i32, cluster_start, logits, dist, cI, ret_ids, est_ids,
+                           ret_tok_off, ret_start, row_src, row_src_stride, meta, BG, gs, nc, np, es, page, max_pages,
+                           scale, workspace, workspace_bytes, false, stream);
+}
+
+extern "C" int ri_score_select_f16(const void* q, const void* centroids, const uint8_t* mask,
+                                   const int32_t* cluster_size_i32, const int32_t* cluster_start,
+                                   float* logits, void* dist, int64_t* cI, int32_t* ret_ids,
+                                   int32_t* est_ids, int32_t* ret_tok_off, int32_t* ret_start,
+                                   int32_t* row_src, int row_src_stride, int32_t* meta, int BG, int gs, int nc, int np,
+                                   int es, int page, int max_pages, float scale, void* workspace,
+                                   size_t workspace_bytes, ri_stream_t stream) {
+  return score_select_impl(q, centroids, mask, cluster_size_i32, cluster_start, logits, dist, cI, ret_ids, est_ids,
+                           ret_tok_off, ret_start, row_src, row_src_stride, meta, BG, gs, nc, np, es, page, max_pages,
+                           scale, workspace, workspace_bytes, true, stream);
+}
+
+static int score_logits_impl(const void* q, const void* centroids, float* logits, int BG, int gs, int nc, float scale,
+                             void* workspace, size_t workspace_bytes, bool half, ri_stream_t stream) {
   if (!q || !centroids || !logits || !workspace) return RI_ERR_ARG;
   if (ri_any_misaligned16(q, centroids, logits, workspace)) return RI_ERR_ARG;
   if (BG <= 0 || gs <= 0 || gs > 16 || nc <= 0 || (nc % 4) != 0) return RI_ERR_ARG;
@@ -485,5 +527,15 @@ extern "C" int ri_score_logits(const void* q, const void* centroids, float* logi
   const int ntiles = (nc + RI_SCORE_TILE - 1) / RI_SCORE_TILE;
   float* tmax = (float*)workspace;
   float* tsum = (float*)((char*)workspace + align256((size_t)BG * ntiles * gs * sizeof(float)));
-  return ri_launch_score(q, centroids, logits, tmax, tsum, BG, gs, nc, scale, (hipStream_t)stream);
+  return ri_launch_score(q, centroids, logits, tmax, tsum, BG, gs, nc, scale, half, (hipStream_t)stream);
+}
+
+extern "C" int ri_score_logits(const void* q, const void* centroids, float* logits, int BG, int gs, int nc,
+                               float scale, void* workspace, size_t workspace_bytes, ri_stream_t stream) {
+  return score_logits_impl(q, centroids, logits, BG, gs, nc, scale, workspace, workspace_bytes, false, stream);
+}
+
+extern "C" int ri_score_logits_f16(const void* q, const void* centroids, float* logits, int BG, int gs, int nc,
+                                   float scale, void* workspace, size_t workspace_bytes, ri_stream_t stream) {
+  return score_logits_impl(q, centroids, logits, BG, gs, nc, scale, workspace, workspace_bytes, true, stream);
 }

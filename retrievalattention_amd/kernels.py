@@ -13,9 +13,16 @@ import torch
 
 from ._lib import lib, check
 
-# 16-bit element types of the reference's operators (batch_gemm_softmax.cu:185-197, gather_copy.cu:63-67).
-# The fused decode path and the k-means are bfloat16 only.
+# 16-bit element types of the reference's operators and cache (batch_gemm_softmax.cu:185-197,
+# gather_copy.cu:63-67): every wrapper takes either and calls the entry point of that type (name or name_f16).
 _DT = (torch.bfloat16, torch.float16)
+
+
+def _fn(name, dtype):
+    """The entry point `name` for 16-bit tensors of `dtype`."""
+    if dtype not in _DT:
+        raise RuntimeError("Only Half and BFloat16 are supported")
+    return getattr(lib(), name + "_f16" if dtype == torch.float16 else name)
 
 # Named profiler ranges around the stages of a decode step, with the names the reference gives its NVTX
 # ranges (cache_hub/retroinfer_cache.py:558-678); torch's nvtx calls are roctx ranges on ROCm, so
@@ -207,12 +214,13 @@ def weighted_flash_decoding(q, k, v, weight=None, previous_out=None, previous_ls
     S = k.shape[1]
     if one != 1 or D != 128 or k.shape[2] != 1:
         raise ValueError("weighted_flash_decoding: expected q [BG,1,gs,128], k/v [BG,S,1,128]")
+    dt = q.dtype
     for t, nm in ((q, "q"), (k, "k"), (v, "v")):
-        _need(t, torch.bfloat16, nm)
+        _need(t, dt, nm)
     if weight is not None:
-        _need(weight, torch.bfloat16, "weight")
+        _need(weight, dt, "weight")
     if previous_out is not None:
-        _need(previous_out, torch.bfloat16, "previous_out")
+        _need(previous_out, dt, "previous_out")
         _need(previous_lse, torch.float32, "previous_lse")
     if cache_seqlens is not None:
         _need(cache_seqlens, torch.int32, "cache_seqlens")
@@ -220,7 +228,7 @@ def weighted_flash_decoding(q, k, v, weight=None, previous_out=None, previous_ls
     lse = torch.empty((BG, gs), dtype=torch.float32, device=q.device) if return_softmax_lse else None
     nb = lib().ri_flash_decoding_workspace_bytes(BG, gs)
     ws = _workspace(nb, q.device, "attn")
-    check(lib().ri_weighted_flash_decoding(_p(q), _p(k), _p(v), _p(weight), _p(cache_seqlens), _p(previous_out),
+    check(_fn("ri_weighted_flash_decoding", dt)(_p(q), _p(k), _p(v), _p(weight), _p(cache_seqlens), _p(previous_out),
                                            _p(previous_lse), _p(out), _p(lse), BG, gs, S, S,
                                            1.0 / math.sqrt(D), _p(ws), ws.numel(), _stream()),
           "weighted_flash_decoding")
@@ -328,7 +336,8 @@ def score_select(q, centroids, mask, cluster_size_i32, cluster_start, logits, di
     nc = centroids.shape[1]
     nb = lib().ri_score_select_workspace_bytes(BG, gs, nc)
     ws = _workspace(nb, q.device, f"score{slot}")
-    check(lib().ri_score_select(_p(q), _p(centroids), _p(mask), _p(cluster_size_i32), _p(cluster_start),
+    _need(centroids, q.dtype, "centroids")
+    check(_fn("ri_score_select", q.dtype)(_p(q), _p(centroids), _p(mask), _p(cluster_size_i32), _p(cluster_start),
                                 _p(logits), _p(dist), _p(cI), _p(ret_ids), _p(est_ids), _p(ret_tok_off),
                                 _p(ret_start), _p(row_src), 0 if row_src is None else row_src.shape[1], _p(meta),
                                 BG, gs, nc,
@@ -341,7 +350,8 @@ def score_logits(q, centroids, logits, scale, slot=0):
     BG, gs, D = q.shape
     nc = centroids.shape[1]
     ws = _workspace(lib().ri_score_select_workspace_bytes(BG, gs, nc), q.device, f"score{slot}")
-    check(lib().ri_score_logits(_p(q), _p(centroids), _p(logits), BG, gs, nc, float(scale), _p(ws), ws.numel(),
+    _need(centroids, q.dtype, "centroids")
+    check(_fn("ri_score_logits", q.dtype)(_p(q), _p(centroids), _p(logits), BG, gs, nc, float(scale), _p(ws), ws.numel(),
                                 _stream()), "score_logits")
 
 
@@ -360,7 +370,9 @@ def wave_attention(q, steady_k, steady_v, static_len, store_k, store_v, row_src,
     nc = value_sum.shape[1]
     nb = lib().ri_wave_attention_workspace_bytes(BG, gs)
     ws = _workspace(nb, q.device, f"attn{slot}")
-    check(lib().ri_wave_attention(_p(q), _p(steady_k), _p(steady_v), steady_k.shape[-2], static_len,
+    for t, nm in ((steady_k, "steady_k"), (store_k, "store_k"), (value_sum, "value_sum"), (out, "out")):
+        _need(t, q.dtype, nm)
+    check(_fn("ri_wave_attention", q.dtype)(_p(q), _p(steady_k), _p(steady_v), steady_k.shape[-2], static_len,
                                   _p(static_len_dev), _p(store_k),
                                   _p(store_v), store_k.shape[-2], _p(row_src),
                                   0 if row_src is None else row_src.shape[1], _p(ret_tok_off), _p(ret_start),
@@ -379,7 +391,7 @@ def wave_attention_part(q, steady_k, steady_v, static_len, store_k, store_v, row
     BG, gs, D = q.shape
     nc = value_sum.shape[1]
     ws = _workspace(lib().ri_wave_attention_workspace_bytes(BG, gs), q.device, f"attn{slot}")
-    check(lib().ri_wave_attention_part(
+    check(_fn("ri_wave_attention_part", q.dtype)(
         _p(q), _p(steady_k), _p(steady_v), steady_k.shape[-2], static_len, None, _p(store_k), _p(store_v),
         store_k.shape[-2], _p(row_src), row_src.shape[1], int(src_row_lo), int(src_row_hi), _p(meta), _p(est_ids),
         _p(logits), _p(value_sum), _p(cluster_size_bf16), _p(prev_out), _p(prev_lse), _p(out), _p(lse_out),
@@ -394,7 +406,7 @@ def wave_attention_static(q, steady_k, steady_v, static_len, store_k, store_v, r
     (ri_wave_attention_static), so the call allocates nothing.  Calls on one GPU must not overlap."""
     BG, gs, D = q.shape
     nc = value_sum.shape[1]
-    check(lib().ri_wave_attention_static(
+    check(_fn("ri_wave_attention_static", q.dtype)(
         _p(q), _p(steady_k), _p(steady_v), steady_k.shape[-2], static_len, _p(static_len_dev), _p(store_k),
         _p(store_v), store_k.shape[-2], _p(row_src), 0 if row_src is None else row_src.shape[1], _p(ret_tok_off),
         _p(ret_start), 0 if ret_start is None else ret_start.shape[1], _p(meta), _p(est_ids), _p(logits),
@@ -410,7 +422,7 @@ def buffer_attention(q, buf_k, buf_v, cache_seqlens, est_ids, logits, value_sum,
     nc = value_sum.shape[1]
     stride = buf_k.shape[-3] if buf_k.dim() == 4 else buf_k.shape[-2]
     ws = _workspace(lib().ri_wave_attention_workspace_bytes(BG, gs), q.device, f"attn{slot}")
-    check(lib().ri_buffer_attention(_p(q), _p(buf_k), _p(buf_v), stride, _p(cache_seqlens), stride, _p(est_ids),
+    check(_fn("ri_buffer_attention", q.dtype)(_p(q), _p(buf_k), _p(buf_v), stride, _p(cache_seqlens), stride, _p(est_ids),
                                     _p(logits), _p(value_sum), _p(cluster_size_bf16), _p(out), BG, gs, nc, es,
                                     float(scale), _p(ws), ws.numel(), _stream()), "buffer_attention")
 
@@ -451,7 +463,7 @@ class DeviceLru:
 
 
 def kmeans_assign(data, centroids, assign, P, N, nc, seg, head_rows):
-    check(lib().ri_kmeans_assign(_p(data), _p(centroids), _p(assign), P, N, nc, seg, head_rows, _stream()),
+    check(_fn("ri_kmeans_assign", data.dtype)(_p(data), _p(centroids), _p(assign), P, N, nc, seg, head_rows, _stream()),
           "kmeans_assign")
 
 
@@ -465,13 +477,13 @@ def kmeans_build_lists(assign, counts, offsets, members, P, N, nc, slot=0):
 
 def kmeans_update(data, counts, offsets, members, centroids, P, N, nc, seg, head_rows, normalize, slot=0):
     ws = _workspace(lib().ri_kmeans_reduce_workspace_bytes(P, N, nc), data.device, f"kmeans_reduce{slot}")
-    check(lib().ri_kmeans_update(_p(data), _p(counts), _p(offsets), _p(members), _p(centroids), P, N, nc, seg,
+    check(_fn("ri_kmeans_update", data.dtype)(_p(data), _p(counts), _p(offsets), _p(members), _p(centroids), P, N, nc, seg,
                                  head_rows, int(bool(normalize)), _p(ws), ws.numel(), _stream()), "kmeans_update")
 
 
 def kmeans_value_sum(values, counts, offsets, members, value_sum, P, N, nc, slot=0):
     ws = _workspace(lib().ri_kmeans_reduce_workspace_bytes(P, N, nc), values.device, f"kmeans_reduce{slot}")
-    check(lib().ri_kmeans_value_sum(_p(values), _p(counts), _p(offsets), _p(members), _p(value_sum), P, N, nc,
+    check(_fn("ri_kmeans_value_sum", values.dtype)(_p(values), _p(counts), _p(offsets), _p(members), _p(value_sum), P, N, nc,
                                     _p(ws), ws.numel(), _stream()), "kmeans_value_sum")
 
 

@@ -17,7 +17,7 @@ it to the band; the tally reports how often it was needed.
 import numpy as np
 import torch
 
-from oracle.numerics import bf16_ulp
+from oracle.numerics import bf16_ulp, ulp16
 
 
 def bf16_bits_i(x):
@@ -30,7 +30,7 @@ def ulp_distance_bf16(a, b):
     return (bf16_bits_i(a) - bf16_bits_i(b)).abs()
 
 
-def score_interval(logits, mask=None, rel=4e-6):
+def score_interval(logits, mask=None, rel=4e-6, dtype=torch.bfloat16):
     """(lo, hi) bf16 [BG, nc]: the scores bf16(sum_j bf16(p_j)) with every head's probability
     p_j = exp(bf16(x_j) - m_j) / Z_j (evaluated in float64 from fp32 logits [BG, gs, nc]) scaled by
     (1 - rel) and (1 + rel), the bf16 probabilities added in fp32 in head order.  rel covers a fast fp32 exp, the order of the fp32 sum behind Z and a
@@ -40,16 +40,16 @@ def score_interval(logits, mask=None, rel=4e-6):
     x = logits.double()
     m = x.max(dim=-1, keepdim=True).values
     z = torch.exp(x - m).sum(dim=-1, keepdim=True)
-    p = torch.exp(logits.to(torch.bfloat16).double() - m) / z
+    p = torch.exp(logits.to(dtype).double() - m) / z
     out = []
     for f in (1.0 - rel, 1.0 + rel):
-        pb = (p * f).float().to(torch.bfloat16).float()
+        pb = (p * f).float().to(dtype).float()
         d = torch.zeros_like(pb[:, 0])
         for j in range(pb.shape[1]):   # fp32 sum in head order: a head of 2^-24 of the sum can decide a tie
             d = d + pb[:, j]
-        d = d.to(torch.bfloat16)
+        d = d.to(dtype)
         if mask is not None:
-            d = d.masked_fill(mask.bool(), torch.finfo(torch.bfloat16).min)
+            d = d.masked_fill(mask.bool(), torch.finfo(dtype).min)
         out.append(d)
     return out[0], out[1]
 
@@ -80,6 +80,7 @@ def check_zone_sets(dist, ret, est, ret_ref, est_ref, nprobe, es, band=1.0, labe
     Returns the number of tolerated boundary swaps (a ZoneSwaps: .beyond1 counts those whose score is
     more than one ulp from the boundary); asserts on anything else.  slack [BG, nc] (optional): per-cluster
     score uncertainty from flip_slack, added for the cluster and for the worst cluster it can swap with."""
+    ulp = lambda t: ulp16(t, dist.dtype if dist.dtype in (torch.bfloat16, torch.float16) else torch.bfloat16)
     d = dist.float()
     swaps, beyond1, flips = 0, 0, 0
     for g in range(d.shape[0]):
@@ -98,8 +99,8 @@ def check_zone_sets(dist, ret, est, ret_ref, est_ref, nprobe, es, band=1.0, labe
             worst = max(float(slack[g, c]) for c in diff) if slack is not None else 0.0
             for c in diff:
                 extra = (float(slack[g, c]) + worst) if slack is not None else 0.0
-                ulps = min(abs(float(d[g, c]) - float(t)) / float(bf16_ulp(t.reshape(1))) for t in bounds)
-                flip = min((abs(float(d[g, c]) - float(t)) - extra) / float(bf16_ulp(t.reshape(1))) for t in bounds)
+                ulps = min(abs(float(d[g, c]) - float(t)) / float(ulp(t.reshape(1))) for t in bounds)
+                flip = min((abs(float(d[g, c]) - float(t)) - extra) / float(ulp(t.reshape(1))) for t in bounds)
                 assert flip <= band, f"group {g}: cluster {c} score {float(d[g, c])} is not a boundary tie ({[float(t) for t in bounds]})"
                 if ulps > band:          # acceptable only because of a rounding flip of a logit
                     flips += 1
@@ -124,7 +125,7 @@ def check_rank_order(dist, ret, band=1.0, slack=None, label=None):
         ids = ret[g].long()
         s = d[g, ids]
         viol = s[1:] - s[:-1]
-        lim = band * bf16_ulp(s[1:])
+        lim = band * ulp16(s[1:], dist.dtype if dist.dtype in (torch.bfloat16, torch.float16) else torch.bfloat16)
         if slack is not None:
             sl = slack[g, ids]
             flips = int(((viol > lim) & (viol <= lim + sl[1:] + sl[:-1])).sum())

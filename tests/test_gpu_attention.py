@@ -25,8 +25,8 @@ def _same_up_to_rounding(a, b, abs_tol, ulps=1):
     assert bool(((a - b).abs() <= lim).all()), f"max-abs {float((a - b).abs().max())}"
 
 
-def _rand(shape, g, scale=1.0):
-    return (torch.randn(*shape, generator=g) * scale).to(torch.bfloat16)
+def _rand(shape, g, scale=1.0, dt=torch.bfloat16):
+    return (torch.randn(*shape, generator=g) * scale).to(dt)
 
 
 @pytest.mark.parametrize("BG,gs,S,weighted,prev,ragged", [
@@ -38,14 +38,14 @@ def _rand(shape, g, scale=1.0):
     (1, 1, 1, False, False, False),
     (2, 4, 1900, True, False, False),   # the estimation call: weights = cluster sizes
 ])
-def test_weighted_flash_decoding(dev, BG, gs, S, weighted, prev, ragged):
+def test_weighted_flash_decoding(dev, BG, gs, S, weighted, prev, ragged, dt=torch.bfloat16):
     from retrievalattention_amd import kernels
     g = torch.Generator().manual_seed(S + gs)
-    q = _rand((BG, gs, 128), g)
-    k = _rand((BG, S, 128), g)
-    v = _rand((BG, S, 128), g)
-    w = torch.randint(1, 60, (BG, S), generator=g).to(torch.bfloat16) if weighted else None
-    po = _rand((BG, gs, 128), g, 0.3) if prev else None
+    q = _rand((BG, gs, 128), g, dt=dt)
+    k = _rand((BG, S, 128), g, dt=dt)
+    v = _rand((BG, S, 128), g, dt=dt)
+    w = torch.randint(1, 60, (BG, S), generator=g).to(dt) if weighted else None
+    po = _rand((BG, gs, 128), g, 0.3, dt=dt) if prev else None
     pl = (torch.randn(BG, gs, generator=g) + 6.0) if prev else None
     sl = torch.randint(max(1, S // 3), S + 1, (BG,), generator=g, dtype=torch.int32) if ragged else None
     out, lse = kernels.weighted_flash_decoding(
@@ -58,6 +58,16 @@ def test_weighted_flash_decoding(dev, BG, gs, S, weighted, prev, ragged):
     ro, rl = attention.weighted_flash_decoding(q, k, v, w, po, pl, sl)
     _close(out.cpu().view(BG, gs, 128), ro)
     assert torch.allclose(lse.cpu(), rl, atol=2e-3, rtol=1e-4)
+    assert out.dtype == dt
+
+
+@pytest.mark.parametrize("BG,gs,S,weighted,prev,ragged", [
+    (3, 4, 2421, False, True, True), (5, 7, 1000, True, False, False), (2, 8, 4773, True, True, True),
+    (2, 16, 77, True, True, True), (1, 1, 1, False, False, False),
+])
+def test_weighted_flash_decoding_float16(dev, BG, gs, S, weighted, prev, ragged):
+    """IEEE half elements (the reference's harnesses default to fp16, simple_test.py:29): same tolerance."""
+    test_weighted_flash_decoding(dev, BG, gs, S, weighted, prev, ragged, dt=torch.float16)
 
 
 def test_weighted_flash_decoding_with_an_empty_group(dev):
@@ -161,7 +171,7 @@ def test_closed_form_estimation_exact_for_singletons_and_identical_keys(dev):
     (1, 4, 30000, 3000, 1000, 69, 9),
     (1, 8, 16384, 4096, 0, 10, 10),     # the longest probe list
 ])
-def test_wave_attention(dev, BG, gs, nc, nprobe, es, static_len, seed):
+def test_wave_attention(dev, BG, gs, nc, nprobe, es, static_len, seed, dt=torch.bfloat16):
     """score_select + wave_attention against the oracle's composition of steps 4-8 of
     retroinfer_cache.compute (cache_hub/retroinfer_cache.py:598-674)."""
     from retrievalattention_amd import kernels
@@ -169,12 +179,12 @@ def test_wave_attention(dev, BG, gs, nc, nprobe, es, static_len, seed):
     size = torch.randint(0, 33, (BG, nc), generator=g, dtype=torch.int32)
     start = (torch.cumsum(size, 1) - size).to(torch.int32)
     ntok = int(size.sum(1).max())
-    cent = _rand((BG, nc, 128), g)
+    cent = _rand((BG, nc, 128), g, dt=dt)
     cent[:, :, :4] *= 4
-    q = _rand((BG, gs, 128), g)
-    store_k, store_v = _rand((BG, ntok, 128), g), _rand((BG, ntok, 128), g)
-    steady_k, steady_v = _rand((BG, static_len + 5, 128), g), _rand((BG, static_len + 5, 128), g)
-    vsum = _rand((BG, nc, 128), g, 4.0)
+    q = _rand((BG, gs, 128), g, dt=dt)
+    store_k, store_v = _rand((BG, ntok, 128), g, dt=dt), _rand((BG, ntok, 128), g, dt=dt)
+    steady_k, steady_v = _rand((BG, static_len + 5, 128), g, dt=dt), _rand((BG, static_len + 5, 128), g, dt=dt)
+    vsum = _rand((BG, nc, 128), g, 4.0, dt=dt)
     mask = size == 0
     scale = 1 / math.sqrt(128)
     page, max_pages = 8, max(4 * nprobe, 16) * 4
@@ -184,9 +194,9 @@ def test_wave_attention(dev, BG, gs, nc, nprobe, es, static_len, seed):
     off = torch.empty(BG, nprobe + 1, dtype=torch.int32, device=dev)
     rows = torch.zeros(BG, max_pages * page, dtype=torch.int32, device=dev)
     meta = torch.empty(BG, 4, dtype=torch.int32, device=dev)
-    out = torch.empty(BG, gs, 128, dtype=torch.bfloat16, device=dev)
+    out = torch.empty(BG, gs, 128, dtype=dt, device=dev)
     vl = torch.empty(BG, dtype=torch.int32, device=dev)
-    size_bf = size.to(torch.bfloat16)
+    size_bf = size.to(dt)
     qd = q.to(dev)
     kernels.score_select(qd, cent.to(dev), mask.to(torch.uint8).to(dev), size.to(dev), start.to(dev), logits, None,
                          None, ret, est if es else None, off, rows, meta, nprobe, es, page, max_pages, scale)
@@ -236,7 +246,7 @@ def test_wave_attention(dev, BG, gs, nc, nprobe, es, static_len, seed):
     kept, offs = scoring.retrieval_layout(ret_c, size, page, max_pages)
     assert torch.equal(vl.cpu().long(), static_len + offs[:, -1])
     # oracle on the kernel's selection
-    ref = torch.empty(BG, gs, 128, dtype=torch.bfloat16)
+    ref = torch.empty(BG, gs, 128, dtype=dt)
     for b in range(BG):
         ks, vs = [steady_k[b, :static_len]], [steady_v[b, :static_len]]
         for c in ret_c[b, :int(kept[b])]:
@@ -246,13 +256,23 @@ def test_wave_attention(dev, BG, gs, nc, nprobe, es, static_len, seed):
         po = pl = None
         if es:
             eo, el = attention.estimation(lg[b:b + 1], est_c[b:b + 1], vsum[b:b + 1], size_bf[b:b + 1])
-            po, pl = eo.to(torch.bfloat16), el.float()   # the reference hands es_out over in bf16
+            po, pl = eo.to(dt), el.float()   # the reference hands es_out over in the 16-bit type
         ref[b] = attention.weighted_flash_decoding(q[b:b + 1], kk, vv, None, po, pl)[0][0]
     _close(out.cpu(), ref)
     _close(out_t.cpu(), ref)
     _close(out_c.cpu(), ref)
     _close(out_p.cpu(), ref)
     _same_up_to_rounding(out_p, out, 1.6e-2)   # the first part went through bf16
+
+
+@pytest.mark.parametrize("BG,gs,nc,nprobe,es,static_len,seed", [
+    (4, 4, 512, 9, 118, 69, 20), (2, 4, 8192, 147, 1900, 69, 21), (3, 7, 3840, 69, 890, 200, 22),
+    (2, 8, 2048, 36, 0, 68, 23), (2, 16, 1024, 20, 100, 69, 24), (2, 5, 512, 33, 77, 1, 26),
+    (1, 3, 256, 1, 255, 0, 27), (1, 16, 112, 10, 0, 0, 3044), (1, 4, 15000, 1500, 2250, 69, 28),
+])
+def test_wave_attention_float16(dev, BG, gs, nc, nprobe, es, static_len, seed):
+    """Every mode of test_wave_attention with IEEE half elements."""
+    test_wave_attention(dev, BG, gs, nc, nprobe, es, static_len, seed, dt=torch.float16)
 
 
 def test_wave_attention_random_shapes(dev):

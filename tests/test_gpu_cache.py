@@ -18,7 +18,8 @@ def _close(got, ref):
 
 
 def _make_cache(dev, residency, layers, B, Hkv, gs, ctx, n_centroids, n_segment, nprobe, es, new=8,
-                cache_cluster_num=None, use_cluster_estimation=False, device_positions=False, valid_start=None):
+                cache_cluster_num=None, use_cluster_estimation=False, device_positions=False, valid_start=None,
+                dt=torch.bfloat16):
     from retrievalattention_amd.cache_hub import retroinfer_cache
     # "host-cpu": host-resident store with the reference's worker-thread block cache manager;
     # "host": the same store with the device-side manager
@@ -30,7 +31,7 @@ def _make_cache(dev, residency, layers, B, Hkv, gs, ctx, n_centroids, n_segment,
     residency = "host" if residency == "host-cpu" else residency
     return retroinfer_cache(
         valid_start=valid_start or [0] * B, layer_num=layers, batch_size=B, max_length=ctx + new, num_key_value_heads=Hkv,
-        num_heads=Hkv * gs, head_dim=128, dtype=torch.bfloat16, layer_mapping={str(l): "cuda:0" for l in range(layers)},
+        num_heads=Hkv * gs, head_dim=128, dtype=dt, layer_mapping={str(l): "cuda:0" for l in range(layers)},
         max_new_length=new, static_pattern_start=4, static_pattern_end=64, core=4, n_centroids=n_centroids,
         n_segment=n_segment, nprobe=nprobe, max_compute_cluster_num=nprobe + es, cache_unit_size=8,
         cache_cluster_num=cache_cluster_num if cache_cluster_num is not None else 3 * nprobe, num_gpus=1,
@@ -49,24 +50,24 @@ def _prefill(cache, K, V, layers, B):
     cache.prepare_cache()
 
 
-def _gen(layers, B, Hkv, gs, ctx, nmix, dev, seed):
+def _gen(layers, B, Hkv, gs, ctx, nmix, dev, seed, dt=torch.bfloat16):
     from retrievalattention_amd import synth
     K, V = [], []
     for l in range(layers):
-        k, v, _ = synth.make_batch(seed + l, B, Hkv, ctx, nmix, gs, outliers=True)
+        k, v, _ = synth.make_batch(seed + l, B, Hkv, ctx, nmix, gs, outliers=True, dtype=dt)
         K.append([k[b].transpose(0, 1)[None].contiguous().to(dev) for b in range(B)])
         V.append([v[b].transpose(0, 1)[None].contiguous().to(dev) for b in range(B)])
     return K, V
 
 
 @pytest.mark.parametrize("residency", ["device", "host", "host-overlap", "host-cpu"])
-def test_decode_matches_oracle(dev, residency):
+def test_decode_matches_oracle(dev, residency, dt=torch.bfloat16):
     """Prefill + three decode steps; every compute() is compared with the oracle's decode step
     run on the index the cache actually holds."""
     layers, B, Hkv, gs, ctx = 2, 2, 2, 4, 4096 + 68
     nc, S, nprobe, es = 256, 1, 8, 60
-    cache = _make_cache(dev, residency, layers, B, Hkv, gs, ctx, nc, S, nprobe, es)
-    K, V = _gen(layers, B, Hkv, gs, ctx, 256, dev, 0)
+    cache = _make_cache(dev, residency, layers, B, Hkv, gs, ctx, nc, S, nprobe, es, dt=dt)
+    K, V = _gen(layers, B, Hkv, gs, ctx, 256, dev, 0, dt=dt)
     _prefill(cache, K, V, layers, B)
     assert cache.context == ctx
     BG = B * Hkv
@@ -93,9 +94,9 @@ def test_decode_matches_oracle(dev, residency):
         stores.append((sk, sv, torch.stack(st)))
     for step in range(3):
         for l in range(layers):
-            k_new = torch.randn(B, 1, Hkv, 128, generator=g).to(torch.bfloat16)
-            v_new = torch.randn(B, 1, Hkv, 128, generator=g).to(torch.bfloat16)
-            q = torch.randn(B, 1, Hkv * gs, 128, generator=g).to(torch.bfloat16)
+            k_new = torch.randn(B, 1, Hkv, 128, generator=g).to(dt)
+            v_new = torch.randn(B, 1, Hkv, 128, generator=g).to(dt)
+            q = torch.randn(B, 1, Hkv * gs, 128, generator=g).to(dt)
             cache.decode_update_kv_cache(k_new.to(dev), v_new.to(dev), l)
             out = cache.compute(q.to(dev), l)
             torch.cuda.synchronize()
@@ -114,7 +115,14 @@ def test_decode_matches_oracle(dev, residency):
             assert torch.equal(cache.cI[buf][:, :nprobe].cpu(), aux["ret"])
             assert torch.equal(cache.cI[buf][:, nprobe:].cpu(), aux["est"])
             assert torch.equal(cache.valid_lengths[buf].cpu().long(), static_len + aux["offs"][:, -1])
-    assert cache.context == ctx + 3
+    assert cache.context == ctx + 3 and out.dtype == dt
+
+
+@pytest.mark.parametrize("residency", ["device", "host", "host-overlap", "host-cpu"])
+def test_decode_matches_oracle_float16(dev, residency):
+    """The same with IEEE half elements, the default of the reference's harnesses (simple_test.py:29,
+    throughput_eval/test.py:28): index, stores, scores, probabilities and outputs all in fp16."""
+    test_decode_matches_oracle(dev, residency, dt=torch.float16)
 
 
 def test_full_retrieval_equals_dense_attention(dev):

@@ -13,13 +13,13 @@ from oracle import kmeans as okm
 pytestmark = pytest.mark.gpu
 
 
-def _mixture(G, N, K, seed, sigma=0.3):
+def _mixture(G, N, K, seed, sigma=0.3, dt=torch.bfloat16):
     g = torch.Generator().manual_seed(seed)
     centers = torch.randn(G, K, 128, generator=g)
     a = torch.randint(K, (G, N), generator=g)
     keys = torch.gather(centers, 1, a[..., None].expand(G, N, 128)) + sigma * torch.randn(G, N, 128, generator=g)
     vals = torch.randn(G, N, 128, generator=g)
-    return keys.to(torch.bfloat16), vals.to(torch.bfloat16)
+    return keys.to(dt), vals.to(dt)
 
 
 def _check_assign(data, cent, got):
@@ -35,9 +35,9 @@ def _check_assign(data, cent, got):
 
 
 @pytest.mark.parametrize("P,N,nc,seed", [(3, 1000, 64, 0), (2, 8192, 512, 1), (1, 4100, 1024, 2), (4, 37, 32, 3)])
-def test_assign_update_valuesum(dev, P, N, nc, seed):
+def test_assign_update_valuesum(dev, P, N, nc, seed, dt=torch.bfloat16):
     from retrievalattention_amd import kernels
-    keys, vals = _mixture(P, N, nc, seed)
+    keys, vals = _mixture(P, N, nc, seed, dt=dt)
     idx = okm.init_indices(N, nc)
     cent = keys[:, idx].contiguous()
     kd, vd, cd = keys.to(dev), vals.to(dev), cent.to(dev).clone()
@@ -45,7 +45,7 @@ def test_assign_update_valuesum(dev, P, N, nc, seed):
     counts = torch.empty(P, nc, dtype=torch.int32, device=dev)
     offsets = torch.empty(P, nc + 1, dtype=torch.int32, device=dev)
     members = torch.empty(P, N, dtype=torch.int32, device=dev)
-    vsum = torch.empty(P, nc, 128, dtype=torch.bfloat16, device=dev)
+    vsum = torch.empty(P, nc, 128, dtype=dt, device=dev)
     kernels.kmeans_assign(kd, cd, assign, P, N, nc, 1, N)
     kernels.kmeans_build_lists(assign, counts, offsets, members, P, N, nc)
     cn = cd.clone()
@@ -70,6 +70,13 @@ def test_assign_update_valuesum(dev, P, N, nc, seed):
         assert torch.equal(cn[p].cpu(), okm.update(cent[p], s, cnt2, True))
         assert torch.equal(cu[p].cpu(), okm.update(cent[p], s, cnt2, False))
         assert torch.equal(vsum[p].cpu(), okm.value_sum(vals[p], A[p].astype(np.int64), nc))
+
+
+@pytest.mark.parametrize("P,N,nc,seed", [(3, 1000, 64, 10), (2, 8192, 512, 11), (1, 4100, 1024, 12), (4, 37, 32, 13)])
+def test_assign_update_valuesum_float16(dev, P, N, nc, seed):
+    """IEEE half keys, values and centroids (the reference's harnesses default to fp16, simple_test.py:29):
+    the same fixed-order fp32 sums, rounded to fp16 on store."""
+    test_assign_update_valuesum(dev, P, N, nc, seed, dt=torch.float16)
 
 
 def test_big_and_empty_clusters(dev):
@@ -117,22 +124,23 @@ def test_medium_clusters_sorted(dev):
         assert np.array_equal(members[p].cpu().numpy(), order.astype(np.int32))
 
 
-def test_long_lists_blocked_sums(dev):
+@pytest.mark.parametrize("dt", [torch.bfloat16, torch.float16], ids=["bf16", "f16"])
+def test_long_lists_blocked_sums(dev, dt):
     """Lists of 1 to several thousand random rows: update and value sums equal the oracle's
     blocked fixed-order sums bit for bit (lists over 256 rows take the block-item path, several
     of them per problem, next to short lists and empty clusters)."""
     from retrievalattention_amd import kernels
     P, N, nc = 3, 20011, 96
     g = torch.Generator().manual_seed(16)
-    keys = torch.randn(P, N, 128, generator=g).to(torch.bfloat16)
-    vals = torch.randn(P, N, 128, generator=g).to(torch.bfloat16)
+    keys = torch.randn(P, N, 128, generator=g).to(dt)
+    vals = torch.randn(P, N, 128, generator=g).to(dt)
     assign = torch.randint(0, 5, (P, N), generator=g, dtype=torch.int32)       # five lists of ~4000
     small = torch.randint(8, 90, (P, N), generator=g, dtype=torch.int32)       # the rest: ~100 each, 90..95 empty
     pick = torch.rand(P, N, generator=g) < 0.4
     assign[pick] = small[pick]
     assign[1, :700] = 7                                                        # 700+: three blocks, last one ragged
     assign[2, 5] = 95                                                          # a single-row list
-    cent = torch.randn(P, nc, 128, generator=g).to(torch.bfloat16)
+    cent = torch.randn(P, nc, 128, generator=g).to(dt)
     ad, kd, vd = assign.to(dev), keys.to(dev), vals.to(dev)
     counts = torch.empty(P, nc, dtype=torch.int32, device=dev)
     offsets = torch.empty(P, nc + 1, dtype=torch.int32, device=dev)
@@ -141,7 +149,7 @@ def test_long_lists_blocked_sums(dev):
     for normalize in (True, False):
         cd = cent.to(dev).clone()
         kernels.kmeans_update(kd, counts, offsets, members, cd, P, N, nc, 1, N, normalize)
-        vs = torch.full((P, nc, 128), 7.0, dtype=torch.bfloat16, device=dev)
+        vs = torch.full((P, nc, 128), 7.0, dtype=dt, device=dev)
         kernels.kmeans_value_sum(vd, counts, offsets, members, vs, P, N, nc)
         torch.cuda.synchronize()
         for p in range(P):
@@ -213,12 +221,12 @@ def test_build_lists_is_a_stable_sort(dev, P, N, nc, seed):
 
 
 @pytest.mark.parametrize("G,N,nc,S,seed", [(2, 4096, 256, 4, 0), (1, 8192, 512, 1, 1), (2, 3001, 192, 3, 2)])
-def test_segment_k_means_teacher_forced(dev, G, N, nc, S, seed):
+def test_segment_k_means_teacher_forced(dev, G, N, nc, S, seed, dt=torch.bfloat16):
     """Whole driver against the oracle, iteration by iteration: every step is checked on the
     state the kernels actually produced (the trajectory itself is chaotic under near-ties)."""
     from retrievalattention_amd import kernels
     from retrievalattention_amd.cache_hub.kmeans import segment_k_means, segment_k_means_csr, csr_to_dense
-    keys, vals = _mixture(G, N, nc, seed)
+    keys, vals = _mixture(G, N, nc, seed, dt=dt)
     kd, vd = keys.to(dev), vals.to(dev)
     cent, vsum, clusters, csize = segment_k_means(kd, vd, nc, 10, S)
     torch.cuda.synchronize()
@@ -260,3 +268,8 @@ def test_segment_k_means_teacher_forced(dev, G, N, nc, S, seed):
         assert np.array_equal(clusters.cpu().numpy()[gi][:, :lists.shape[1]], lists)
     # invariants: every token in exactly one list, sizes add up
     assert int(csize.sum()) == G * N
+
+
+@pytest.mark.parametrize("G,N,nc,S,seed", [(2, 4096, 256, 4, 10), (2, 3001, 192, 3, 12)])
+def test_segment_k_means_teacher_forced_float16(dev, G, N, nc, S, seed):
+    test_segment_k_means_teacher_forced(dev, G, N, nc, S, seed, dt=torch.float16)

@@ -12,13 +12,13 @@ from tests.parity import (bf16_bits_i, check_zone_sets, check_rank_order, flip_s
 pytestmark = pytest.mark.gpu
 
 
-def _mixture(BG, gs, nc, seed, outliers=True):
+def _mixture(BG, gs, nc, seed, outliers=True, dt=torch.bfloat16):
     g = torch.Generator().manual_seed(seed)
     cent = torch.randn(BG, nc, 128, generator=g)
     if outliers:
         cent[:, :, :4] *= 8
     q = torch.randn(BG, gs, 128, generator=g)
-    return q.to(torch.bfloat16), cent.to(torch.bfloat16)
+    return q.to(dt), cent.to(dt)
 
 
 def test_batch_gemm_softmax_matches_reference_test(dev):
@@ -102,9 +102,9 @@ def test_batch_gemm_softmax_half(dev):
     (1, 4, 30000, 3000, 4500, 9),    #   nprobe = 10 % of the clusters): 240K and 480K tokens of context
     (1, 8, 40960, 4096, 100, 10),    # the longest probe list the entry point takes
 ])
-def test_score_select(dev, BG, gs, nc, nprobe, es, seed):
+def test_score_select(dev, BG, gs, nc, nprobe, es, seed, dt=torch.bfloat16):
     from retrievalattention_amd import kernels
-    q, cent = _mixture(BG, gs, nc, seed)
+    q, cent = _mixture(BG, gs, nc, seed, dt=dt)
     g = torch.Generator().manual_seed(seed + 100)
     mask = torch.rand(BG, nc, generator=g) < 0.02
     size = torch.randint(1, 40, (BG, nc), generator=g, dtype=torch.int32)
@@ -115,7 +115,7 @@ def test_score_select(dev, BG, gs, nc, nprobe, es, seed):
     k2 = nprobe + es
     o = dict(
         logits=torch.empty(BG, gs, nc, dtype=torch.float32, device=dev),
-        dist=torch.empty(BG, nc, dtype=torch.bfloat16, device=dev),
+        dist=torch.empty(BG, nc, dtype=dt, device=dev),
         cI=torch.empty(BG, k2, dtype=torch.int64, device=dev),
         ret=torch.empty(BG, nprobe, dtype=torch.int32, device=dev),
         est=torch.empty(BG, max(es, 1), dtype=torch.int32, device=dev),
@@ -136,10 +136,10 @@ def test_score_select(dev, BG, gs, nc, nprobe, es, seed):
 
     # (2) score pipeline on the kernel's own logits: inside the interval that a 4e-6 relative tolerance of the
     # fp32 probabilities leaves open (the oracle's own value wherever no head sits on a bf16 rounding boundary)
-    _, _, _, soft = scoring.softmax_from_logits(o["logits"])
+    _, _, _, soft = scoring.softmax_from_logits(o["logits"], dt)
     dist_ref = scoring.dist_from_softmax(soft, mask)
     dd = ulp_distance_bf16(o["dist"], dist_ref)
-    lo, hi = score_interval(o["logits"], mask)
+    lo, hi = score_interval(o["logits"], mask, dtype=dt)
     kb = bf16_bits_i(o["dist"])
     assert bool(((kb >= bf16_bits_i(lo)) & (kb <= bf16_bits_i(hi))).all())
     assert int(ulp_distance_bf16(lo, hi).max()) <= 2 and int(dd.max()) <= 2
@@ -152,12 +152,12 @@ def test_score_select(dev, BG, gs, nc, nprobe, es, seed):
     assert torch.equal(o["cI"][:, :nprobe], ret_x) and torch.equal(o["cI"][:, nprobe:], est_x)
 
     # (4) end to end against the oracle's scores: identical up to boundary ties
-    dist_of = lambda x: scoring.dist_from_softmax(scoring.softmax_from_logits(x)[3], mask)
+    dist_of = lambda x: scoring.dist_from_softmax(scoring.softmax_from_logits(x, dt)[3], mask)
     dist_o = dist_of(x_ref)
     ret_o, est_o = scoring.select(dist_o, nprobe, es)
     # the band, plus what a bf16 rounding flip of a logit inside the logits' own tolerance can move a score
     slack = flip_slack(x_ref, dist_of, delta=2e-5)
-    label = f"score_select BG{BG} gs{gs} nc{nc}"
+    label = f"score_select BG{BG} gs{gs} nc{nc}" + (" f16" if dt == torch.float16 else "")
     check_zone_sets(dist_o, ret, est, ret_o, est_o, nprobe, es, band=1.0, label=label, slack=slack)
     check_rank_order(dist_o, ret, band=1.0, slack=slack, label=label)
 
@@ -170,6 +170,16 @@ def test_score_select(dev, BG, gs, nc, nprobe, es, seed):
         exp_rows = torch.cat([start[gi, c] + torch.arange(int(size[gi, c])) for c in ret[gi, :int(kept[gi])]]
                              + [torch.zeros(0, dtype=torch.int64)])
         assert torch.equal(o["rows"][gi, :exp_rows.numel()].long(), exp_rows.long())
+
+
+@pytest.mark.parametrize("BG,gs,nc,nprobe,es,seed", [
+    (8, 4, 512, 9, 118, 20), (4, 4, 8192, 147, 1900, 21), (4, 7, 3840, 69, 890, 22), (2, 8, 16384, 294, 3801, 23),
+    (3, 1, 64, 1, 0, 24), (2, 16, 1000, 20, 980, 25), (1, 4, 32768, 300, 3000, 26), (2, 4, 15000, 1500, 2250, 27),
+])
+def test_score_select_float16(dev, BG, gs, nc, nprobe, es, seed):
+    """The same checks with IEEE half elements (the reference's harnesses default to fp16:
+    simple_test.py:29, throughput_eval/test.py:28): logits, probabilities and scores round to fp16."""
+    test_score_select(dev, BG, gs, nc, nprobe, es, seed, dt=torch.float16)
 
 
 def test_score_select_many_seeds(dev):
