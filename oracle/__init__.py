@@ -4,7 +4,8 @@ TEST INFRASTRUCTURE ONLY.  Nothing under this package is part of the product: it
 checker that tests/, __graft_entry__.smoke() and the cpu_baseline leg of bench.py compare the
 HIP kernels against.  The product (retrievalattention_amd/) never imports it.
 
-Every function cites the reference file:line it follows.  The reference stores no golden vectors
+Every function cites the reference file:line it follows.  The 16-bit element type (bfloat16 or IEEE
+half, the two the reference runs in) is taken from the inputs: roundings go to that type.  The reference stores no golden vectors
 for this path; tests/golden/known_answers.json holds hand-worked known answers for every part below
 (initial tokens, a clustering followed by hand, softmax cases in closed form, ties and masked clusters
 in the selection, the buffer cut-off, a block cache trace, rational attention results), derived in
@@ -21,10 +22,11 @@ tests/golden/make_known_answers.py without this package.  How each function is p
                                   same hit/miss/update lists step by step, block id values aside);
                                   a hand-followed trace; invariants (hit <=> resident, capacity,
                                   unique block ids, least-recently-touched eviction)
-  wavebuf.DeviceLruModel          the policy of the device-side block cache manager, which is this
-                                  build's own (the reference manages the cache on CPU threads):
-                                  invariants (every requested cluster once, hit <=> resident, unique
-                                  block ids, blocks conserved, victims not newer than survivors)
+  wavebuf.DeviceLruModel          the device-side block cache manager's arithmetic (recency as a step
+                                  stamp plus the order inside the step, victims by (stamp, order)):
+                                  the same policy as LruModel, pinned to it over random multi-probe
+                                  traces (hit/miss lists, residency and eviction order; block id
+                                  values aside) and by the same invariants
   kmeans.*                        brute force on tiny inputs in fp64, plus invariants (partition of
                                   the tokens, centroid*size = sum of keys, empty cluster keeps its
                                   centroid, float32 init formula, remainder tokens); the fixed
