@@ -21,6 +21,9 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK = 8.0e12  # bytes/s, MI355X
+# 16-bit element type of queries, keys, values and the index (--dtype): bfloat16 is the benchmark's, IEEE half
+# the default of the reference's harnesses (simple_test.py:29, throughput_eval/test.py:28)
+DT, DT_NAME = torch.bfloat16, "bf16"
 
 # HBM bytes per attend_kernel launch come from rocprofv3 counter runs of this script (FETCH_SIZE and
 # WRITE_SIZE, each scaled by what the counter reads for the known-size copy of --copy-probe): the figures
@@ -80,7 +83,7 @@ def build_cache(cfg, L, dev, residency="device", block_cache="device", estimate_
     ctx = N + synth.STEADY_START + synth.STEADY_END
     cache = retroinfer_cache(
         valid_start=[0] * B, layer_num=L, batch_size=B, max_length=ctx + new, num_key_value_heads=Hkv,
-        num_heads=Hkv * gs, head_dim=128, dtype=torch.bfloat16, layer_mapping={str(l): "cuda:0" for l in range(L)},
+        num_heads=Hkv * gs, head_dim=128, dtype=DT, layer_mapping={str(l): "cuda:0" for l in range(L)},
         max_new_length=new, static_pattern_start=synth.STEADY_START, static_pattern_end=synth.STEADY_END, core=8,
         n_centroids=cfg["nc"], n_segment=cfg["S"], nprobe=nprobe, max_compute_cluster_num=nprobe + es,
         cache_unit_size=8, cache_cluster_num=max(int(cfg["nc"] * 0.05), nprobe), num_gpus=1, model_size=0,
@@ -97,9 +100,9 @@ def build_cache(cfg, L, dev, residency="device", block_cache="device", estimate_
                 k, v, q = synth.make_group(l, b, h, N, cfg["K"], gs, outliers=cfg["outliers"],
                                            n_extra=synth.STEADY_START + synth.STEADY_END, device=dev)
                 # steady zone = the extra tokens: 4 first, 64 last
-                k = torch.cat([k[N:N + 4], k[:N], k[N + 4:]]).to(torch.bfloat16)
-                v = torch.cat([v[N:N + 4], v[:N], v[N + 4:]]).to(torch.bfloat16)
-                ks.append(k); vs.append(v); qs.append(q.to(torch.bfloat16))
+                k = torch.cat([k[N:N + 4], k[:N], k[N + 4:]]).to(DT)
+                v = torch.cat([v[N:N + 4], v[:N], v[N + 4:]]).to(DT)
+                ks.append(k); vs.append(v); qs.append(q.to(DT))
             K = torch.stack(ks, 1)[None].contiguous()   # [1, ctx, Hkv, D]
             V = torch.stack(vs, 1)[None].contiguous()
             cache.prefill_update_kv_cache(None, K, V, l, b)
@@ -115,8 +118,8 @@ def build_cache(cfg, L, dev, residency="device", block_cache="device", estimate_
     # one generated token per layer so that the steady zone has its 69th entry
     g = torch.Generator(device=dev).manual_seed(12345)
     for l in range(L):
-        kn = torch.randn(B, 1, Hkv, 128, generator=g, device=dev).to(torch.bfloat16)
-        vn = torch.randn(B, 1, Hkv, 128, generator=g, device=dev).to(torch.bfloat16)
+        kn = torch.randn(B, 1, Hkv, 128, generator=g, device=dev).to(DT)
+        vn = torch.randn(B, 1, Hkv, 128, generator=g, device=dev).to(DT)
         cache.decode_update_kv_cache(kn, vn, l)
     return cache, queries, nprobe, es
 
@@ -191,7 +194,7 @@ def bench_kmeans(cfg, dev, iters=10, reps=3):
     ks, vs = [], []
     for h in range(Hkv):
         k, v, _ = synth.make_group(0, 0, h, N, cfg["K"], cfg["gs"], outliers=cfg["outliers"], n_extra=0, device=dev)
-        ks.append(k.to(torch.bfloat16)); vs.append(v.to(torch.bfloat16))
+        ks.append(k.to(DT)); vs.append(v.to(DT))
     K, V = torch.stack(ks).contiguous(), torch.stack(vs).contiguous()
     K = (K - K.mean(dim=1, keepdim=True)).contiguous()          # keys are centred before clustering
     r = segment_k_means_csr(K, V, nc, iters, S, reuse_graph=False)   # warm-up; its result is kept below
@@ -234,7 +237,7 @@ def kmeans_cpu_baseline(cfg, iters=10):
     Hkv, N, nc, S = cfg["Hkv"], cfg["N"], cfg["nc"], cfg["S"]
     nseg, ncs = N // S, nc // S
     k, _, _ = synth.make_group(0, 0, 0, N, cfg["K"], cfg["gs"], outliers=cfg["outliers"], n_extra=0)
-    k = k.to(torch.bfloat16)
+    k = k.to(DT)
     k = (k - k.mean(dim=0, keepdim=True)).contiguous()
     cent = k[okm.init_indices(N, nc)].clone()
     d, c = k[:nseg], cent[:ncs]
@@ -367,7 +370,7 @@ def bench_end_to_end(args, cfg, dev):
     print(json.dumps({
         "metric": "decode tokens/s end to end (random-weight model of the config's shape around the wave-index cache)",
         "value": B / t, "unit": "tokens/s", "n_gpus": 1, "steps": tokens, "warmup": args.warmup, "ms_per_step": t * 1e3,
-        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": DT_NAME, "data": "synthetic",
         "config": {"workload": f"{args.config}: {cfg['desc']}; {L} layers, hidden {shape.hidden_size}, MLP "
                                f"{shape.intermediate_size}, vocabulary {shape.vocab_size}; one HIP graph per token",
                    "batch": B, "context_tokens": ctx, "weight_bytes": weights,
@@ -474,7 +477,7 @@ def bench_host(args, cfg, cache, queries, L, nprobe, es, static_len, config_name
         n_k = max(L, min(args.steps, 128) // L * L)
         ev = [[torch.cuda.Event(enable_timing=True) for _ in range(6)] for _ in range(n_k)]
         D, rows, stage0 = 128, cache.cache_blocks * cache.page_size, cache.cache_size * cache.page_size
-        out_tmp = torch.empty((BG, gs, D), dtype=torch.bfloat16, device=queries[0].device)
+        out_tmp = torch.empty((BG, gs, D), dtype=DT, device=queries[0].device)
         for i in range(n_k):
             l, e = i % L, ev[i]
             q = queries[l].view(BG, gs, D)
@@ -506,7 +509,7 @@ def bench_host(args, cfg, cache, queries, L, nprobe, es, static_len, config_name
         from retrievalattention_amd import kernels
         l, n_k = L - 1, 32
         buf = l % 2
-        out_tmp = torch.empty((BG, gs, 128), dtype=torch.bfloat16, device=queries[0].device)
+        out_tmp = torch.empty((BG, gs, 128), dtype=DT, device=queries[0].device)
         ev = [[torch.cuda.Event(enable_timing=True) for _ in range(2)] for _ in range(n_k)]
         for e in ev:
             e[0].record()
@@ -562,7 +565,7 @@ def bench_host(args, cfg, cache, queries, L, nprobe, es, static_len, config_name
         "metric": "decode tokens/s at 128K ctx (attention only, B / (L * t_layer_step)); us/layer-step and % HBM roofline alongside",
         "value": B / (cfg["L"] * t_warm), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": t_warm * 1e3, "us_per_layer_step": t_warm * 1e6, "cold_us_per_layer_step": t_cold * 1e6,
-        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": DT_NAME, "data": "synthetic",
         "config": {"workload": f"{args.config}: {cfg['desc']}; clustered K/V in pinned host memory, block cache of "
                                f"{cache.cache_size if hasattr(cache, 'cache_size') else '?'} blocks per group, "
                                f"block cache manager on the {cache.block_cache}, miss staging "
@@ -735,7 +738,7 @@ def bench_device(args, cfg, config_name, L, dev, extras=True):
     stream = torch.cuda.current_stream().cuda_stream
     n_k = min(args.steps, 256)
     ev = [[torch.cuda.Event(enable_timing=True) for _ in range(4)] for _ in range(n_k)]
-    out_tmp = torch.empty((BG, gs, 128), dtype=torch.bfloat16, device=dev)
+    out_tmp = torch.empty((BG, gs, 128), dtype=DT, device=dev)
 
     def attend(l, slot):
         kernels.wave_attention(
@@ -774,7 +777,7 @@ def bench_device(args, cfg, config_name, L, dev, extras=True):
         "timed_region": {"repeats": len(reps_t), "statistic": "median", "min_us_per_layer_step": reps_t[0] * 1e6,
                          "max_us_per_layer_step": reps_t[-1] * 1e6, "layer_steps_per_region": args.steps * inner,
                          "replays_of_the_steps_per_region": inner},
-        "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "scaling": "weak", "vs_baseline": None, "dtype": DT_NAME, "data": "synthetic",
         "config": {"workload": f"{config_name}: {cfg['desc']}; nprobe {nprobe}, estimation zone {es}, "
                                f"steady zone {static_len}, {L} layers with independent seeds (seeded Gaussian-mixture "
                                f"K/V drawn by torch's generator on the device), "
@@ -830,6 +833,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=64)
     ap.add_argument("--config", default="c2", choices=sorted(CONFIGS))
     ap.add_argument("--layers", type=int, default=0, help="distinct layers (default: the config's)")
+    ap.add_argument("--dtype", default="bf16", choices=["bf16", "fp16"],
+                    help="16-bit element type of the tensors (bf16: the benchmark's; fp16: the reference harnesses' default)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-graph", action="store_true", help="time eager launches instead of HIP graph replays")
     ap.add_argument("--residency", default="device", choices=["device", "host"],
@@ -860,6 +865,9 @@ def main():
     ap.add_argument("--copy-probe", action="store_true",
                     help="also run 8 device copies of 256 MiB (a known-size kernel to scale rocprofv3 byte counters by)")
     args = ap.parse_args()
+    global DT, DT_NAME
+    if args.dtype == "fp16":
+        DT, DT_NAME = torch.float16, "f16"
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: the wave-index path has no cross-GPU exchange (run with --gpus 1)")
     if not torch.cuda.is_available():

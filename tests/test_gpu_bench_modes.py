@@ -18,6 +18,8 @@ COMMON = ["--config", "c1", "--steps", "16", "--warmup", "4", "--repeats", "3", 
     ["--residency", "host", "--layers", "2"],                 # host store, block cache managed on the device
     ["--residency", "host", "--layers", "2", "--overlap"],    # ... cached rows attended beside the miss staging
     ["--residency", "host", "--layers", "2", "--block-cache", "host"],   # ... managed by the worker threads
+    ["--dtype", "fp16", "--no-other-configs"],                # IEEE half elements, device-resident store
+    ["--dtype", "fp16", "--residency", "host", "--layers", "2"],   # ... host store
 ])
 def test_bench_mode_prints_the_contract_line(dev, mode):
     r = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py")] + COMMON + mode, capture_output=True, text=True,
@@ -31,6 +33,8 @@ def test_bench_mode_prints_the_contract_line(dev, mode):
     assert "workload" in line["config"]
     assert line["roofline"] is not None and line["roofline"]["bound"] == "hbm" and 0 < line["roofline"]["frac"] < 1
     assert line["cpu_baseline"] is not None and line["cpu_baseline"]["kind"] in ("port", "reference")
+    assert line["dtype"] == ("f16" if "fp16" in mode else "bf16")
+    assert line["cpu_baseline"]["max_abs_vs_gpu"] <= 2e-2     # the oracle's output of the same step
 
 
 def test_bench_refuses_more_than_one_gpu():

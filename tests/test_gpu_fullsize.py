@@ -25,7 +25,7 @@ SHAPES = {
 }
 
 
-def _build(dev, cfg):
+def _build(dev, cfg, dt=torch.bfloat16):
     """One layer of the cache at a benchmark shape, K/V from the seeded generator on the device."""
     from retrievalattention_amd import synth
     from retrievalattention_amd.cache_hub import retroinfer_cache
@@ -34,7 +34,7 @@ def _build(dev, cfg):
     ctx = N + synth.STEADY_START + synth.STEADY_END
     cache = retroinfer_cache(
         valid_start=[0] * B, layer_num=1, batch_size=B, max_length=ctx + 4, num_key_value_heads=Hkv,
-        num_heads=Hkv * gs, head_dim=128, dtype=torch.bfloat16, layer_mapping={"0": "cuda:0"}, max_new_length=4,
+        num_heads=Hkv * gs, head_dim=128, dtype=dt, layer_mapping={"0": "cuda:0"}, max_new_length=4,
         static_pattern_start=synth.STEADY_START, static_pattern_end=synth.STEADY_END, core=8, n_centroids=nc,
         n_segment=cfg["S"], nprobe=nprobe, max_compute_cluster_num=nprobe + es, cache_unit_size=8,
         cache_cluster_num=max(int(nc * 0.05), nprobe), num_gpus=1, model_size=0, kv_residency=cfg["residency"])
@@ -44,9 +44,9 @@ def _build(dev, cfg):
         for h in range(Hkv):
             k, v, q = synth.make_group(cfg["seed"], b, h, N, nc, gs, outliers=cfg["outliers"],
                                        n_extra=synth.STEADY_START + synth.STEADY_END, device=dev)
-            ks.append(torch.cat([k[N:N + 4], k[:N], k[N + 4:]]).to(torch.bfloat16))
-            vs.append(torch.cat([v[N:N + 4], v[:N], v[N + 4:]]).to(torch.bfloat16))
-            qs.append(q.to(torch.bfloat16))
+            ks.append(torch.cat([k[N:N + 4], k[:N], k[N + 4:]]).to(dt))
+            vs.append(torch.cat([v[N:N + 4], v[:N], v[N + 4:]]).to(dt))
+            qs.append(q.to(dt))
         K = torch.stack(ks, 1)[None].contiguous()
         V = torch.stack(vs, 1)[None].contiguous()
         cache.prefill_update_kv_cache(None, K, V, 0, b)
@@ -76,8 +76,8 @@ def _oracle_step(cache, q, static_len, nprobe, es):
 
 def _step(cache, q, dev, seed):
     g = torch.Generator(device=dev).manual_seed(seed)
-    kn = torch.randn(cache.batch_size, 1, cache.kv_head, 128, generator=g, device=dev).to(torch.bfloat16)
-    vn = torch.randn(cache.batch_size, 1, cache.kv_head, 128, generator=g, device=dev).to(torch.bfloat16)
+    kn = torch.randn(cache.batch_size, 1, cache.kv_head, 128, generator=g, device=dev).to(q.dtype)
+    vn = torch.randn(cache.batch_size, 1, cache.kv_head, 128, generator=g, device=dev).to(q.dtype)
     cache.decode_update_kv_cache(kn, vn, 0)
     out = cache.compute(q, 0)
     torch.cuda.synchronize()
@@ -85,9 +85,9 @@ def _step(cache, q, dev, seed):
 
 
 @pytest.mark.parametrize("name", ["c1", "c2", "c5", "c4"])
-def test_benchmark_shape_decode(dev, name):
+def test_benchmark_shape_decode(dev, name, dt=torch.bfloat16):
     cfg = SHAPES[name]
-    cache, q, nprobe, es = _build(dev, cfg)
+    cache, q, nprobe, es = _build(dev, cfg, dt)
     BG, gs = cache.batch_groups, cache.group_size
     # clustering invariants at full size
     if cache.kv_residency == "device":
@@ -106,7 +106,7 @@ def test_benchmark_shape_decode(dev, name):
     # selections against the oracle's scores: equal except ties within one bf16 ulp of a zone boundary
     cI = cache.cI[0].cpu()
     swaps = check_zone_sets(aux["dist"], cI[:, :nprobe], cI[:, nprobe:], aux["ret"], aux["est"], nprobe, es, band=1.0,
-                            label=f"full size {name}")
+                            label=f"full size {name}" + (" f16" if dt == torch.float16 else ""))
     assert swaps <= BG * 8
     if cache.kv_residency == "host":
         # second step with the same query: blocks admitted by the first step now hit
@@ -127,11 +127,24 @@ def test_benchmark_shape_decode(dev, name):
     out2 = cache.compute(q, 0)
     torch.cuda.synchronize()
     assert torch.equal(cache.cI[0], sel_before)
-    assert torch.equal(out2.view(torch.int16), (out1 * 2).view(torch.int16))
+    if dt == torch.float16:
+        # an output below the smallest normal half (2^-14) was rounded on the coarser subnormal grid (2^-24)
+        normal = out1.abs() >= 2.0 ** -14
+        assert torch.equal(out2[normal], (out1 * 2)[normal])
+        assert float((out2.float() - 2 * out1.float()).abs().max()) <= 2.0 ** -24
+    else:
+        assert torch.equal(out2.view(torch.int16), (out1 * 2).view(torch.int16))
     # and the step is reproducible run to run
     out3 = cache.compute(q, 0)
     torch.cuda.synchronize()
     assert torch.equal(out3, out2)
+
+
+@pytest.mark.parametrize("name", ["c1", "c2", "c4"])
+def test_benchmark_shape_decode_float16(dev, name):
+    """The benchmark shapes with IEEE half elements (the default of the reference's harnesses, simple_test.py:29):
+    the same checks, scores and probabilities rounded to fp16."""
+    test_benchmark_shape_decode(dev, name, dt=torch.float16)
 
 
 @pytest.mark.parametrize("S", [16, 1])
