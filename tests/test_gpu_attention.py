@@ -290,6 +290,20 @@ def test_wave_attention_random_shapes(dev):
         test_wave_attention(dev, BG, gs, nc, nprobe, es, static_len, 3000 + it)
 
 
+def test_wave_attention_random_shapes_float16(dev):
+    """Twelve random shapes with IEEE half elements."""
+    import random
+    rnd = random.Random(31338)
+    for it in range(12):
+        BG = rnd.choice([1, 2, 3])
+        gs = rnd.choice([1, 2, 3, 4, 5, 7, 8, 9, 12, 16])
+        nc = 8 * rnd.randint(4, rnd.choice([64, 300, 1200]))
+        nprobe = rnd.randint(1, min(1023, max(1, nc // 4)))
+        es = 0 if rnd.random() < 0.2 else rnd.randint(0, nc - nprobe)
+        static_len = rnd.choice([0, 1, 5, 69, 200, 700])
+        test_wave_attention(dev, BG, gs, nc, nprobe, es, static_len, 3100 + it, dt=torch.float16)
+
+
 def test_wave_attention_part_that_attends_nothing(dev):
     """A part with no steady zone, no estimation zone and a row window that holds none of the table's rows writes zeros and a log-sum-exp
     of -inf; a part that merges such a result (even one whose output holds NaN) ignores it."""

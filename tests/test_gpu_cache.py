@@ -332,25 +332,25 @@ def test_residencies_agree_with_cluster_estimation_random_shapes(dev):
 
 
 @pytest.mark.parametrize("residency", ["device", "host", "host-overlap", "host-cpu"])
-def test_next_layer_cluster_estimation(dev, residency):
+def test_next_layer_cluster_estimation(dev, residency, dt=torch.bfloat16):
     """use_cluster_estimation (reference: retroinfer_cache.py:565, 582-595): layers 0 and 1 choose their
     zones from their own query; every later layer uses the zones the previous layer chose from a
     predicted query, scores its estimation zone with the true query and attends the retrieval zone
     exactly.  Checked against the oracle with the same split between zone query and true query."""
     layers, B, Hkv, gs, ctx = 4, 2, 2, 4, 4096 + 68
     nc, nprobe, es = 256, 8, 60
-    cache = _make_cache(dev, residency, layers, B, Hkv, gs, ctx, nc, 1, nprobe, es, use_cluster_estimation=True)
-    K, V = _gen(layers, B, Hkv, gs, ctx, 256, dev, 11)
+    cache = _make_cache(dev, residency, layers, B, Hkv, gs, ctx, nc, 1, nprobe, es, use_cluster_estimation=True, dt=dt)
+    K, V = _gen(layers, B, Hkv, gs, ctx, 256, dev, 11, dt=dt)
     _prefill(cache, K, V, layers, B)
     BG = B * Hkv
     g = torch.Generator().manual_seed(12)
-    q_true = [torch.randn(B, 1, Hkv * gs, 128, generator=g).to(torch.bfloat16) for _ in range(layers)]
+    q_true = [torch.randn(B, 1, Hkv * gs, 128, generator=g).to(dt) for _ in range(layers)]
     # the prediction for layer l (made at layer l-1) is off by a fair amount: zones differ from the true ones
-    q_pred = [(q.float() + 0.5 * torch.randn(q.shape, generator=g)).to(torch.bfloat16) for q in q_true]
+    q_pred = [(q.float() + 0.5 * torch.randn(q.shape, generator=g)).to(dt) for q in q_true]
     differs = 0
     for l in range(layers):
-        kn = torch.randn(B, 1, Hkv, 128, generator=g).to(torch.bfloat16)
-        vn = torch.randn(B, 1, Hkv, 128, generator=g).to(torch.bfloat16)
+        kn = torch.randn(B, 1, Hkv, 128, generator=g).to(dt)
+        vn = torch.randn(B, 1, Hkv, 128, generator=g).to(dt)
         cache.decode_update_kv_cache(kn.to(dev), vn.to(dev), l)
         nxt = q_pred[l + 1].to(dev) if l + 1 < layers else None
         out = cache.compute(q_true[l].to(dev), l, nxt)
@@ -386,6 +386,10 @@ def test_next_layer_cluster_estimation(dev, residency):
             differs += int((aux_true["ret"] != aux["ret"]).any())
     assert differs > 0
 
+
+@pytest.mark.parametrize("residency", ["device", "host", "host-cpu"])
+def test_next_layer_cluster_estimation_float16(dev, residency):
+    test_next_layer_cluster_estimation(dev, residency, dt=torch.float16)
 
 
 def test_reference_stale_row_switch(dev):
@@ -442,7 +446,7 @@ def test_reference_stale_row_switch(dev):
 
 
 @pytest.mark.parametrize("residency", ["device", "host", "host-cpu", "device-pos"])
-def test_index_growth_after_1024_generated_tokens(dev, residency):
+def test_index_growth_after_1024_generated_tokens(dev, residency, dt=torch.bfloat16):
     """Decode-time index update (reference: retroinfer_cache.py:462-546): once the steady zone holds
     1024 tokens beyond its 4 + 64, they are clustered into 64 new centroids and appended to the index
     and the store; the last 64 stay as the local window.  Checked: the appended store rows are exactly
@@ -452,15 +456,15 @@ def test_index_growth_after_1024_generated_tokens(dev, residency):
     # the first sequence is left-padded: it holds fewer clustered tokens than the second, so the groups
     # append their folded tokens at different store rows (reference: wave_buffer_cpu.cpp:658)
     vstart = [64, 0]
-    cache = _make_cache(dev, residency, layers, B, Hkv, gs, ctx, nc, 1, nprobe, es, new=new, valid_start=vstart)
-    K, V = _gen(layers, B, Hkv, gs, ctx, 128, dev, 21)
+    cache = _make_cache(dev, residency, layers, B, Hkv, gs, ctx, nc, 1, nprobe, es, new=new, valid_start=vstart, dt=dt)
+    K, V = _gen(layers, B, Hkv, gs, ctx, 128, dev, 21, dt=dt)
     _prefill(cache, K, V, layers, B)
     BG = B * Hkv
     Ng = [ctx - 68 - vstart[gi // Hkv] for gi in range(BG)]     # clustered prompt tokens per group
     g = torch.Generator().manual_seed(22)
-    gk = torch.randn(B, 1030, Hkv, 128, generator=g).to(torch.bfloat16)
-    gv = torch.randn(B, 1030, Hkv, 128, generator=g).to(torch.bfloat16)
-    q = torch.randn(B, 1, Hkv * gs, 128, generator=g).to(torch.bfloat16).to(dev)
+    gk = torch.randn(B, 1030, Hkv, 128, generator=g).to(dt)
+    gv = torch.randn(B, 1030, Hkv, 128, generator=g).to(dt)
+    q = torch.randn(B, 1, Hkv * gs, 128, generator=g).to(dt).to(dev)
     lk, lv = cache.list_keys[0].view(BG, -1, 128), cache.list_values[0].view(BG, -1, 128)
     before_k = [lk[gi, :Ng[gi]].cpu().clone() for gi in range(BG)]
     before_v = [lv[gi, :Ng[gi]].cpu().clone() for gi in range(BG)]
@@ -516,6 +520,11 @@ def test_index_growth_after_1024_generated_tokens(dev, residency):
     _close(out.cpu().view(BG, gs, 128), ref)
     cI = cache.cI[0].cpu()
     check_zone_sets(aux["dist"], cI[:, :nprobe], cI[:, nprobe:], aux["ret"], aux["est"], nprobe, es, band=1.0)
+
+
+@pytest.mark.parametrize("residency", ["device", "host"])
+def test_index_growth_after_1024_generated_tokens_float16(dev, residency):
+    test_index_growth_after_1024_generated_tokens(dev, residency, dt=torch.float16)
 
 
 def test_captured_steps_replay_token_after_token(dev):

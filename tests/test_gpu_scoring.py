@@ -211,6 +211,23 @@ def test_score_select_random_shapes(dev):
         test_score_select(dev, BG, gs, nc, nprobe, es, 1100 + it)
 
 
+def test_score_select_random_shapes_float16(dev):
+    """Twenty of the random shapes with IEEE half elements, four of them with more than 1023 probes."""
+    import random
+    rnd = random.Random(778)
+    for it in range(20):
+        BG = rnd.choice([1, 2, 3])
+        gs = rnd.choice([1, 2, 3, 4, 5, 7, 8, 9, 12, 16])
+        if it < 16:
+            nc = 8 * rnd.randint(4, rnd.choice([64, 600, 3000, 6000]))
+            nprobe = rnd.randint(1, min(1023, max(1, nc // 4)))
+        else:
+            nc = 8 * rnd.randint(640, 4000)
+            nprobe = rnd.randint(1024, min(4096, nc // 3))
+        es = 0 if rnd.random() < 0.2 else rnd.randint(0, nc - nprobe)
+        test_score_select(dev, BG, gs, nc, nprobe, es, 1200 + it, dt=torch.float16)
+
+
 @pytest.mark.parametrize("kind", ["all_equal", "mostly_masked", "two_values"])
 def test_score_select_degenerate_scores(dev, kind):
     """Score distributions that put (nearly) every cluster on one score: identical centroids, 97 % of the
