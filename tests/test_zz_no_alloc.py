@@ -13,11 +13,10 @@ import torch
 pytestmark = pytest.mark.gpu
 
 
-def _case(dev, BG, gs, nc, N, nprobe, es, seed):
+def _case(dev, BG, gs, nc, N, nprobe, es, seed, bf=torch.bfloat16):
     """A selected step: runs ri_score_select on random data and returns everything the attention reads."""
     from retrievalattention_amd import kernels
     g = torch.Generator().manual_seed(seed)
-    bf = torch.bfloat16
     rn = lambda *s: torch.randn(*s, generator=g).to(bf).to(dev)
     size = torch.randint(1, 30, (BG, nc), generator=g, dtype=torch.int32)
     size[:, -1] += (N - size.sum(1)).clamp(min=0).int()
@@ -44,30 +43,32 @@ def _attend(dev, d, BG, gs, nc, nprobe, es, static, static_len=71):
     from retrievalattention_amd import _lib
     lib = _lib.lib()
     p = lambda t: None if t is None else C.c_void_p(t.data_ptr())
-    out = torch.zeros(BG, gs, 128, dtype=torch.bfloat16, device=dev)
+    out = torch.zeros(BG, gs, 128, dtype=d["q"].dtype, device=dev)
     vl = torch.zeros(BG, dtype=torch.int32, device=dev)
     stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    sfx = "_f16" if d["q"].dtype == torch.float16 else ""
     head = (p(d["q"]), p(d["stk"]), p(d["stv"]), 80, static_len, None, p(d["sk"]), p(d["sv"]), d["rows"], None, 0,
             p(d["rto"]), p(d["rst"]), nprobe, p(d["meta"]), p(d["est"]) if es else None, p(d["logits"]) if es else None,
             None, p(d["vsum"]), p(d["csz"]), p(out), p(vl), BG, gs, nc, es, 1 / math.sqrt(128))
     if static:
-        rc = lib.ri_wave_attention_static(*head, stream)
+        rc = getattr(lib, "ri_wave_attention_static" + sfx)(*head, stream)
     else:
         nb = lib.ri_wave_attention_workspace_bytes(BG, gs)
         ws = torch.zeros(nb, dtype=torch.uint8, device=dev)
-        rc = lib.ri_wave_attention(*head, p(ws), nb, stream)
+        rc = getattr(lib, "ri_wave_attention" + sfx)(*head, p(ws), nb, stream)
     assert rc == 0, lib.ri_status_string(rc)
     torch.cuda.synchronize()
     return out.cpu(), vl.cpu()
 
 
-def test_static_scratch_entry_point_matches_the_workspace_one(dev):
+@pytest.mark.parametrize("dt", [torch.bfloat16, torch.float16], ids=["bf16", "f16"])
+def test_static_scratch_entry_point_matches_the_workspace_one(dev, dt):
     from retrievalattention_amd import _lib
     assert _lib.lib().ri_wave_attention_static_scratch_bytes() == 8 << 20
     big = (16, 4, 1024, 16384, 18, 230)        # BG, gs, nc, tokens, nprobe, es
     small = (3, 7, 256, 3000, 5, 0)            # fewer groups, another head padding, no estimation zone
     for i, (BG, gs, nc, N, nprobe, es) in enumerate((big, small, big)):
-        d = _case(dev, BG, gs, nc, N, nprobe, es, seed=40 + i)
+        d = _case(dev, BG, gs, nc, N, nprobe, es, seed=40 + i, bf=dt)
         ref, vl_ref = _attend(dev, d, BG, gs, nc, nprobe, es, static=False)
         got, vl = _attend(dev, d, BG, gs, nc, nprobe, es, static=True)
         assert torch.equal(got.view(torch.int16), ref.view(torch.int16)), f"call {i}: outputs differ"
