@@ -41,6 +41,41 @@ def test_softmax_uses_bf16_logits_for_the_final_value():
     assert float(soft[0, 0, 0]) == float(expect)
 
 
+def test_half_elements_round_to_half():
+    """The 16-bit element type comes from the tensors (batch_gemm_softmax.cu:185-197 dispatches on it; the reference's
+    harnesses default to fp16, simple_test.py:29).  Known answers that tell the two roundings apart: 1 + 2^-9 is a
+    half but not a bfloat16; 1 + 2^-12 is neither and rounds to 1 in half; 70000 overflows half but not bfloat16."""
+    x = torch.tensor([[[1.0 + 2 ** -9, 1.0 + 2 ** -12, 0.0, -3.0]]], dtype=torch.float32)
+    D, m, inv, soft = scoring.softmax_from_logits(x, torch.float16)
+    assert D.dtype == torch.float16 and soft.dtype == torch.float16
+    assert float(D[0, 0, 0]) == 1.0 + 2 ** -9 and float(D[0, 0, 1]) == 1.0
+    z = torch.exp(x - x.max()).sum()
+    expect = (torch.exp(torch.tensor([1.0 + 2 ** -9, 1.0, 0.0, -3.0]) - x.max()) / z).to(torch.float16)
+    assert torch.equal(soft[0, 0], expect)
+    # score sum and mask value in half
+    d = scoring.dist_from_softmax(torch.stack([soft[0, 0], soft[0, 0]])[None], torch.tensor([[False, False, True, False]]))
+    assert d.dtype == torch.float16 and float(d[0, 2]) == torch.finfo(torch.float16).min == -65504.0
+    assert float(d[0, 0]) == float((2 * soft[0, 0, 0].float()).to(torch.float16))
+    # spacing of the two types
+    from oracle.numerics import ulp16
+    t = torch.tensor([1.0, 3.0, 2.0 ** -15, 1000.0])
+    assert ulp16(t, torch.float16).tolist() == [2.0 ** -10, 2.0 ** -9, 2.0 ** -24, 0.5]
+    assert ulp16(t, torch.bfloat16).tolist() == [2.0 ** -7, 2.0 ** -6, 2.0 ** -22, 4.0]
+    # attention and k-means outputs carry the element type of their inputs
+    g = torch.Generator().manual_seed(8)
+    q, k, v = (torch.randn(*s, generator=g).to(torch.float16) for s in ((2, 4, 128), (2, 40, 128), (2, 40, 128)))
+    out, _ = attention.weighted_flash_decoding(q, k, v)
+    ref = torch.nn.functional.scaled_dot_product_attention(q.double(), k.double(), v.double())
+    assert out.dtype == torch.float16 and torch.allclose(out.double(), ref, atol=1e-3)   # bf16 would need 8e-3
+    cent = torch.randn(8, 128, generator=g).to(torch.float16)
+    s = np.full((8, 128), 1.0 + 2 ** -9, dtype=np.float32)
+    upd = okm.update(cent, s, np.array([1, 0, 2, 0, 0, 0, 0, 0], dtype=np.int32), False)
+    assert upd.dtype == torch.float16 and float(upd[0, 0]) == 1.0 + 2 ** -9 and torch.equal(upd[1], cent[1])
+    assert float(upd[2, 0]) == float(torch.tensor((1.0 + 2 ** -9) / 2).to(torch.float16))
+    vs = okm.value_sum(torch.full((3, 128), 30000.0, dtype=torch.float16), np.array([0, 0, 0]), 2)
+    assert vs.dtype == torch.float16 and bool(torch.isinf(vs[0]).all()) and bool((vs[1] == 0).all())   # 90000 > 65504
+
+
 def test_score_interval_brackets_the_oracle_scores():
     """The interval the GPU score check uses is a float64 restatement with a 4e-6 relative tolerance: the oracle's
     fp32 pipeline must fall inside it, and the interval must be a single value for nearly every cluster (else it
