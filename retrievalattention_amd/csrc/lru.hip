@@ -174,17 +174,22 @@ __global__ __launch_bounds__(LRU_THREADS) void lru_kernel(LruParams P) {
   }
   // the longest prefix of the misses whose blocks fit the whole cache may be admitted (none when the cache
   // has no blocks: every retrieved cluster then stays a miss, wave_buffer_cpu.cpp:119-130 with capacity 0)
+  // (a step whose clusters all hit — the steady state of a warm cache — admits nothing and skips the scans)
+  const bool any_miss = t5[2] > 0;  // uniform
   bool adm[R];
-  int va[1] = {0}, pa[1], ta[1];
-#pragma unroll
-  for (int i = 0; i < R; ++i) {
-    adm[i] = miss[i] && mb_pre[i] + nb[i] <= P.capacity;
-    va[0] += adm[i] ? nb[i] : 0;
-  }
-  lru_scan<1>(va, pa, ta, sh_scan);
-  const int need = ta[0];
   int adm_pre[R];
-  {
+  int need = 0;
+#pragma unroll
+  for (int i = 0; i < R; ++i) { adm[i] = false; adm_pre[i] = 0; }
+  if (any_miss) {
+    int va[1] = {0}, pa[1], ta[1];
+#pragma unroll
+    for (int i = 0; i < R; ++i) {
+      adm[i] = miss[i] && mb_pre[i] + nb[i] <= P.capacity;
+      va[0] += adm[i] ? nb[i] : 0;
+    }
+    lru_scan<1>(va, pa, ta, sh_scan);
+    need = ta[0];
     int a = pa[0];
 #pragma unroll
     for (int i = 0; i < R; ++i) { adm_pre[i] = a; a += adm[i] ? nb[i] : 0; }
@@ -337,14 +342,14 @@ __global__ __launch_bounds__(LRU_THREADS) void lru_kernel(LruParams P) {
   }
 
   // ---- admission: block ids come off the end of the free list in rank order ----
-  int vb[2] = {0, 0}, pb[2], tb[2];
+  int vb[2] = {0, 0}, pb[2] = {0, 0}, tb[2] = {0, 0};
 #pragma unroll
   for (int i = 0; i < R; ++i) {
     adm[i] = adm[i] && adm_pre[i] + nb[i] <= F;  // (always true: everything resident can be evicted)
     vb[0] += adm[i] ? nb[i] : 0;
     vb[1] += adm[i] ? 1 : 0;
   }
-  lru_scan<2>(vb, pb, tb, sh_scan);
+  if (any_miss) lru_scan<2>(vb, pb, tb, sh_scan);
   int adm_idx = pb[1];
 #pragma unroll
   for (int i = 0; i < R; ++i) {
