@@ -225,7 +225,8 @@ int ri_wave_attention_f16(const void* q, const void* steady_k, const void* stead
 /* One part of a wave attention over a row table (host-resident store, block cache managed on the device;
  * cache_hub/retroinfer_cache.py:629-674, where the reference overlaps the transfer of missed blocks with
  * other work on its copy stream): as ri_wave_attention with row_src, but of the table's rows only those
- * whose source row lies in [src_row_lo, src_row_hi) are attended.  (prev_out [BG, gs, 128] bf16, prev_lse
+ * whose source row lies in [src_row_lo, src_row_hi) are attended (the window may be empty: a block cache of
+ * zero blocks has no cached rows).  (prev_out [BG, gs, 128] bf16, prev_lse
  * [BG, gs] fp32), both or neither, is an earlier part's result that is merged in (log-sum-exp rule);
  * lse_out [BG, gs] fp32 or NULL receives this part's log-sum-exp.  static_len = 0 leaves the steady zone
  * out, es = 0 the estimation zone.  Two calls over complementary windows, the second with the first's

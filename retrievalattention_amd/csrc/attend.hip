@@ -818,7 +818,7 @@ static int ri_wave_attention_part_any(const void* q, const void* steady_k, const
                                       const float* prev_lse, void* out, float* lse_out, int32_t* valid_lengths,
                                       int BG, int gs, int nc, int es, float scale, void* workspace,
                                       size_t workspace_bytes, ri_stream_t stream, bool half) {
-  if (!row_src || src_row_lo >= src_row_hi) return RI_ERR_ARG;
+  if (!row_src || src_row_lo > src_row_hi) return RI_ERR_ARG;   // an empty window attends none of the table's rows
   if (workspace && workspace_bytes < attn_workspace_bytes(BG, gs)) return RI_ERR_WORKSPACE;
   // a part that leaves the steady zone out must not pick its length up from the device either
   if (static_len == 0) static_len_dev = nullptr;

@@ -202,7 +202,7 @@ def test_host_and_device_residency_agree_and_cache_warms(dev, host_kind):
         assert checked > 0
 
 
-@pytest.mark.parametrize("host_kind", ["host", "host-cpu"])
+@pytest.mark.parametrize("host_kind", ["host", "host-overlap", "host-cpu"])
 def test_no_block_cache(dev, host_kind):
     """cache_cluster_num = 0, as the reference's throughput harness sets it (throughput_eval/test.py:77: no GPU
     block cache): every retrieved cluster is read from the host store at every step and nothing is admitted
