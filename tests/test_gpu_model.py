@@ -7,23 +7,24 @@ import torch
 pytestmark = pytest.mark.gpu
 
 
-def _models(dev, device_positions=False):
+def _models(dev, device_positions=False, dt=torch.bfloat16):
     from retrievalattention_amd.model_hub import LlamaModel, LlamaShape
     shape = LlamaShape(hidden_size=256, intermediate_size=512, num_layers=2, num_heads=8, num_key_value_heads=2,
                        head_dim=128, vocab_size=1000)
     B, ctx, new = 2, 1024 + 68, 8
     g = torch.Generator().manual_seed(3)
     ids = torch.randint(0, shape.vocab_size, (B, ctx), generator=g).to(dev)
-    wave = LlamaModel(shape, ctx + new, device=dev, seed=1)
-    dense = LlamaModel(shape, ctx + new, device=dev, seed=1)
+    wave = LlamaModel(shape, ctx + new, dtype=dt, device=dev, seed=1)
+    dense = LlamaModel(shape, ctx + new, dtype=dt, device=dev, seed=1)
     wave.init_kv_cache("RetroInfer", B, ctx, new, dict(n_centroids=64, n_segment=1, nprobe=64, max_compute_cluster_num=64),
                        device_positions=device_positions)
     dense.init_kv_cache("Full_Flash_Attn", B, ctx, new)
     return wave, dense, ids, new
 
 
-def test_full_probe_decodes_like_dense_attention(dev):
-    wave, dense, ids, new = _models(dev)
+@pytest.mark.parametrize("dt", [torch.bfloat16, torch.float16], ids=["bf16", "f16"])
+def test_full_probe_decodes_like_dense_attention(dev, dt):
+    wave, dense, ids, new = _models(dev, dt=dt)
     lw, ld = wave.prefill_forward(ids), dense.prefill_forward(ids)
     assert torch.equal(lw, ld)               # prefill attention is the same dense kernel
     tok = ld.argmax(-1)
@@ -38,9 +39,10 @@ def test_full_probe_decodes_like_dense_attention(dev):
     assert wave.kv_cache.context == dense.kv_cache.context == ids.shape[1] + new - 1
 
 
-def test_whole_token_replays_as_one_graph(dev):
+@pytest.mark.parametrize("dt", [torch.bfloat16, torch.float16], ids=["bf16", "f16"])
+def test_whole_token_replays_as_one_graph(dev, dt):
     """Every layer of a decoded token captured once, replayed for the following tokens."""
-    wave, dense, ids, new = _models(dev, device_positions=True)
+    wave, dense, ids, new = _models(dev, device_positions=True, dt=dt)
     lw, ld = wave.prefill_forward(ids), dense.prefill_forward(ids)
     tok_in = ld.argmax(-1).clone()
     # first decoded token eagerly on a side stream (warm-up for the capture), then capture
