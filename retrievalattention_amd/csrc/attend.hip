@@ -693,6 +693,7 @@ static int wave_attention_impl(const void* q, const void* steady_k, const void* 
   if (ri_any_misaligned16(q, steady_k, steady_v, store_k, store_v, value_sum, est_centroids, out, scratch))
     return RI_ERR_ARG;
   if (!row_src && (!ret_tok_off || !ret_start || np <= 0 || np > RI_MAX_PROBES)) return RI_ERR_ARG;
+  if ((row_src && row_src_stride <= 0) || store_stride < 0) return RI_ERR_ARG;
   if (BG <= 0 || BG > RI_MAX_GROUPS || gs <= 0 || gs > 16 || static_len < 0 || static_len > steady_stride ||
       es < 0 || nc <= 0)
     return RI_ERR_ARG;
