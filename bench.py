@@ -74,7 +74,7 @@ def log(*a):
 
 
 def build_cache(cfg, L, dev, residency="device", block_cache="device", estimate_next=False, new=2,
-                device_positions=False, overlap_miss_staging=True):
+                device_positions=False, overlap_miss_staging=False):
     from retrievalattention_amd import synth
     from retrievalattention_amd.cache_hub import retroinfer_cache
     B, Hkv, gs, N = cfg["B"], cfg["Hkv"], cfg["gs"], cfg["N"]
