@@ -37,6 +37,19 @@ def test_bench_mode_prints_the_contract_line(dev, mode):
     assert line["cpu_baseline"]["max_abs_vs_gpu"] <= 2e-2     # the oracle's output of the same step
 
 
+@pytest.mark.parametrize("mode", [
+    ["--estimate-next", "--layers", "4"],     # zones of the next layer chosen from a predicted query on a side stream
+    ["--end-to-end"],                         # the random-weight model around the path, whole tokens per graph
+])
+def test_bench_side_modes_run(dev, mode):
+    """The two modes that measure something other than the contract's metric still run and print one JSON line."""
+    r = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py")] + COMMON + mode, capture_output=True, text=True,
+                       timeout=110, cwd=ROOT)
+    assert r.returncode == 0, r.stderr[-2000:]
+    line = json.loads(r.stdout.strip().splitlines()[-1])
+    assert line["value"] > 0 and line["n_gpus"] == 1 and "workload" in line["config"]
+
+
 def test_bench_refuses_more_than_one_gpu():
     r = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--gpus", "2"], capture_output=True, text=True,
                        timeout=110, cwd=ROOT)
