@@ -46,3 +46,30 @@ def test_missing_library_is_a_loud_error(monkeypatch, tmp_path):
     import pytest
     with pytest.raises(RuntimeError, match="no CPU or PyTorch fallback"):
         _lib.lib()
+
+
+def test_header_is_plain_c_and_cxx(tmp_path):
+    """What a cgo / JNI / ctypes binding would include: the header compiles as C99 and as C++11 on its own."""
+    import shutil
+    import subprocess
+    src = '#include "retro_mi355.h"\nint main(void) { return (int)sizeof(ri_stream_t) * 0; }\n'
+    for cc, name, std in (("gcc", "t.c", "-std=c99"), ("g++", "t.cpp", "-std=c++11")):
+        if shutil.which(cc) is None:
+            continue
+        f = tmp_path / name
+        f.write_text(src)
+        r = subprocess.run([cc, std, "-Wall", "-Wextra", "-pedantic", "-Werror", "-I", os.path.join(ROOT, "include"),
+                            "-fsyntax-only", str(f)], capture_output=True, text=True)
+        assert r.returncode == 0, r.stderr
+
+
+def test_binding_argument_counts_match_the_header():
+    """Every prototype of the header has as many parameters as the ctypes signature that binds it."""
+    from retrievalattention_amd import _lib
+    text = re.sub(r"/\*.*?\*/", "", open(HEADER).read(), flags=re.S)
+    protos = dict(re.findall(r"\b(ri_[a-z0-9_]+)\s*\(([^;{]*?)\)\s*;", text, flags=re.S))
+    assert sorted(protos) == sorted(_lib.SIGNATURES)
+    for name, params in protos.items():
+        params = params.strip()
+        n = 0 if params in ("", "void") else params.count(",") + 1
+        assert n == len(_lib.SIGNATURES[name][1]), (name, n, len(_lib.SIGNATURES[name][1]))
