@@ -63,13 +63,31 @@ def test_header_is_plain_c_and_cxx(tmp_path):
         assert r.returncode == 0, r.stderr
 
 
-def test_binding_argument_counts_match_the_header():
-    """Every prototype of the header has as many parameters as the ctypes signature that binds it."""
+def test_binding_arguments_match_the_header():
+    """Every prototype of the header has as many parameters, of the same kinds, as the ctypes signature that binds it."""
     from retrievalattention_amd import _lib
     text = re.sub(r"/\*.*?\*/", "", open(HEADER).read(), flags=re.S)
     protos = dict(re.findall(r"\b(ri_[a-z0-9_]+)\s*\(([^;{]*?)\)\s*;", text, flags=re.S))
     assert sorted(protos) == sorted(_lib.SIGNATURES)
+    def kind(decl):
+        decl = decl.strip()
+        if "*" in decl or re.match(r"(const\s+)?ri_stream_t\b", decl):
+            return ctypes.c_void_p
+        base = re.sub(r"\b(const|unsigned)\b", "", decl).split()[0]
+        return {"int": ctypes.c_int, "int32_t": ctypes.c_int, "int64_t": ctypes.c_int64, "float": ctypes.c_float,
+                "size_t": ctypes.c_size_t}[base]
+
     for name, params in protos.items():
         params = params.strip()
-        n = 0 if params in ("", "void") else params.count(",") + 1
-        assert n == len(_lib.SIGNATURES[name][1]), (name, n, len(_lib.SIGNATURES[name][1]))
+        kinds = [] if params in ("", "void") else [kind(x) for x in params.split(",")]
+        bound = _lib.SIGNATURES[name][1]
+        assert len(kinds) == len(bound), (name, len(kinds), len(bound))
+        # and of the same kind: a 64-bit stride or a size bound as int would be cut in half without any error
+        for i, (a, b) in enumerate(zip(kinds, bound)):
+            assert a is b, (name, i, a, b)
+    rets = dict((n, r.strip()) for r, n in re.findall(r"([A-Za-z_][\w \*]*?)\s*\b(ri_[a-z0-9_]+)\s*\(", text))
+    for name, (restype, _) in _lib.SIGNATURES.items():
+        r = rets[name]
+        want = ctypes.c_char_p if r == "const char*" else ctypes.c_void_p if "*" in r else \
+            {"int": ctypes.c_int, "size_t": ctypes.c_size_t, "int64_t": ctypes.c_int64, "void": None}[r]
+        assert restype is want, (name, r, restype)
