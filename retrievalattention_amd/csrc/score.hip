@@ -102,7 +102,7 @@ __device__ __forceinline__ void score_body(
     sh_sum[wave][r] = lsum;
   }
   __syncthreads();
-  if (threadIdx.x < gs) {
+  if ((int)threadIdx.x < gs) {
     const int j = threadIdx.x;
     float m = sh_max[0][j];
 #pragma unroll
