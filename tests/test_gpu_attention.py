@@ -170,6 +170,7 @@ def test_closed_form_estimation_exact_for_singletons_and_identical_keys(dev):
     (1, 4, 15000, 1500, 2250, 69, 8),   # probe lists of the reference's throughput harness (10 % of the clusters)
     (1, 4, 30000, 3000, 1000, 69, 9),
     (1, 8, 16384, 4096, 0, 10, 10),     # the longest probe list
+    (4096, 1, 64, 4, 20, 5, 11),        # the most groups a launch takes (one counter each in the workspace)
 ])
 def test_wave_attention(dev, BG, gs, nc, nprobe, es, static_len, seed, dt=torch.bfloat16):
     """score_select + wave_attention against the oracle's composition of steps 4-8 of

@@ -101,6 +101,7 @@ def test_batch_gemm_softmax_half(dev):
     (2, 4, 15000, 1500, 2250, 8),    # probe lists of the reference's throughput harness (throughput_eval/test.py:74,
     (1, 4, 30000, 3000, 4500, 9),    #   nprobe = 10 % of the clusters): 240K and 480K tokens of context
     (1, 8, 40960, 4096, 100, 10),    # the longest probe list the entry point takes
+    (4096, 1, 64, 4, 20, 11),        # as many groups as an attention launch takes
 ])
 def test_score_select(dev, BG, gs, nc, nprobe, es, seed, dt=torch.bfloat16):
     from retrievalattention_amd import kernels
