@@ -52,6 +52,9 @@ class retroinfer_cache(KV_Cache):
         if num_heads % num_key_value_heads != 0 or num_heads // num_key_value_heads > kernels.MAX_GROUP_SIZE:
             raise ValueError(f"at most {kernels.MAX_GROUP_SIZE} query heads per KV head (got {num_heads} / "
                              f"{num_key_value_heads})")
+        if batch_size * num_key_value_heads > kernels.MAX_GROUPS:
+            raise ValueError(f"at most {kernels.MAX_GROUPS} groups (batch x KV heads) per attention launch (got "
+                             f"{batch_size} x {num_key_value_heads})")
         if not 1 <= nprobe <= kernels.MAX_PROBES:
             raise ValueError(f"nprobe must be in 1..{kernels.MAX_PROBES} (got {nprobe})")
         if n_centroids % 8 != 0 or n_centroids + n_new > kernels.MAX_CLUSTERS:

@@ -126,6 +126,7 @@ def release_cached_graphs(retired_workspaces=True):
 MAX_PROBES = 4096          # ri_score_select / ri_wave_attention / ri_lru_access_update: retrieval zone per group
 MAX_CLUSTERS = 65536       # ri_score_select / ri_lru_access_update: clusters per group (16-bit ids in the selection)
 MAX_GROUP_SIZE = 16        # query heads per KV head
+MAX_GROUPS = 4096          # ri_wave_attention / ri_weighted_flash_decoding: batch x KV heads of one launch
 
 
 # ----------------------------------------------------------------------------------------

@@ -243,6 +243,8 @@ def test_limits_are_checked_at_construction(dev):
         _make_cache(dev, "device", 1, 1, 1, 32, 4096 + 68, 256, 1, 8, 60)
     with pytest.raises(ValueError, match="must not be negative"):
         _make_cache(dev, "host", 1, 1, 1, 4, 4096 + 68, 256, 1, 8, 60, cache_cluster_num=-1)
+    with pytest.raises(ValueError, match="at most 4096 groups"):
+        _make_cache(dev, "device", 1, 1025, 4, 1, 4096 + 68, 256, 1, 8, 60)
 
 
 def test_residencies_agree_random_shapes(dev):
