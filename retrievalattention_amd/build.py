@@ -52,7 +52,23 @@ def build(verbose=False):
                 print(o)
     objs = [j[1] for j in jobs]
     _run([hipcc, "-shared", "-fPIC", f"--offload-arch={ARCH}", "-o", LIB] + objs + ["-pthread"])
+    build_capi_example(hipcc)
     return LIB
+
+
+# A plain HIP program that drives a decode step through the C ABI (no Python, no torch); tests/test_gpu_capi.py
+# runs it.  It finds the library next to the package through its run path.
+CAPI_EXAMPLE_SRC = os.path.join(os.path.dirname(HERE), "tests", "capi_decode_step.cpp")
+CAPI_EXAMPLE = os.path.join(os.path.dirname(HERE), "tests", "capi_decode_step")
+
+
+def build_capi_example(hipcc):
+    if not os.path.exists(CAPI_EXAMPLE_SRC):
+        return None
+    _run([hipcc, "-O2", "-std=c++17", f"--offload-arch={ARCH}", "-I", os.path.join(os.path.dirname(HERE), "include"),
+          CAPI_EXAMPLE_SRC, "-o", CAPI_EXAMPLE, "-L", HERE, "-l:libretro_mi355.so",
+          "-Wl,-rpath,$ORIGIN/../retrievalattention_amd"])
+    return CAPI_EXAMPLE
 
 
 if __name__ == "__main__":
