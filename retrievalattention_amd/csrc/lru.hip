@@ -76,7 +76,7 @@ __device__ __forceinline__ void lru_scan(const int (&v)[N], int (&pre)[N], int (
 template <int R>
 __global__ __launch_bounds__(LRU_THREADS) void lru_kernel(LruParams P) {
   constexpr int NPMAX = LRU_THREADS * R;
-  __shared__ int sh_scan[6 * LRU_WAVES];
+  __shared__ int sh_scan[7 * LRU_WAVES];
   __shared__ int sh_hist[LRU_DIGIT];
   __shared__ int sh_cut[2];  // selected digit, blocks freed by clusters with a larger one
   // token offsets and sources of the ranks for the row table; later the blocks of the boundary step's
@@ -121,13 +121,14 @@ __global__ __launch_bounds__(LRU_THREADS) void lru_kernel(LruParams P) {
     }
     nb_sum += nb[i];
   }
-  int v1[1] = {nb_sum}, p1[1], t1[1];
-  lru_scan<1>(v1, p1, t1, sh_scan);
-  // the walk stops at the first cluster whose blocks no longer fit: everything after it is dropped
+  // The walk stops at the first cluster whose blocks no longer fit: everything after it is dropped.  Whether
+  // anything is dropped is only known from the block prefix, so the counts are first taken as if nothing were
+  // (one scan for the block prefix and the counts together) and only recounted when the list was cut.
   bool keep[R], hit[R], miss[R];
-  int v5[6] = {0, 0, 0, 0, 0, 0}, p5[6], t5[6];
-  {
-    int run = p1[0];
+  int v5[6], p5[6], t5[6];
+  auto count = [&](int run) {
+#pragma unroll
+    for (int k = 0; k < 6; ++k) v5[k] = 0;
 #pragma unroll
     for (int i = 0; i < R; ++i) {
       keep[i] = c[i] >= 0 && nb[i] > 0 && run + nb[i] <= P.buffer_size;
@@ -141,8 +142,22 @@ __global__ __launch_bounds__(LRU_THREADS) void lru_kernel(LruParams P) {
       v5[4] += keep[i] ? 1 : 0;
       v5[5] += hit[i] ? 1 : 0;
     }
+  };
+  {
+    count(INT32_MIN / 2);   // no cut-off: every valid cluster with blocks is kept
+    int v7[7], p7[7], t7[7];
+#pragma unroll
+    for (int k = 0; k < 6; ++k) v7[k] = v5[k];
+    v7[6] = nb_sum;
+    lru_scan<7>(v7, p7, t7, sh_scan);
+    if (t7[6] <= P.buffer_size) {   // uniform: the whole list fits
+#pragma unroll
+      for (int k = 0; k < 6; ++k) { p5[k] = p7[k]; t5[k] = t7[k]; }
+    } else {
+      count(p7[6]);
+      lru_scan<6>(v5, p5, t5, sh_scan);
+    }
   }
-  lru_scan<6>(v5, p5, t5, sh_scan);
   // per rank: hit blocks, kept tokens, miss blocks, miss tokens, hits of the lower ranks
   int hb_pre[R], tok_pre[R], mb_pre[R], mt_pre[R], hit_idx[R];
   {
@@ -207,7 +222,7 @@ __global__ __launch_bounds__(LRU_THREADS) void lru_kernel(LruParams P) {
     __syncthreads();
     int32_t* table = P.row_src + (size_t)g * P.row_src_stride;
     for (int t = tid; t < t5[1]; t += LRU_THREADS) {
-      int lo_r = 0, hi_r = NPMAX;  // first rank whose offset exceeds t
+      int lo_r = 0, hi_r = min(NPMAX, P.np);  // first rank whose offset exceeds t (ranks past the list hold the total)
       while (lo_r < hi_r) {
         const int mid = (lo_r + hi_r) >> 1;
         if (sh_off[mid] > t) hi_r = mid; else lo_r = mid + 1;
